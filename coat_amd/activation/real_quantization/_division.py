@@ -1,0 +1,36 @@
+"""Per-tensor FP8 quantize by a given scalar scale.
+Reference: coat/activation/real_quantization/_division.py:153-207."""
+import torch
+
+from ... import _hip
+from .common import FP8_MAX_VALUE, SCALE_MIN_THRES, as_fp8_dtype, flatten_2d, no_stochastic, restore
+
+
+def absmax_scale(x, fp8type):
+    """(x.abs().max() + 1e-10) / fp8max in x's dtype (reference :178-179), one pass over x."""
+    amax = torch.zeros((), dtype=torch.float32, device=x.device)
+    _hip.check(_hip.lib().coat_absmax(_hip.ptr(x), _hip.dt(x), _hip.ptr(amax), x.numel(), _hip.stream(x.device)), "absmax")
+    return (amax.to(x.dtype) + SCALE_MIN_THRES) / FP8_MAX_VALUE[fp8type]
+
+
+def _division(x, fp8type, s_y, want_q, want_qt, what):
+    M, N = x.shape
+    if s_y is None:
+        s_y = absmax_scale(x, fp8type)
+    if s_y.numel() != 1:
+        raise ValueError(f"{what}: the scale must be a single element, got shape {tuple(s_y.shape)}")
+    s_dev = s_y if s_y.is_cuda else s_y.to(x.device)
+    y = torch.empty_like(x, dtype=fp8type) if want_q else None
+    y_t = torch.empty((N, M), dtype=fp8type, device=x.device) if want_qt else None
+    _hip.check(_hip.lib().coat_fp8_division(_hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.dt(s_dev), _hip.ptr(y),
+                                            _hip.ptr(y_t), M, N, _hip.fp8(fp8type), _hip.stream(x.device)), what)
+    return y, s_y, y_t
+
+
+def fp8_division(x, QB, fp8type, s_y=None, stochastic=False):
+    """x -> (y fp8, s_y); y = fp8(x / float(s_y)); s_y defaults to (absmax + 1e-10) / fp8max."""
+    no_stochastic(stochastic)
+    x, batch = flatten_2d(x)
+    x = _hip.dense(x)
+    y, s_y, _ = _division(x, as_fp8_dtype(fp8type), s_y, True, False, "fp8_division")
+    return restore(y, batch), s_y

@@ -1,0 +1,23 @@
+"""Per-tensor FP8 quantize through Group Scaling, with the transposed copy the backward GEMMs need.
+Reference: coat/activation/real_quantization/_quantize_pertensor_transpose.py:106-150."""
+import torch
+
+from ... import _hip
+from ._division import _division
+from ._quantize_pertensor import group_scales_and_max
+from .common import convert_str_to_fp8, flatten_2d, no_stochastic, restore
+
+
+def fp8_quantize_pertensor_transpose(x, QB, fp8type, transpose_output_2d=False, stochastic=False,
+                                     scale_dtype=torch.bfloat16):
+    """Returns (qy, s_y_max 0-dim, qy_t); qy_t is [N, M] unless the input was 3-D and
+    transpose_output_2d is False (then it is reshaped per batch, reference :145-150)."""
+    no_stochastic(stochastic)
+    x, batch = flatten_2d(x)
+    x = _hip.dense(x)
+    fp8type = convert_str_to_fp8[fp8type]
+    _, s_y_max = group_scales_and_max(x, QB, fp8type, scale_dtype, want_pg=False)
+    qy, s_y_max, qy_t = _division(x, fp8type, s_y_max, True, True, "fp8_quantize_pertensor_transpose")
+    if batch is not None and not transpose_output_2d:
+        qy_t = qy_t.reshape(batch, -1, qy_t.shape[-1])
+    return restore(qy, batch), s_y_max, qy_t

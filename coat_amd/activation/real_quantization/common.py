@@ -1,0 +1,45 @@
+"""Constants of the FP8 op library (reference: coat/activation/real_quantization/common.py:20-31)."""
+import torch
+
+SCALE_MIN_THRES = 1e-10
+
+FP8_MAX_VALUE = {
+    torch.float8_e4m3fn: 448.0,
+    torch.float8_e5m2: 57344.0,
+}
+
+convert_str_to_fp8 = {"E4M3": torch.float8_e4m3fn, "E5M2": torch.float8_e5m2}
+convert_fp8_to_embit = {
+    torch.float8_e4m3fn: (4.0, 3.0),
+    torch.float8_e5m2: (5.0, 2.0),
+}
+
+
+def as_fp8_dtype(fp8type):
+    """Accepts "E4M3"/"E5M2" or a torch fp8 dtype, as the reference entry points do."""
+    if isinstance(fp8type, str):
+        return convert_str_to_fp8[fp8type]
+    if fp8type not in FP8_MAX_VALUE:
+        raise ValueError(f"unsupported fp8 type {fp8type}")
+    return fp8type
+
+
+def flatten_2d(x):
+    """3-D [B, S, C] -> 2-D [B*S, C] as every reference launcher does; returns (x2d, batch or None)."""
+    if x.dim() == 3:
+        return x.reshape(-1, x.shape[-1]), x.shape[0]
+    if x.dim() != 2:
+        raise ValueError(f"expected a 2-D or 3-D tensor, got shape {tuple(x.shape)}")
+    return x, None
+
+
+def restore(y, batch):
+    """Inverse of flatten_2d for an output whose rows follow the input's rows."""
+    return y if batch is None else y.reshape(batch, -1, y.shape[-1])
+
+
+def no_stochastic(stochastic):
+    if stochastic:
+        raise NotImplementedError(
+            "stochastic rounding is not built (no caller in the reference enables it: "
+            "fp8linear.py:88,101; coat_llama.py:297,335,749)")

@@ -1,0 +1,349 @@
+// FP8 AdamW step for gfx950: one fused streaming kernel per parameter tensor.
+//
+// Replaces fp8_adamw_cuda_expand_kernel (Dynamic Range Expansion) and fp8_adamw_cuda_kernel of the
+// reference (one element per thread, 128-thread blocks, every thread recomputing the group constants).
+//
+// Layout: a wave owns 1024 consecutive elements = 8 quantization groups of 128.  Lane l works for group
+// l/8; with lam = l%8 it holds, for j = 0..3, the 4 consecutive elements 32*j + 4*lam .. +3 of its group.
+// A load instruction therefore reads, per group, one full 128-byte line of fp32 params / grads (16 bytes
+// per lane) and one 32-byte piece of FP8 codes; all 16 elements a lane touches share one group, so group
+// maxima / minima are 15 in-lane operations plus a 3-step DPP reduction over 8 lanes, and the group
+// constants (centre c, exponent k, new scale) are computed once per lane for 16 elements.
+//
+// Numerics: + - * / sqrt are the IEEE fp32 operations of the reference source in the same order without
+// FMA contraction, so the plain (non-expand) step is bit-exact against the CPU restatement.  The x^y of
+// the expand step is exp2(y * log2(x)) on the hardware v_log_f32 / v_exp_f32 (about 1e-6 relative),
+// with the IEEE special cases of powf (y = 0, y = inf, x = 0, x = 1) reproduced explicitly.
+// The reference's order-dependent zero-skipping minimum is reproduced exactly: when a group holds an
+// exact zero the kernel walks the reference's 32-lane shuffle tree, otherwise that tree equals a plain min.
+#include <math.h>
+
+#include "coat_device.h"
+#include "coat_host.h"
+
+namespace coat {
+
+constexpr int kGroup = 128;
+constexpr float kLog2RatioUpperBound = 16.61470984411521f;  // log2(448 * 448 / 2), rounded to fp32
+constexpr float kFltMax = 3.402823466e+38f;
+
+struct AdamArgs {
+    float beta1, beta2, lr, wd, eps;
+    float one_minus_beta1, one_minus_beta2;
+    float correction1, correction2_sqrt;  // 1 - beta1^step, sqrt(1 - beta2^step), evaluated on the host
+    float expand_min;
+};
+
+__device__ __forceinline__ float log2_hw(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// x^y for x >= 0 in the common case 0 < y < inf (x = 0 -> 0 falls out of log2(0) = -inf).
+__device__ __forceinline__ float pow_fast(float x, float y) { return exp2_hw(log2_hw(x) * y); }
+// Same with the IEEE special cases: pow(x, 0) = 1, pow(1, y) = 1, pow(x, +inf) in {0, 1, inf}.
+__device__ __forceinline__ float pow_full(float x, float y) {
+    float t = log2_hw(x) * y;
+    t = (y == 0.0f || x == 1.0f) ? 0.0f : t;
+    return exp2_hw(t);
+}
+
+// The reference's combine step for the minimum: skip the partner when it is zero (NaN > 0 is false too).
+__device__ __forceinline__ float min_skip_zero(float own, float partner) {
+    float a = fabsf(partner);
+    return (a > 0.0f) ? fminf(own, a) : own;
+}
+
+// Group minimum exactly as thread 0 of the reference block ends up holding it, for a[j][i] = |value| of
+// reference thread 32*j + 4*lam + i (FLT_MAX where out of range).  Result valid in the lam == 0 lane.
+__device__ __forceinline__ float reference_tree_min(const float (&a)[4][4]) {
+    float w[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {  // reference warp j: shuffle offsets 16, 8, 4 move 4, 2, 1 lanes; 2 and 1 stay in-lane
+        float s[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float x = a[j][i];
+            x = min_skip_zero(x, dpp_f32<0x104>(x));  // row_shl:4  (lane reads lane+4)
+            x = min_skip_zero(x, dpp_f32<0x102>(x));  // row_shl:2
+            x = min_skip_zero(x, dpp_f32<0x101>(x));  // row_shl:1
+            s[i] = x;
+        }
+        s[0] = min_skip_zero(s[0], s[2]);
+        s[1] = min_skip_zero(s[1], s[3]);
+        w[j] = min_skip_zero(s[0], s[1]);
+    }
+    // block level: threads 0..3 hold w[0..3], every other thread holds 1e9; offsets 16, 8, 4 meet only fillers
+#pragma unroll
+    for (int j = 0; j < 4; j++) w[j] = fminf(w[j], 1e9f);
+    float t0 = min_skip_zero(w[0], w[2]);
+    float t1 = min_skip_zero(w[1], w[3]);
+    return min_skip_zero(t0, t1);
+}
+
+template <int PDT> struct PVec { static constexpr int kBytes = (PDT == kF32) ? 16 : 8; };
+
+template <int PDT> __device__ __forceinline__ void load4(const void* base, int64_t e, int64_t numel, float* o) {
+    if (e + 3 < numel) {
+        if (PDT == kF32) {
+            float4 t = *(const float4*)((const float*)base + e);
+            o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+        } else {
+            uint2 t = *(const uint2*)((const uint16_t*)base + e);
+            o[0] = PDT == kBF16 ? bf16lo(t.x) : f16lo(t.x);
+            o[1] = PDT == kBF16 ? bf16hi(t.x) : f16hi(t.x);
+            o[2] = PDT == kBF16 ? bf16lo(t.y) : f16lo(t.y);
+            o[3] = PDT == kBF16 ? bf16hi(t.y) : f16hi(t.y);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = (e + i < numel) ? load_as_f32<PDT>(base, e + i) : 0.0f;
+    }
+}
+template <int PDT> __device__ __forceinline__ void store4(void* base, int64_t e, int64_t numel, const float* v) {
+    if (e + 3 < numel) {
+        if (PDT == kF32) *(float4*)((float*)base + e) = make_float4(v[0], v[1], v[2], v[3]);
+        else if (PDT == kBF16) *(uint2*)((uint16_t*)base + e) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        else *(uint2*)((uint16_t*)base + e) = make_uint2(f2f16(v[0]) | (f2f16(v[1]) << 16), f2f16(v[2]) | (f2f16(v[3]) << 16));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (e + i < numel) store_from_f32<PDT>(base, e + i, v[i]);
+    }
+}
+__device__ __forceinline__ uint32_t load_codes4(const uint8_t* base, int64_t e, int64_t numel) {
+    if (e + 3 < numel) return *(const uint32_t*)(base + e);
+    uint32_t w = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (e + i < numel) w |= (uint32_t)base[e + i] << (8 * i);
+    return w;
+}
+__device__ __forceinline__ void store_codes4(uint8_t* base, int64_t e, int64_t numel, uint32_t w) {
+    if (e + 3 < numel) *(uint32_t*)(base + e) = w;
+    else {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (e + i < numel) base[e + i] = (uint8_t)(w >> (8 * i));
+    }
+}
+
+template <int PDT, bool EXPAND>
+__global__ __launch_bounds__(256) void k_fp8_adamw(void* __restrict__ params, const void* __restrict__ grads,
+                                                    uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
+                                                    float* __restrict__ expand_m, float* __restrict__ sqrtmm_m,
+                                                    uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
+                                                    float* __restrict__ expand_v, float* __restrict__ sqrtmm_v,
+                                                    AdamArgs A, int64_t numel, int64_t ngroups) {
+    enable_fp8_saturation();
+    const int lane = threadIdx.x & 63, lam = lane & 7;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t gi = wave * 8 + (lane >> 3);
+    if (wave * 8 >= ngroups) return;  // whole wave out of range (wave-uniform)
+    const bool gvalid = gi < ngroups;
+    const int64_t gidx = gvalid ? gi : ngroups - 1;  // clamp: lanes of absent groups redo the last group, stores masked
+    const int64_t e0 = gidx * kGroup + lam * 4;
+    const int64_t lim = gvalid ? numel : 0;  // element validity bound for this lane
+
+    // ---- loads
+    float p[4][4], g[4][4];
+    uint32_t cm[4], cv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        load4<PDT>(params, e0 + 32 * j, numel, p[j]);
+        load4<PDT>(grads, e0 + 32 * j, numel, g[j]);
+        cm[j] = load_codes4(exp_avg, e0 + 32 * j, numel);
+        cv[j] = load_codes4(exp_avg_sq, e0 + 32 * j, numel);
+    }
+    const float sm = scale_m[gidx], sv = scale_v[gidx];
+    float invk_m = 1.0f, invk_v = 1.0f, c_m = 1.0f, c_v = 1.0f;
+    bool odd_pow = false;
+    if (EXPAND) {
+        invk_m = 1 / expand_m[gidx];
+        invk_v = 1 / expand_v[gidx];
+        c_m = sqrtmm_m[gidx];
+        c_v = sqrtmm_v[gidx];
+        // exponents outside (0, inf) need the special cases of powf; decide once per wave
+        bool odd = !(invk_m > 0.0f && invk_m < INFINITY) || !(invk_v > 0.0f && invk_v < INFINITY);
+        odd_pow = __builtin_amdgcn_ballot_w64(odd) != 0;
+    }
+
+    // ---- dequantize, Adam update
+    float m[4][4], v[4][4];
+    float mx_m = 0.0f, mx_v = 0.0f, mn_m = kFltMax, mn_v = kFltMax;
+    bool has_zero = false;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float fm[4], fv[4];
+        fp8x4_to_f32<kE4M3>(cm[j], fm);
+        fp8x4_to_f32<kE4M3>(cv[j], fv);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const bool ok = e0 + 32 * j + i < lim;
+            float em = fm[i] * sm, ev = fv[i] * sv;
+            if (EXPAND) {
+                float pm = odd_pow ? pow_full(fabsf(em), invk_m) : pow_fast(fabsf(em), invk_m);
+                float pv = odd_pow ? pow_full(ev, invk_v) : pow_fast(ev, invk_v);
+                em = copysignf(pm * c_m, em);
+                ev = pv * c_v;
+            }
+            const float gr = g[j][i], pr = p[j][i];
+            em = A.beta1 * em + A.one_minus_beta1 * gr;
+            ev = A.beta2 * ev + (A.one_minus_beta2 * gr) * gr;
+            float denom = (sqrtf(ev) / A.correction2_sqrt + A.eps) * A.correction1;
+            float update = (em / denom) + (A.wd * pr);
+            p[j][i] = pr - (A.lr * update);
+            m[j][i] = em;
+            v[j][i] = ev;
+            float am = ok ? fabsf(em) : 0.0f, av = ok ? fabsf(ev) : 0.0f;
+            mx_m = fmaxf(mx_m, am);
+            mx_v = fmaxf(mx_v, av);
+            if (EXPAND) {
+                mn_m = fminf(mn_m, ok ? am : kFltMax);
+                mn_v = fminf(mn_v, ok ? av : kFltMax);
+                has_zero |= ok && !(am > 0.0f && av > 0.0f);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) store4<PDT>(params, e0 + 32 * j, lim, p[j]);
+
+    // ---- group statistics (8 lanes per group)
+    mx_m = cluster_max<8>(mx_m);
+    mx_v = cluster_max<8>(mx_v);
+    float snew_m, snew_v, k_m = 1.0f, k_v = 1.0f, cn_m = 1.0f, cn_v = 1.0f;
+    bool odd_k = false;
+    if (EXPAND) {
+        if (__builtin_amdgcn_ballot_w64(has_zero) != 0) {
+            // some moment is exactly zero (or NaN): walk the reference's shuffle tree
+            float a[4][4], b[4][4];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const bool ok = e0 + 32 * j + i < lim;
+                    a[j][i] = ok ? fabsf(m[j][i]) : kFltMax;
+                    b[j][i] = ok ? fabsf(v[j][i]) : kFltMax;
+                }
+            mn_m = reference_tree_min(a);
+            mn_v = reference_tree_min(b);
+            // broadcast from the lam == 0 lane of each group
+            mn_m = u2f((uint32_t)__builtin_amdgcn_ds_bpermute((lane & ~7) << 2, (int)f2u(mn_m)));
+            mn_v = u2f((uint32_t)__builtin_amdgcn_ds_bpermute((lane & ~7) << 2, (int)f2u(mn_v)));
+        } else {
+            // all values positive: the tree is a plain minimum, capped by the 1e9 filler of the block level
+            mn_m = fminf(-cluster_max<8>(-mn_m), 1e9f);
+            mn_v = fminf(-cluster_max<8>(-mn_v), 1e9f);
+        }
+        // "+ 1e-30" is a double-precision add narrowed to float in the reference
+        const float Mx_m = (float)((double)mx_m + 1e-30), Mn_m = (float)((double)mn_m + 1e-30);
+        const float Mx_v = (float)((double)mx_v + 1e-30), Mn_v = (float)((double)mn_v + 1e-30);
+        const float ratio_m = Mx_m / Mn_m, ratio_v = Mx_v / Mn_v;
+        cn_m = sqrtf(Mx_m) * sqrtf(Mn_m);
+        cn_v = sqrtf(Mx_v) * sqrtf(Mn_v);
+        k_m = floorf((kLog2RatioUpperBound / log2_hw(ratio_m)) * A.expand_min) / A.expand_min;
+        k_v = floorf((kLog2RatioUpperBound / log2_hw(ratio_v)) * A.expand_min) / A.expand_min;
+        snew_m = pow_full(Mx_m / cn_m, k_m) / 448.0f;
+        snew_v = pow_full(Mx_v / cn_v, k_v) / 448.0f;
+        bool odd = !(k_m > 0.0f && k_m < INFINITY) || !(k_v > 0.0f && k_v < INFINITY);
+        odd_k = __builtin_amdgcn_ballot_w64(odd) != 0;
+    } else {
+        snew_m = (float)((double)mx_m + 1e-20) / 448.0f;
+        snew_v = (float)((double)mx_v + 1e-20) / 448.0f;
+    }
+
+    // ---- requantize
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float qm[4], qv[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float em = m[j][i], ev = v[j][i];
+            if (EXPAND) {
+                float xm = fabsf(em) / cn_m, xv = ev / cn_v;
+                float pm = odd_k ? pow_full(xm, k_m) : pow_fast(xm, k_m);
+                float pv = odd_k ? pow_full(xv, k_v) : pow_fast(xv, k_v);
+                em = copysignf(pm, em);
+                ev = pv;
+            }
+            qm[i] = em / snew_m;
+            qv[i] = ev / snew_v;
+        }
+        store_codes4(exp_avg, e0 + 32 * j, lim, cvt4_fp8<kE4M3>(qm[0], qm[1], qm[2], qm[3]));
+        store_codes4(exp_avg_sq, e0 + 32 * j, lim, cvt4_fp8<kE4M3>(qv[0], qv[1], qv[2], qv[3]));
+    }
+    if (gvalid && lam == 0) {
+        scale_m[gi] = snew_m;
+        scale_v[gi] = snew_v;
+        if (EXPAND) {
+            expand_m[gi] = k_m;
+            expand_v[gi] = k_v;
+            sqrtmm_m[gi] = cn_m;
+            sqrtmm_v[gi] = cn_v;
+        }
+    }
+}
+
+}  // namespace coat
+
+using namespace coat;
+
+static int adamw_common(void* params, const void* grads, int p_dtype, void* exp_avg, float* scale_m, float* expand_m,
+                        float* sqrtmm_m, void* exp_avg_sq, float* scale_v, float* expand_v, float* sqrtmm_v,
+                        float beta1, float beta2, float lr, float wd, float eps, int step, int qgroup_size,
+                        int expand_min, bool expand, int64_t numel, int64_t n_scale, void* stream) {
+    if (qgroup_size != kGroup) return COAT_EQGROUP;  // "Only Support 128 per-group quantization currently"
+    if (numel < 0) return COAT_EINVAL;
+    const int64_t ngroups = (numel + kGroup - 1) / kGroup;
+    if (n_scale != ngroups) return COAT_ESHAPE;  // AT_ASSERTM(grid_dim == scale_exp_avg.numel())
+    if (numel == 0) return COAT_OK;
+    if (!params || !grads || !exp_avg || !exp_avg_sq || !scale_m || !scale_v) return COAT_EINVAL;
+    if (expand && (!expand_m || !expand_v || !sqrtmm_m || !sqrtmm_v)) return COAT_EINVAL;
+    if (!coat_aligned16(params) || !coat_aligned16(grads) || !coat_aligned16(exp_avg) || !coat_aligned16(exp_avg_sq))
+        return COAT_EALIGN;
+    AdamArgs A;
+    A.beta1 = beta1; A.beta2 = beta2; A.lr = lr; A.wd = wd; A.eps = eps;
+    A.one_minus_beta1 = 1 - beta1;
+    A.one_minus_beta2 = 1 - beta2;
+    // correctly rounded powf(beta, step): double pow rounded once
+    A.correction1 = 1.0f - (float)pow((double)beta1, (double)(float)step);
+    A.correction2_sqrt = sqrtf(1.0f - (float)pow((double)beta2, (double)(float)step));
+    A.expand_min = (float)expand_min;
+    const int64_t waves = (ngroups + 7) / 8;
+    const int64_t blocks = (waves + 3) / 4;
+    hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(PDT)                                                                                                   \
+    if (expand)                                                                                                       \
+        hipLaunchKernelGGL((k_fp8_adamw<PDT, true>), dim3((unsigned)blocks), dim3(256), 0, st, params, grads,         \
+                           (uint8_t*)exp_avg, scale_m, expand_m, sqrtmm_m, (uint8_t*)exp_avg_sq, scale_v, expand_v,   \
+                           sqrtmm_v, A, numel, ngroups);                                                              \
+    else                                                                                                              \
+        hipLaunchKernelGGL((k_fp8_adamw<PDT, false>), dim3((unsigned)blocks), dim3(256), 0, st, params, grads,        \
+                           (uint8_t*)exp_avg, scale_m, nullptr, nullptr, (uint8_t*)exp_avg_sq, scale_v, nullptr,      \
+                           nullptr, A, numel, ngroups);
+    switch (p_dtype) {
+        case COAT_F32: LAUNCH(kF32); break;
+        case COAT_BF16: LAUNCH(kBF16); break;
+        case COAT_F16: LAUNCH(kF16); break;
+        default: return COAT_EDTYPE;
+    }
+#undef LAUNCH
+    return coat_launch_status();
+}
+
+extern "C" int coat_fp8_adamw_expand_step(void* params, const void* grads, int p_dtype, void* exp_avg,
+                                          float* scale_exp_avg, float* expand_exp_avg, float* sqrtminmax_exp_avg,
+                                          void* exp_avg_sq, float* scale_exp_avg_sq, float* expand_exp_avg_sq,
+                                          float* sqrtminmax_exp_avg_sq, float beta1, float beta2, float lr, float wd,
+                                          float eps, int step, int qgroup_size, int expand_min, int64_t numel,
+                                          int64_t n_scale, void* stream) {
+    return adamw_common(params, grads, p_dtype, exp_avg, scale_exp_avg, expand_exp_avg, sqrtminmax_exp_avg, exp_avg_sq,
+                        scale_exp_avg_sq, expand_exp_avg_sq, sqrtminmax_exp_avg_sq, beta1, beta2, lr, wd, eps, step,
+                        qgroup_size, expand_min, true, numel, n_scale, stream);
+}
+
+extern "C" int coat_fp8_adamw_step(void* params, const void* grads, int p_dtype, void* exp_avg, float* scale_exp_avg,
+                                   void* exp_avg_sq, float* scale_exp_avg_sq, float beta1, float beta2, float lr,
+                                   float wd, float eps, int step, int qgroup_size, int64_t numel, int64_t n_scale,
+                                   void* stream) {
+    return adamw_common(params, grads, p_dtype, exp_avg, scale_exp_avg, nullptr, nullptr, exp_avg_sq, scale_exp_avg_sq,
+                        nullptr, nullptr, beta1, beta2, lr, wd, eps, step, qgroup_size, 0, false, numel, n_scale, stream);
+}

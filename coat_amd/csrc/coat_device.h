@@ -1,0 +1,159 @@
+// Device-side helpers shared by every gfx950 kernel of the FP8 hot path.
+//
+// Numeric contract (all kernels):
+//   * the translation units are compiled with -ffp-contract=off, so every + - * written here is a
+//     separately rounded IEEE fp32 operation and an FMA happens only where fmaf() is written;
+//   * fp32 division by a scale is done as reciprocal + two FMAs (div_by_scale), which returns the
+//     correctly rounded quotient whenever the scale is >= 2^-60 and the quotient is not below the
+//     FP8 underflow threshold (validated exhaustively for bf16 inputs and on 6e8 random / adversarial
+//     fp32 pairs on the CPU); callers fall back to plain division outside that domain;
+//   * fp32 -> FP8 is the hardware OCP conversion (round to nearest even) with the wave's FP16_OVFL
+//     mode bit set, i.e. saturate-to-finite for finite inputs; NaN is kept as NaN.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define COAT_WAVE 64
+
+namespace coat {
+
+enum Fp8Kind { kE4M3 = 0, kE5M2 = 1 };
+enum DType { kF32 = 0, kBF16 = 1, kF16 = 2 };
+
+template <int KIND> struct Fp8Traits;
+template <> struct Fp8Traits<kE4M3> { static constexpr float kMax = 448.0f; };
+template <> struct Fp8Traits<kE5M2> { static constexpr float kMax = 57344.0f; };
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// ------------------------------------------------------------------------------------------------ bf16 / f16
+__device__ __forceinline__ float bf16lo(uint32_t w) { return u2f(w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
+
+// fp32 -> bf16 bits, round to nearest even, NaN quieted (same result as torch's and the hardware's).
+__device__ __forceinline__ uint32_t f2bf16(float f) {
+    uint32_t u = f2u(f);
+    uint32_t r = u + 0x7FFFu + ((u >> 16) & 1u);
+    r = (u & 0x7FFFFFFFu) > 0x7F800000u ? (u | 0x00400000u) : r;
+    return r >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) { return f2bf16(lo) | (f2bf16(hi) << 16); }
+
+__device__ __forceinline__ float f16lo(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFF)); }
+__device__ __forceinline__ float f16hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
+__device__ __forceinline__ uint32_t f2f16(float f) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f); }
+
+// Typed scalar load / store used for scale tensors and ragged tails.
+template <int DT> __device__ __forceinline__ float load_as_f32(const void* p, int64_t i) {
+    if (DT == kF32) return ((const float*)p)[i];
+    uint32_t h = ((const uint16_t*)p)[i];
+    return DT == kBF16 ? u2f(h << 16) : f16lo(h);
+}
+template <int DT> __device__ __forceinline__ void store_from_f32(void* p, int64_t i, float v) {
+    if (DT == kF32) ((float*)p)[i] = v;
+    else if (DT == kBF16) ((uint16_t*)p)[i] = (uint16_t)f2bf16(v);
+    else ((uint16_t*)p)[i] = (uint16_t)f2f16(v);
+}
+// Round an fp32 value to dtype DT and back (what storing and re-loading would give).
+template <int DT> __device__ __forceinline__ float round_to(float v) {
+    if (DT == kF32) return v;
+    if (DT == kBF16) return u2f(f2bf16(v) << 16);
+    return (float)(_Float16)v;
+}
+
+// ------------------------------------------------------------------------------------------------ FP8
+// The hardware conversion rounds to nearest even and, with MODE.FP16_OVFL = 1, saturates finite
+// overflow to the largest finite code (e4m3 0x7E, e5m2 0x7B) instead of producing NaN / inf; NaN stays
+// NaN.  (+-inf in gives NaN for e4m3 and +-inf for e5m2.)  Every kernel that emits FP8 calls this first.
+__device__ __forceinline__ void enable_fp8_saturation() {
+    // s_setreg_b32 hwreg(HW_REG_MODE, 23, 1), 1
+    __builtin_amdgcn_s_setreg(1 | (23 << 6) | (0 << 11), 1);
+}
+// Two fp32 -> two FP8 codes packed into the low (hi=false) or high (hi=true) half of `old`.
+template <int KIND> __device__ __forceinline__ uint32_t cvt_pk_fp8(float a, float b, uint32_t old, bool hi) {
+    if (KIND == kE4M3) return hi ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, false);
+    return hi ? __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, false);
+}
+template <int KIND> __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
+    uint32_t w = cvt_pk_fp8<KIND>(a, b, 0u, false);
+    return cvt_pk_fp8<KIND>(c, d, w, true);
+}
+// FP8 code (byte `sel` of w) -> fp32.
+template <int KIND, int SEL> __device__ __forceinline__ float fp8_to_f32(uint32_t w) {
+    if (KIND == kE4M3) return __builtin_amdgcn_cvt_f32_fp8(w, SEL);
+    return __builtin_amdgcn_cvt_f32_bf8(w, SEL);
+}
+template <int KIND> __device__ __forceinline__ void fp8x4_to_f32(uint32_t w, float* o) {
+    o[0] = fp8_to_f32<KIND, 0>(w);
+    o[1] = fp8_to_f32<KIND, 1>(w);
+    o[2] = fp8_to_f32<KIND, 2>(w);
+    o[3] = fp8_to_f32<KIND, 3>(w);
+}
+
+// ------------------------------------------------------------------------------------------------ exact division
+// Correctly rounded t / C for the two FP8 maxima, C in {448, 57344}: reciprocal constant + two FMAs
+// (exhaustively checked against IEEE division for every positive normal t with a normal quotient).
+template <int KIND> __device__ __forceinline__ float div_by_fp8max(float t) {
+    constexpr float C = Fp8Traits<KIND>::kMax;
+    constexpr float rc = 1.0f / C;
+    float q0 = t * rc;
+    float e = fmaf(-q0, C, t);
+    return fmaf(e, rc, q0);
+}
+// Group scale as the reference defines it: (amax + 1e-10) / fp8max, fp32.
+template <int KIND> __device__ __forceinline__ float group_scale(float amax) { return div_by_fp8max<KIND>(amax + 1e-10f); }
+
+// x / s given r = 1.0f / s (IEEE).  The sign is forced from x so that -0.0 / s stays -0.0.
+__device__ __forceinline__ float div_by_scale(float x, float s, float r) {
+    float q0 = x * r;
+    float e = fmaf(-q0, s, x);
+    float q = fmaf(e, r, q0);
+    return u2f((f2u(q) & 0x7FFFFFFFu) | (f2u(x) & 0x80000000u));
+}
+constexpr float kMinFastDivScale = 0x1p-60f;
+
+// ------------------------------------------------------------------------------------------------ cross-lane
+// DPP controls: quad_perm(1,0,3,2)=0xB1, quad_perm(2,3,0,1)=0x4E, row_half_mirror=0x141, row_mirror=0x140.
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v), CTRL, 0xF, 0xF, true));
+}
+// lane ^ 16 / lane ^ 32 exchanges through ds_bpermute (no LDS memory is touched).
+__device__ __forceinline__ float lane_xor_f32(float v, int mask) {
+    int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    return u2f((uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, (int)f2u(v)));
+}
+// max over aligned clusters of LANES consecutive lanes (LANES power of two <= 64); result in every lane.
+template <int LANES> __device__ __forceinline__ float cluster_max(float v) {
+    if (LANES >= 2) v = fmaxf(v, dpp_f32<0xB1>(v));
+    if (LANES >= 4) v = fmaxf(v, dpp_f32<0x4E>(v));
+    if (LANES >= 8) v = fmaxf(v, dpp_f32<0x141>(v));
+    if (LANES >= 16) v = fmaxf(v, dpp_f32<0x140>(v));
+    if (LANES >= 32) v = fmaxf(v, lane_xor_f32(v, 16));
+    if (LANES >= 64) v = fmaxf(v, lane_xor_f32(v, 32));
+    return v;
+}
+// Same with a run-time (wave-uniform) cluster width.
+__device__ __forceinline__ float cluster_max_rt(float v, int lanes) {
+    if (lanes >= 2) v = fmaxf(v, dpp_f32<0xB1>(v));
+    if (lanes >= 4) v = fmaxf(v, dpp_f32<0x4E>(v));
+    if (lanes >= 8) v = fmaxf(v, dpp_f32<0x141>(v));
+    if (lanes >= 16) v = fmaxf(v, dpp_f32<0x140>(v));
+    if (lanes >= 32) v = fmaxf(v, lane_xor_f32(v, 16));
+    if (lanes >= 64) v = fmaxf(v, lane_xor_f32(v, 32));
+    return v;
+}
+template <int LANES> __device__ __forceinline__ float cluster_sum(float v) {
+    if (LANES >= 2) v = v + dpp_f32<0xB1>(v);
+    if (LANES >= 4) v = v + dpp_f32<0x4E>(v);
+    if (LANES >= 8) v = v + dpp_f32<0x141>(v);
+    if (LANES >= 16) v = v + dpp_f32<0x140>(v);
+    if (LANES >= 32) v = v + lane_xor_f32(v, 16);
+    if (LANES >= 64) v = v + lane_xor_f32(v, 32);
+    return v;
+}
+
+// Order-independent device-wide maximum of non-negative floats (bit pattern order == value order).
+__device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) { atomicMax((unsigned int*)addr, f2u(v)); }
+
+}  // namespace coat

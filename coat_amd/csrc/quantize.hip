@@ -1,0 +1,538 @@
+// Streaming FP8 quantize family for gfx950: per-group quantize (+transpose), per-group scales with a
+// device-wide maximum, per-tensor division (+transpose), byte transpose, dequantize, abs-max.
+//
+// All of these are HBM-bound.  Layout rules used throughout:
+//   * every lane moves 16 bytes per global load (8 two-byte elements or 4 fp32), consecutive lanes
+//     touch consecutive 16-byte chunks, so a wave instruction covers 1 KiB of contiguous memory;
+//   * a 1 x QB group is QB/VEC consecutive lanes; its amax is a DPP reduction inside one 16-lane row;
+//   * transposed outputs are staged through LDS tiles so that global stores are 16 bytes per lane
+//     with neighbouring lanes writing neighbouring chunks of one output row.
+#include "coat_device.h"
+#include "coat_host.h"
+
+namespace coat {
+
+template <int XDT> struct VecOf { static constexpr int kVec = (XDT == kF32) ? 4 : 8; };
+
+// 16-byte load of VEC elements starting at element index e (e % VEC == 0) converted to fp32.
+template <int XDT> __device__ __forceinline__ void load_vec(const void* x, int64_t e, float* v) {
+    if (XDT == kF32) {
+        float4 t = *(const float4*)((const float*)x + e);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else {
+        uint4 t = *(const uint4*)((const uint16_t*)x + e);
+        uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = XDT == kBF16 ? bf16lo(w[i]) : f16lo(w[i]);
+            v[2 * i + 1] = XDT == kBF16 ? bf16hi(w[i]) : f16hi(w[i]);
+        }
+    }
+}
+
+template <int VEC> __device__ __forceinline__ float vec_amax(const float* v) {
+    float a = fmaxf(fabsf(v[0]), fabsf(v[1]));
+#pragma unroll
+    for (int i = 2; i < VEC; i++) a = fmaxf(a, fabsf(v[i]));
+    return a;
+}
+
+// VEC fp32 -> VEC FP8 codes (VEC/4 dwords), dividing by s through the reciprocal r.
+template <int KIND, int VEC> __device__ __forceinline__ void quantize_vec(const float* v, float s, float r, uint32_t* out) {
+#pragma unroll
+    for (int i = 0; i < VEC / 4; i++)
+        out[i] = cvt4_fp8<KIND>(div_by_scale(v[4 * i], s, r), div_by_scale(v[4 * i + 1], s, r),
+                                div_by_scale(v[4 * i + 2], s, r), div_by_scale(v[4 * i + 3], s, r));
+}
+template <int KIND, int VEC> __device__ __forceinline__ void quantize_vec_slow(const float* v, float s, uint32_t* out) {
+#pragma unroll
+    for (int i = 0; i < VEC / 4; i++)
+        out[i] = cvt4_fp8<KIND>(v[4 * i] / s, v[4 * i + 1] / s, v[4 * i + 2] / s, v[4 * i + 3] / s);
+}
+template <int VEC> __device__ __forceinline__ void store_codes(void* q, int64_t e, const uint32_t* c) {
+    if (VEC == 8) *(uint2*)((uint8_t*)q + e) = make_uint2(c[0], c[1]);
+    else *(uint32_t*)((uint8_t*)q + e) = c[0];
+}
+
+// ------------------------------------------------------------------------------------------------
+// K1 / K3: per-group quantize over the flat [M*N] array (groups never straddle rows since N % QB == 0).
+//   WRITE_Q   store the FP8 codes
+//   WRITE_S   store the per-group scales
+//   WITH_MAX  accumulate the maximum fp32 group scale into *s_max (atomic, order independent)
+template <int XDT, int SDT, int KIND, int QB, bool WRITE_Q, bool WRITE_S, bool WITH_MAX, int UNROLL>
+__global__ __launch_bounds__(256) void k_quantize_pg(const void* __restrict__ x, void* __restrict__ q,
+                                                      void* __restrict__ s_out, float* __restrict__ s_max,
+                                                      int64_t nvec, int qb_rt) {
+    constexpr int VEC = VecOf<XDT>::kVec;
+    const int LPG = (QB ? QB : qb_rt) / VEC;  // lanes per group (QB == 0: group size given at run time)
+    enable_fp8_saturation();
+    const int64_t base = ((int64_t)blockIdx.x * UNROLL) * 256 + threadIdx.x;
+    float v[UNROLL][VEC];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        int64_t i = base + (int64_t)u * 256;
+        ok[u] = i < nvec;
+        if (ok[u]) load_vec<XDT>(x, i * VEC, v[u]);
+        else {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) v[u][k] = 0.0f;
+        }
+    }
+    float wmax = 0.0f;
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        int64_t i = base + (int64_t)u * 256;
+        float amax = QB ? cluster_max<(QB ? QB : 16) / VEC>(vec_amax<VEC>(v[u])) : cluster_max_rt(vec_amax<VEC>(v[u]), LPG);
+        float s = group_scale<KIND>(amax);
+        if (WITH_MAX) wmax = fmaxf(wmax, ok[u] ? s : 0.0f);
+        if (WRITE_Q) {
+            float r = 1.0f / s;
+            uint32_t c[VEC / 4];
+            quantize_vec<KIND, VEC>(v[u], s, r, c);
+            if (ok[u]) store_codes<VEC>(q, i * VEC, c);
+        }
+        if (WRITE_S && ok[u] && (threadIdx.x % LPG) == 0) store_from_f32<SDT>(s_out, i / LPG, s);
+    }
+    if (WITH_MAX) {
+        wmax = cluster_max<64>(wmax);
+        if ((threadIdx.x & 63) == 0) atomic_max_nonneg(s_max, wmax);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Q5: max|x| over a flat array (atomic into *amax, which the caller zeroed).
+template <int XDT, int UNROLL>
+__global__ __launch_bounds__(256) void k_absmax(const void* __restrict__ x, float* __restrict__ amax, int64_t nvec,
+                                                 int64_t numel) {
+    constexpr int VEC = VecOf<XDT>::kVec;
+    const int64_t base = ((int64_t)blockIdx.x * UNROLL) * 256 + threadIdx.x;
+    float m = 0.0f;
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        int64_t i = base + (int64_t)u * 256;
+        if (i < nvec) {
+            float v[VEC];
+            load_vec<XDT>(x, i * VEC, v);
+            m = fmaxf(m, vec_amax<VEC>(v));
+        }
+    }
+    // ragged tail (numel % VEC elements), handled by the first threads of block 0
+    if (blockIdx.x == 0 && threadIdx.x < numel - nvec * VEC) m = fmaxf(m, fabsf(load_as_f32<XDT>(x, nvec * VEC + threadIdx.x)));
+    m = cluster_max<64>(m);
+    if ((threadIdx.x & 63) == 0) atomic_max_nonneg(amax, m);
+}
+
+// ------------------------------------------------------------------------------------------------
+// K4: per-tensor division over the flat array, q = fp8(x / float(*s)).
+template <int XDT, int SDT, int KIND, int UNROLL>
+__global__ __launch_bounds__(256) void k_division(const void* __restrict__ x, const void* __restrict__ s_ptr,
+                                                   void* __restrict__ q, int64_t nvec, int64_t numel) {
+    constexpr int VEC = VecOf<XDT>::kVec;
+    enable_fp8_saturation();
+    const float s = load_as_f32<SDT>(s_ptr, 0);
+    const float r = 1.0f / s;
+    const bool fast = s >= kMinFastDivScale && s < 0x1p100f;  // uniform across the grid
+    const int64_t base = ((int64_t)blockIdx.x * UNROLL) * 256 + threadIdx.x;
+    float v[UNROLL][VEC];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        int64_t i = base + (int64_t)u * 256;
+        if (i < nvec) load_vec<XDT>(x, i * VEC, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        int64_t i = base + (int64_t)u * 256;
+        if (i < nvec) {
+            uint32_t c[VEC / 4];
+            if (fast) quantize_vec<KIND, VEC>(v[u], s, r, c);
+            else quantize_vec_slow<KIND, VEC>(v[u], s, c);
+            store_codes<VEC>(q, i * VEC, c);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < numel - nvec * VEC) {
+        int64_t e = nvec * VEC + threadIdx.x;
+        uint32_t w = cvt_pk_fp8<KIND>(load_as_f32<XDT>(x, e) / s, 0.0f, 0u, false);
+        ((uint8_t*)q)[e] = (uint8_t)(w & 0xFF);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// K7: y = bf16(float(q) * float(s_group)).  One lane: 16 codes (one 16-byte load), two 16-byte stores.
+template <int SDT, int KIND>
+__global__ __launch_bounds__(256) void k_dequantize(const void* __restrict__ q, const void* __restrict__ s,
+                                                     void* __restrict__ y, int64_t nchunk, int QB) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // chunk of 16 elements
+    if (i >= nchunk) return;
+    uint4 c = *(const uint4*)((const uint8_t*)q + i * 16);
+    float sc = load_as_f32<SDT>(s, (i * 16) / QB);
+    uint32_t w[4] = {c.x, c.y, c.z, c.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float f[4];
+        fp8x4_to_f32<KIND>(w[k], f);
+        o[2 * k] = pack_bf16x2(f[0] * sc, f[1] * sc);
+        o[2 * k + 1] = pack_bf16x2(f[2] * sc, f[3] * sc);
+    }
+    uint4* yo = (uint4*)((uint16_t*)y + i * 16);
+    yo[0] = make_uint4(o[0], o[1], o[2], o[3]);
+    yo[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Byte-tile transpose helpers.  A block owns a TM x 64 tile of FP8 codes in LDS (row pitch 17 dwords so
+// that the column-quad reads below hit every bank exactly twice per wave, the minimum for 256 bytes).
+constexpr int kTileN = 64;
+constexpr int kPitchDw = kTileN / 4 + 1;
+
+// 4x4 byte transpose: r[j] holds row j (4 columns); returns c[j] = column j (4 rows).
+__device__ __forceinline__ void transpose4x4_bytes(const uint32_t* r, uint32_t* c) {
+    // v_perm_b32(hi, lo, sel): byte k of the result = byte sel[k] of {hi:7..4, lo:3..0}
+    uint32_t t0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);  // r0b0 r1b0 r0b1 r1b1
+    uint32_t t1 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);  // r2b0 r3b0 r2b1 r3b1
+    uint32_t t2 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);  // r0b2 r1b2 r0b3 r1b3
+    uint32_t t3 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    c[0] = __builtin_amdgcn_perm(t1, t0, 0x05040100u);  // r0b0 r1b0 r2b0 r3b0
+    c[1] = __builtin_amdgcn_perm(t1, t0, 0x07060302u);
+    c[2] = __builtin_amdgcn_perm(t3, t2, 0x05040100u);
+    c[3] = __builtin_amdgcn_perm(t3, t2, 0x07060302u);
+}
+
+// Write the transposed TM x 64 byte tile held in LDS to yt[N, M] (row pitch M bytes).
+// Lane job = (column quad nq, 16-row chunk mc): 16 dword reads, four 16-byte stores.
+template <int TM>
+__device__ __forceinline__ void store_tile_transposed(const uint32_t* tile, void* __restrict__ yt, int64_t M, int64_t N,
+                                                      int64_t m0, int64_t n0) {
+    constexpr int MC = TM / 16;              // 16-row chunks per tile
+    constexpr int JOBS = MC * (kTileN / 4);  // (mc, nq) pairs
+    for (int job = threadIdx.x; job < JOBS; job += 256) {
+        int mc = job % MC, nq = job / MC;
+        int64_t m = m0 + mc * 16, n = n0 + nq * 4;
+        if (m >= M || n >= N) continue;  // M % 16 == 0 and N % 4 == 0: chunks are whole or absent
+        uint32_t col[4][4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            uint32_t r[4], c[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) r[j] = tile[(mc * 16 + b * 4 + j) * kPitchDw + nq];
+            transpose4x4_bytes(r, c);
+#pragma unroll
+            for (int j = 0; j < 4; j++) col[j][b] = c[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            *(uint4*)((uint8_t*)yt + (n + j) * M + m) = make_uint4(col[j][0], col[j][1], col[j][2], col[j][3]);
+    }
+}
+
+// K5 / K6: q = fp8(x / *s) and/or its transpose; RAW = input already FP8 bytes (pure transpose).
+// Requires N % 16 == 0 and M % 16 == 0.
+template <int XDT, int SDT, int KIND, bool RAW, bool WRITE_Q, int TM>
+__global__ __launch_bounds__(256) void k_division_transpose(const void* __restrict__ x, const void* __restrict__ s_ptr,
+                                                             void* __restrict__ q, void* __restrict__ qt, int64_t M,
+                                                             int64_t N) {
+    __shared__ uint32_t tile[TM * kPitchDw];
+    enable_fp8_saturation();
+    const int64_t tiles_n = (N + kTileN - 1) / kTileN;
+    const int64_t m0 = (blockIdx.x / tiles_n) * TM, n0 = (blockIdx.x % tiles_n) * kTileN;
+    float s = 1.0f, r = 1.0f;
+    bool fast = true;
+    if (!RAW) {
+        s = load_as_f32<SDT>(s_ptr, 0);
+        r = 1.0f / s;
+        fast = s >= kMinFastDivScale && s < 0x1p100f;
+    }
+    // phase 1: each job converts 16 consecutive elements of one row into 4 dwords of the tile
+    constexpr int JOBS = TM * (kTileN / 16);
+    for (int job = threadIdx.x; job < JOBS; job += 256) {
+        int row = job / (kTileN / 16), c16 = job % (kTileN / 16);
+        int64_t m = m0 + row, n = n0 + c16 * 16;
+        uint32_t c[4] = {0, 0, 0, 0};
+        if (m < M && n < N) {
+            if (RAW) {
+                uint4 t = *(const uint4*)((const uint8_t*)x + m * N + n);
+                c[0] = t.x; c[1] = t.y; c[2] = t.z; c[3] = t.w;
+            } else {
+                constexpr int VEC = VecOf<XDT>::kVec;
+#pragma unroll
+                for (int h = 0; h < 16 / VEC; h++) {
+                    float v[VEC];
+                    load_vec<XDT>(x, m * N + n + h * VEC, v);
+                    if (fast) quantize_vec<KIND, VEC>(v, s, r, c + h * (VEC / 4));
+                    else quantize_vec_slow<KIND, VEC>(v, s, c + h * (VEC / 4));
+                }
+                if (WRITE_Q) *(uint4*)((uint8_t*)q + m * N + n) = make_uint4(c[0], c[1], c[2], c[3]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) tile[row * kPitchDw + c16 * 4 + k] = c[k];
+    }
+    __syncthreads();
+    store_tile_transposed<TM>(tile, qt, M, N, m0, n0);
+}
+
+// ------------------------------------------------------------------------------------------------
+// K2: per-group quantize of x and of x^T in one pass over x.
+// Tile = TM x 64 fp32 values in LDS (pitch 65 words).  Phase 1 does the row-direction groups exactly like
+// k_quantize_pg and parks the fp32 values in LDS; phase 2 gives every lane a (column, 16-row chunk) job:
+// amax over the chunk (and over QB/16 neighbouring lanes), quantize, one 16-byte store into qt.
+template <int XDT, int SDT, int KIND, int QB, int TM>
+__global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restrict__ x, void* __restrict__ q,
+                                                             void* __restrict__ s_out, void* __restrict__ qt,
+                                                             void* __restrict__ st_out, int64_t M, int64_t N) {
+    constexpr int VEC = VecOf<XDT>::kVec;
+    constexpr int LPG = QB / VEC;
+    constexpr int PITCH = kTileN + 1;
+    static_assert(QB <= kTileN && TM % QB == 0, "tile must hold whole groups in both directions");
+    __shared__ float tile[TM * PITCH];
+    enable_fp8_saturation();
+    const int64_t tiles_n = (N + kTileN - 1) / kTileN;
+    const int64_t m0 = (blockIdx.x / tiles_n) * TM, n0 = (blockIdx.x % tiles_n) * kTileN;
+    const int64_t SN = N / QB, SM = M / QB;
+
+    // phase 1: jobs of VEC consecutive elements; a row of the tile is 64/VEC jobs (a multiple of LPG)
+    constexpr int JPR = kTileN / VEC;
+    constexpr int JOBS = TM * JPR;
+    static_assert(JOBS % 256 == 0, "phase 1 keeps all lanes of a group in the same iteration");
+    for (int job = threadIdx.x; job < JOBS; job += 256) {
+        int row = job / JPR, cv = job % JPR;
+        int64_t m = m0 + row, n = n0 + cv * VEC;
+        bool ok = m < M && n < N;  // N % QB == 0: a group is inside or outside as a whole
+        float v[VEC];
+        if (ok) load_vec<XDT>(x, m * N + n, v);
+        else {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) v[k] = 0.0f;
+        }
+        float amax = cluster_max<LPG>(vec_amax<VEC>(v));
+        float s = group_scale<KIND>(amax);
+        float r = 1.0f / s;
+        uint32_t c[VEC / 4];
+        quantize_vec<KIND, VEC>(v, s, r, c);
+        if (ok) {
+            store_codes<VEC>(q, m * N + n, c);
+            if ((threadIdx.x % LPG) == 0) store_from_f32<SDT>(s_out, m * SN + n / QB, s);
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; k++) tile[row * PITCH + cv * VEC + k] = v[k];
+    }
+    __syncthreads();
+
+    // phase 2: job = (column n, 16-row chunk mc), mc fastest so that neighbouring lanes write
+    // neighbouring 16-byte pieces of one qt row; groups of QB rows are QB/16 neighbouring lanes.
+    constexpr int MC = TM / 16;
+    constexpr int LPG_T = QB / 16;
+    constexpr int JOBS2 = MC * kTileN;
+    static_assert(JOBS2 % 256 == 0, "phase 2 keeps all lanes of a group in the same iteration");
+    for (int job = threadIdx.x; job < JOBS2; job += 256) {
+        int mc = job % MC, col = job / MC;
+        int64_t m = m0 + mc * 16, n = n0 + col;
+        bool ok = m < M && n < N;  // M % QB == 0: whole groups again
+        float v[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) v[i] = tile[(mc * 16 + i) * PITCH + col];
+        float amax = cluster_max<LPG_T>(vec_amax<16>(v));
+        float s = group_scale<KIND>(amax);
+        float r = 1.0f / s;
+        uint32_t c[4];
+        quantize_vec<KIND, 16>(v, s, r, c);
+        if (ok) {
+            *(uint4*)((uint8_t*)qt + n * M + m) = make_uint4(c[0], c[1], c[2], c[3]);
+            if ((mc % LPG_T) == 0) store_from_f32<SDT>(st_out, n * SM + m / QB, s);
+        }
+    }
+}
+
+}  // namespace coat
+
+// ================================================================================================ C ABI
+using namespace coat;
+
+#define DISPATCH_XDT(XDT_VAR, ...)                                   \
+    switch (XDT_VAR) {                                               \
+        case COAT_F32: { constexpr int XDT = kF32; __VA_ARGS__; break; }   \
+        case COAT_BF16: { constexpr int XDT = kBF16; __VA_ARGS__; break; } \
+        case COAT_F16: { constexpr int XDT = kF16; __VA_ARGS__; break; }   \
+        default: return COAT_EDTYPE;                                 \
+    }
+#define DISPATCH_SDT(SDT_VAR, ...)                                   \
+    switch (SDT_VAR) {                                               \
+        case COAT_F32: { constexpr int SDT = kF32; __VA_ARGS__; break; }   \
+        case COAT_BF16: { constexpr int SDT = kBF16; __VA_ARGS__; break; } \
+        case COAT_F16: { constexpr int SDT = kF16; __VA_ARGS__; break; }   \
+        default: return COAT_EDTYPE;                                 \
+    }
+#define DISPATCH_KIND(KIND_VAR, ...)                                 \
+    switch (KIND_VAR) {                                              \
+        case COAT_E4M3: { constexpr int KIND = kE4M3; __VA_ARGS__; break; } \
+        case COAT_E5M2: { constexpr int KIND = kE5M2; __VA_ARGS__; break; } \
+        default: return COAT_EINVAL;                                 \
+    }
+/* QB 16 (the activation group size) is compiled in; 32 / 64 / 128 share one run-time variant (QB = 0). */
+#define DISPATCH_QB(QB_VAR, ...)                                     \
+    switch (QB_VAR) {                                                \
+        case 16: { constexpr int QB = 16; const int QB_RT = 16; (void)QB_RT; __VA_ARGS__; break; } \
+        case 32: case 64: case 128: { const int QB_RT = QB_VAR; constexpr int QB = 0; (void)QB_RT; __VA_ARGS__; break; } \
+        default: return COAT_ESHAPE;                                 \
+    }
+
+static inline int check_mn(int64_t M, int64_t N, int QB) {
+    if (M < 0 || N < 0) return COAT_EINVAL;
+    if (QB <= 0 || N % QB != 0) return COAT_ESHAPE;
+    return COAT_OK;
+}
+
+template <int XDT, int SDT, int KIND, int QB, bool WQ, bool WS, bool WMAX>
+static int launch_quantize_pg(const void* x, void* q, void* s, float* s_max, int64_t numel, int qb, hipStream_t st) {
+    constexpr int VEC = VecOf<XDT>::kVec;
+    int64_t nvec = numel / VEC;
+    if (nvec == 0) return COAT_OK;
+    // small problems: one vector per lane to spread over the chip; large ones: 4 independent loads per lane
+    if (nvec >= (int64_t)256 * 4 * 2048) {
+        int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
+        hipLaunchKernelGGL((k_quantize_pg<XDT, SDT, KIND, QB, WQ, WS, WMAX, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, q, s, s_max, nvec, qb);
+    } else {
+        int64_t blocks = (nvec + 256 * 2 - 1) / (256 * 2);
+        hipLaunchKernelGGL((k_quantize_pg<XDT, SDT, KIND, QB, WQ, WS, WMAX, 2>), dim3((unsigned)blocks), dim3(256), 0, st, x, q, s, s_max, nvec, qb);
+    }
+    return coat_launch_status();
+}
+
+extern "C" int coat_fp8_quantize(const void* x, int x_dtype, void* q, void* s, int s_dtype, int64_t M, int64_t N, int QB,
+                                 int fp8, void* stream) {
+    if (int e = check_mn(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !q || !s) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(q)) return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, DISPATCH_QB(QB,
+        return launch_quantize_pg<XDT, SDT, KIND, QB, true, true, false>(x, q, s, nullptr, M * N, QB_RT, st)))));
+    return COAT_EINVAL;
+}
+
+extern "C" int coat_fp8_group_scales(const void* x, int x_dtype, void* s_pg, int s_dtype, float* s_max, int64_t M,
+                                     int64_t N, int QB, int fp8, void* stream) {
+    if (int e = check_mn(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !s_max) return COAT_EINVAL;
+    if (!coat_aligned16(x)) return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    if (s_pg) {
+        DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, DISPATCH_QB(QB,
+            return launch_quantize_pg<XDT, SDT, KIND, QB, false, true, true>(x, nullptr, s_pg, s_max, M * N, QB_RT, st)))));
+    } else {
+        DISPATCH_XDT(x_dtype, DISPATCH_KIND(fp8, DISPATCH_QB(QB,
+            return launch_quantize_pg<XDT, kF32, KIND, QB, false, false, true>(x, nullptr, nullptr, s_max, M * N, QB_RT, st))));
+    }
+    return COAT_EINVAL;
+}
+
+extern "C" int coat_absmax(const void* x, int x_dtype, float* amax, int64_t numel, void* stream) {
+    if (numel < 0 || !amax) return COAT_EINVAL;
+    if (numel == 0) return COAT_OK;
+    if (!x) return COAT_EINVAL;
+    if (!coat_aligned16(x)) return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_XDT(x_dtype, {
+        constexpr int VEC = VecOf<XDT>::kVec;
+        int64_t nvec = numel / VEC;
+        int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
+        if (blocks == 0) blocks = 1;
+        hipLaunchKernelGGL((k_absmax<XDT, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, amax, nvec, numel);
+        return coat_launch_status();
+    });
+    return COAT_EINVAL;
+}
+
+extern "C" int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
+                                 int64_t N, int fp8, void* stream) {
+    if (M < 0 || N < 0) return COAT_EINVAL;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !s || (!q && !qt)) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(q) || !coat_aligned16(qt)) return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    if (!qt) {
+        DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
+            constexpr int VEC = VecOf<XDT>::kVec;
+            int64_t numel = M * N, nvec = numel / VEC;
+            int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
+            if (blocks == 0) blocks = 1;
+            hipLaunchKernelGGL((k_division<XDT, SDT, KIND, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, nvec, numel);
+            return coat_launch_status();
+        })));
+        return COAT_EINVAL;
+    }
+    if (M % 16 != 0 || N % 16 != 0) return COAT_ESHAPE;
+    constexpr int TM = 64;
+    int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
+    if (q) {
+        DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
+            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, true, TM>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N);
+            return coat_launch_status();
+        })));
+    } else {
+        DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
+            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, false, TM>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N);
+            return coat_launch_status();
+        })));
+    }
+    return COAT_EINVAL;
+}
+
+extern "C" int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, void* stream) {
+    if (M < 0 || N < 0) return COAT_EINVAL;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !y) return COAT_EINVAL;
+    if (M % 16 != 0 || N % 16 != 0) return COAT_ESHAPE;
+    if (!coat_aligned16(x) || !coat_aligned16(y)) return COAT_EALIGN;
+    constexpr int TM = 64;
+    int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
+    hipLaunchKernelGGL((k_division_transpose<kBF16, kBF16, kE4M3, true, false, TM>), dim3((unsigned)blocks), dim3(256), 0,
+                       (hipStream_t)stream, x, nullptr, nullptr, y, M, N);
+    return coat_launch_status();
+}
+
+extern "C" int coat_fp8_dequantize(const void* q, int fp8, const void* s, int s_dtype, void* y, int64_t M, int64_t N,
+                                   int QB, void* stream) {
+    if (int e = check_mn(M, N, QB)) return e;
+    if (QB % 16 != 0) return COAT_ESHAPE;
+    if (M * N == 0) return COAT_OK;
+    if (!q || !s || !y) return COAT_EINVAL;
+    if (!coat_aligned16(q) || !coat_aligned16(y)) return COAT_EALIGN;
+    int64_t nchunk = M * N / 16;
+    int64_t blocks = (nchunk + 255) / 256;
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
+        hipLaunchKernelGGL((k_dequantize<SDT, KIND>), dim3((unsigned)blocks), dim3(256), 0, st, q, s, y, nchunk, QB);
+        return coat_launch_status();
+    }));
+    return COAT_EINVAL;
+}
+
+extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, void* s, void* qt, void* st_out,
+                                           int s_dtype, int64_t M, int64_t N, int QB, int fp8, void* stream) {
+    if (int e = check_mn(M, N, QB)) return e;
+    if (M % QB != 0) return COAT_ESHAPE;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !q || !s || !qt || !st_out) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(q) || !coat_aligned16(qt)) return COAT_EALIGN;
+    if (QB > 64) return COAT_ESHAPE;  // column groups must fit the 64-wide tile
+    hipStream_t st = (hipStream_t)stream;
+    constexpr int TM = 64;
+    int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
+#define LAUNCH_QT(QBV)                                                                                               \
+    DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                 \
+        hipLaunchKernelGGL((k_quantize_transpose<XDT, SDT, KIND, QBV, TM>), dim3((unsigned)blocks), dim3(256), 0, st, \
+                           x, q, s, qt, st_out, M, N);                                                               \
+        return coat_launch_status();                                                                                 \
+    })))
+    switch (QB) {
+        case 16: LAUNCH_QT(16); break;
+        case 32: LAUNCH_QT(32); break;
+        case 64: LAUNCH_QT(64); break;
+        default: return COAT_ESHAPE;
+    }
+#undef LAUNCH_QT
+    return COAT_EINVAL;
+}

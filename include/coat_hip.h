@@ -1,0 +1,97 @@
+/* C ABI of libcoat_hip.so: the MI355X (gfx950) kernels of COAT's FP8 hot path.
+ *
+ * Every entry point
+ *   - takes raw device pointers, sizes, small enums and the HIP stream to launch on
+ *     (`stream` is a hipStream_t passed as void*; NULL is the default stream);
+ *   - allocates nothing, frees nothing, keeps no global state, never synchronises the host;
+ *   - returns COAT_OK (0), a negative COAT_E* code for a rejected argument, or the positive
+ *     hipError_t of a failed launch.
+ * Tensors are row-major and contiguous.  "pg" = per-group scales, one per 1 x QB group along the
+ * last dimension; "pt" = per-tensor scale, a single element in device memory.
+ *
+ * Citations name the reference interface each entry point replaces (paths relative to the
+ * NVlabs/COAT repository; rq/ = coat/activation/real_quantization/).
+ */
+#ifndef COAT_HIP_H
+#define COAT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum coat_status {
+    COAT_OK = 0,
+    COAT_EINVAL = -1,   /* null pointer, negative size, unknown enum */
+    COAT_ESHAPE = -2,   /* divisibility / shape contract violated (N % QB, M % QB for transposes, ...) */
+    COAT_EDTYPE = -3,   /* dtype combination not supported */
+    COAT_EQGROUP = -4,  /* optimizer group size other than 128 (fp8_adamw_expand_cuda_kernel.cu:221) */
+    COAT_EALIGN = -5    /* a tensor base address is not 16-byte aligned */
+};
+
+enum coat_dtype { COAT_F32 = 0, COAT_BF16 = 1, COAT_F16 = 2 };
+enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.float8_e5m2 (rq/common.py:22-27) */
+
+const char* coat_version(void);
+const char* coat_status_string(int status);
+
+/* ---- quantize family -------------------------------------------------------------------------- */
+
+/* rq/_quantize.py:120 fp8_quantize (kernel :37-113): q = fp8(x / s32), s = (amax_g + 1e-10) / fp8max.
+ * x [M,N] x_dtype -> q [M,N] fp8, s [M,N/QB] s_dtype.  QB in {16,32,64,128}, N % QB == 0. */
+int coat_fp8_quantize(const void* x, int x_dtype, void* q, void* s, int s_dtype, int64_t M, int64_t N, int QB,
+                      int fp8, void* stream);
+
+/* rq/_quantize_transpose.py:175 fp8_quantize_transpose (kernel :39-167): the above for x and for x^T
+ * (groups of QB along M).  qt [N,M], st [N,M/QB].  Also M % QB == 0. */
+int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, void* s, void* qt, void* st, int s_dtype,
+                                int64_t M, int64_t N, int QB, int fp8, void* stream);
+
+/* rq/_quantize_pertensor.py:46-103 (+ the `s_y.max()` at :139): per-group scales and their maximum.
+ * s_pg [M,N/QB] s_dtype (may be NULL when only the maximum is wanted); s_max: one fp32 in device
+ * memory that must hold 0.0f (or a previous partial maximum) on entry and receives max(s32) by
+ * atomic max; round it to s_dtype to obtain the reference's `s_y.max()`. */
+int coat_fp8_group_scales(const void* x, int x_dtype, void* s_pg, int s_dtype, float* s_max, int64_t M, int64_t N,
+                          int QB, int fp8, void* stream);
+
+/* rq/_division.py:178-179: s = (x.abs().max() + 1e-10) / fp8max evaluated in x's dtype.
+ * amax: one fp32 in device memory holding 0.0f on entry; receives max|x| by atomic max. */
+int coat_absmax(const void* x, int x_dtype, float* amax, int64_t numel, void* stream);
+
+/* rq/_division.py:153 fp8_division (kernel :45-126, non-stochastic) and
+ * rq/_division_transpose.py:147 fp8_division_transpose (kernel :48-144): q = fp8(x / float(*s)).
+ * s: one element of s_dtype in device memory.  q [M,N] and/or qt [N,M]; either may be NULL
+ * (qt NULL = fp8_division; q NULL = only_transposed=True). */
+int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
+                      int64_t N, int fp8, void* stream);
+
+/* rq/_transpose.py:85 fp8_transpose (kernel :39-82): byte transpose, x [M,N] -> y [N,M]. */
+int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, void* stream);
+
+/* rq/_dequantize.py:119 fp8_dequantize (kernel :44-116): y = bf16(float(q) * float(s_pg)). */
+int coat_fp8_dequantize(const void* q, int fp8, const void* s, int s_dtype, void* y, int64_t M, int64_t N, int QB,
+                        void* stream);
+
+/* ---- optimizer -------------------------------------------------------------------------------- */
+
+/* qoptim_cuda.fp8_adamw_expand_step (coat/optimizer/kernels/bindings.cpp:7,
+ * include/fp8_adamw_expand.h:6-17, fp8_adamw_expand_cuda_kernel.cu:205-245).
+ * params/grads: p_dtype (F32, BF16 or F16), numel elements, updated in place.
+ * exp_avg / exp_avg_sq: e4m3 codes; scale_*, expand_*, sqrtminmax_*: fp32, ceil(numel/128) each.
+ * Unlike the reference launcher the kernel runs on `stream`, not on the legacy default stream. */
+int coat_fp8_adamw_expand_step(void* params, const void* grads, int p_dtype, void* exp_avg, float* scale_exp_avg,
+                               float* expand_exp_avg, float* sqrtminmax_exp_avg, void* exp_avg_sq,
+                               float* scale_exp_avg_sq, float* expand_exp_avg_sq, float* sqrtminmax_exp_avg_sq,
+                               float beta1, float beta2, float lr, float wd, float eps, int step, int qgroup_size,
+                               int expand_min, int64_t numel, int64_t n_scale, void* stream);
+
+/* qoptim_cuda.fp8_adamw_step (bindings.cpp:6, include/fp8_adamw.h:6-13, fp8_adamw_cuda_kernel.cu:127-159). */
+int coat_fp8_adamw_step(void* params, const void* grads, int p_dtype, void* exp_avg, float* scale_exp_avg,
+                        void* exp_avg_sq, float* scale_exp_avg_sq, float beta1, float beta2, float lr, float wd,
+                        float eps, int step, int qgroup_size, int64_t numel, int64_t n_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COAT_HIP_H */

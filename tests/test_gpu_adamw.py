@@ -1,0 +1,241 @@
+"""GPU parity: the fused FP8 AdamW kernels (through the qoptim_cuda shim / C ABI) against oracle/adamw_ref.c."""
+import pytest
+import torch
+
+from oracle import adamw_ref as A
+
+pytestmark = pytest.mark.gpu
+
+HP = dict(beta1=0.9, beta2=0.95, lr=3e-4, wd=0.1, eps=1e-8)
+KEYS_PLAIN = ("exp_avg", "scale_exp_avg", "exp_avg_sq", "scale_exp_avg_sq")
+KEYS_EXP = ("exp_avg", "scale_exp_avg", "expand_exp_avg", "sqrt_minmax_exp_avg",
+            "exp_avg_sq", "scale_exp_avg_sq", "expand_exp_avg_sq", "sqrt_minmax_exp_avg_sq")
+
+
+def _q():
+    from coat_amd.optimizer import qoptim_cuda
+    return qoptim_cuda
+
+
+def gpu_step(q, p, g, st, step, expand, hp=HP, expand_min=16):
+    if expand:
+        q.fp8_adamw_expand_step(p, g, *[st[k] for k in KEYS_EXP], hp["beta1"], hp["beta2"], hp["lr"], hp["wd"],
+                                hp["eps"], step, 128, expand_min)
+    else:
+        q.fp8_adamw_step(p, g, *[st[k] for k in KEYS_PLAIN], hp["beta1"], hp["beta2"], hp["lr"], hp["wd"], hp["eps"],
+                         step, 128)
+
+
+def cpu_step(p, g, st, step, expand, hp=HP, expand_min=16):
+    if expand:
+        A.adamw_expand_step(p, g, *[st[k] for k in KEYS_EXP], hp["beta1"], hp["beta2"], hp["lr"], hp["wd"], hp["eps"],
+                            step, 128, expand_min)
+    else:
+        A.adamw_step(p, g, *[st[k] for k in KEYS_PLAIN], hp["beta1"], hp["beta2"], hp["lr"], hp["wd"], hp["eps"], step, 128)
+
+
+def to_dev(st, dev):
+    return {k: v.to(dev) for k, v in st.items()}
+
+
+def grads(n, seed, scale=1e-3):
+    return torch.randn(n, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+@pytest.mark.parametrize("n", [128 * 64, 128 * 9 + 37, 127, 1, 1024 * 3 + 5])
+@pytest.mark.parametrize("pdtype", [torch.float32, torch.bfloat16])
+def test_plain_step_bit_exact(dev, n, pdtype):
+    """No transcendental functions on this path: params, codes and scales must match bit for bit over 3 steps."""
+    q = _q()
+    p = (torch.randn(n, generator=torch.Generator().manual_seed(0)) * 0.02).to(pdtype)
+    st = A.fresh_state(p, expand=False)
+    pd, std = p.to(dev), to_dev(st, dev)
+    for step in (1, 2, 3):
+        g = grads(n, step).to(pdtype)
+        cpu_step(p, g, st, step, False)
+        gpu_step(q, pd, g.to(dev), std, step, False)
+        assert torch.equal(pd.cpu(), p), f"params differ at step {step}"
+        for k in KEYS_PLAIN:
+            assert torch.equal(std[k].cpu().view(torch.uint8) if std[k].dtype != torch.float32 else std[k].cpu(),
+                               st[k].view(torch.uint8) if st[k].dtype != torch.float32 else st[k]), (k, step)
+
+
+def compare_expand(pd, std, p, st, n, tag=""):
+    """Stated tolerances for the expand step (hardware log2/exp2, ~1e-6 relative, against correctly rounded powf).
+
+    params: fp32 rtol 2e-6 (atol 1e-9); bf16 within one bf16 ulp.
+    The group minimum Mn is often the result of a cancellation beta1*m + (1-beta1)*g ~ 0, so its absolute error
+    is ~1e-6 of the group maximum Mx, not of Mn: the centre c = sqrt(Mx*Mn) is therefore bounded through
+    |c^2 - c_ref^2| / c_ref^2 <= 4e-5 * Mx/Mn.  Groups whose c agrees to 1e-5 ("well conditioned", at least 80 %
+    of them) must in addition have: the same exponent k (all but 1e-3 of them), the new scale within rtol 1e-4,
+    codes different on < 1e-3 of their elements and by one code step at most."""
+    if p.dtype == torch.float32:
+        assert torch.allclose(pd.cpu(), p, rtol=2e-6, atol=1e-9), tag + " params"
+    else:
+        assert torch.allclose(pd.cpu().float(), p.float(), rtol=2.0 ** -7, atol=1e-30), tag + " params (bf16 ulp)"
+    for name in ("exp_avg", "exp_avg_sq"):
+        c_g, c_c = std["sqrt_minmax_" + name].cpu().double(), st["sqrt_minmax_" + name].double()
+        k_g, k_c = std["expand_" + name].cpu(), st["expand_" + name]
+        s_g, s_c = std["scale_" + name].cpu().double(), st["scale_" + name].double()
+        finite_k = (k_c > 0) & torch.isfinite(k_c)
+        ratio = torch.where(finite_k, (448 * s_c).pow(2 / k_c.double().clamp_min(1e-3)), torch.ones_like(s_c))
+        rel_c2 = (c_g * c_g - c_c * c_c).abs() / (c_c * c_c)
+        assert (rel_c2 <= 4e-5 * ratio + 1e-6).all(), (tag, name, "centre", (rel_c2 / ratio).max().item())
+        well = ((c_g - c_c).abs() <= 1e-5 * c_c) & finite_k
+        ng = k_c.numel()
+        if ng >= 64:
+            assert well.float().mean().item() >= 0.8, (tag, name, well.float().mean().item())
+        same = (k_g == k_c) & well
+        assert (well & ~same).sum().item() <= max(1, int(1e-3 * ng)), (tag, name, "k", (well & ~same).sum().item())
+        assert torch.allclose(s_g[same], s_c[same], rtol=1e-4, atol=0), tag + " scale"
+        pad = ng * 128 - n
+        cg = torch.nn.functional.pad(std[name].cpu().view(torch.uint8).flatten(), (0, pad)).reshape(ng, 128)[same]
+        cc = torch.nn.functional.pad(st[name].view(torch.uint8).flatten(), (0, pad)).reshape(ng, 128)[same]
+        neq = cg != cc
+        assert neq.sum().item() <= max(16, int(1e-3 * neq.numel())), (tag, name, "codes", neq.sum().item(), neq.numel())
+        if neq.any():  # one code step: neighbouring magnitudes with the same sign (or +0 / -0 against the smallest code)
+            a, b = cg[neq].int(), cc[neq].int()
+            assert ((a & 0x7F) - (b & 0x7F)).abs().max().item() <= 1, (tag, name, "code step")
+            assert (((a & 0x80) == (b & 0x80)) | (((a & 0x7F) + (b & 0x7F)) <= 1)).all(), (tag, name, "code sign")
+
+
+@pytest.mark.parametrize("n", [128 * 512, 128 * 9 + 37, 127, 1])
+@pytest.mark.parametrize("pdtype", [torch.float32, torch.bfloat16])
+def test_expand_step_from_identical_state(dev, n, pdtype):
+    q = _q()
+    p = (torch.randn(n, generator=torch.Generator().manual_seed(0)) * 0.02).to(pdtype)
+    st = A.fresh_state(p, expand=True)
+    pd, std = p.to(dev), to_dev(st, dev)
+    # A single-element tensor is degenerate for Dynamic Range Expansion (max == min, k = inf): from its second
+    # step on the reference algorithm itself stores scale = inf and NaN codes, and what follows depends on the
+    # sign bit of a NaN.  Only the steps before that are compared for n == 1.
+    for step in ((1, 2) if n == 1 else (1, 2, 3, 4)):
+        g = grads(n, step).to(pdtype)
+        # each step starts from the oracle's state so that differences do not compound
+        pd, std = p.to(dev), to_dev(st, dev)
+        cpu_step(p, g, st, step, True)
+        gpu_step(q, pd, g.to(dev), std, step, True)
+        compare_expand(pd, std, p, st, n, f"step {step}")
+    if n >= 128:
+        # step 1 from the fresh state has no dequantization error: centre and exponent must be exact
+        p1 = (torch.randn(n, generator=torch.Generator().manual_seed(0)) * 0.02).to(pdtype)
+        s1 = A.fresh_state(p1, True)
+        pd1, sd1 = p1.to(dev), to_dev(s1, dev)
+        g = grads(n, 1).to(pdtype)
+        cpu_step(p1, g, s1, 1, True)
+        gpu_step(q, pd1, g.to(dev), sd1, 1, True)
+        assert torch.equal(sd1["sqrt_minmax_exp_avg"].cpu(), s1["sqrt_minmax_exp_avg"])
+        assert torch.equal(sd1["sqrt_minmax_exp_avg_sq"].cpu(), s1["sqrt_minmax_exp_avg_sq"])
+        assert torch.equal(pd1.cpu(), p1)
+
+
+def test_expand_reference_test_case(dev):
+    """The reference test's configuration: M 2, N 128, step 1000, lr 0.4 (tests/test_fp8_adamw_expand.py:43-51)."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from test_oracle_adamw import _random_expand_state
+    q = _q()
+    hp = dict(beta1=0.9, beta2=0.95, lr=0.4, wd=0.1, eps=1e-8)
+    n = 256
+    gen = torch.Generator().manual_seed(0)
+    p = torch.randn(n, generator=gen)
+    g = torch.randn(n, generator=gen)
+    st = _random_expand_state(n, 1)
+    pd, std = p.to(dev), to_dev(st, dev)
+    cpu_step(p, g, st, 1000, True, hp)
+    gpu_step(q, pd, g.to(dev), std, 1000, True, hp)
+    assert torch.allclose(pd.cpu(), p, rtol=1e-4)  # the reference's own bar
+    compare_expand(pd, std, p, st, n, "ref case")
+
+
+def test_expand_zero_handling_matches_reference_tree(dev):
+    """Exact zeros take the shuffle-tree path: thread-0 zero survives, partner zeros are skipped,
+    all-zero groups stay finite."""
+    q = _q()
+    hp = dict(beta1=0.0, beta2=0.0, lr=0.0, wd=0.0, eps=1e-8)
+    base = torch.linspace(1.0, 2.0, 128)
+    cases = []
+    for pos in (None, 0, 16, 32, 1, 4, 127, 64, 96):
+        g = base.clone()
+        if pos is not None:
+            g[pos] = 0.0
+        cases.append(g)
+    cases.append(torch.zeros(128))
+    g = torch.cat(cases)
+    n = g.numel()
+    p = torch.zeros(n)
+    st = A.fresh_state(p, True)
+    pd, std = p.to(dev), to_dev(st, dev)
+    cpu_step(p, g.clone(), st, 1, True, hp)
+    gpu_step(q, pd, g.to(dev), std, 1, True, hp)
+    for k in ("sqrt_minmax_exp_avg", "sqrt_minmax_exp_avg_sq"):
+        assert torch.equal(std[k].cpu(), st[k]), k  # sqrt(Mx)*sqrt(Mn): exact given the same min / max
+    compare_expand(pd, std, p, st, n, "zeros")
+    # a second step from that state (k = inf / 0 groups exercise the powf special cases)
+    g2 = torch.cat([base * 0.5] * (len(cases) - 1) + [torch.zeros(128)])
+    pd, std = p.to(dev), to_dev(st, dev)
+    cpu_step(p, g2.clone(), st, 2, True, hp)
+    gpu_step(q, pd, g2.to(dev), std, 2, True, hp)
+    assert torch.isfinite(pd).all()
+    compare_expand(pd, std, p, st, n, "zeros step 2")
+
+
+def test_errors(dev):
+    q = _q()
+    p = torch.zeros(256, device=dev)
+    st = to_dev(A.fresh_state(p.cpu(), True), dev)
+    with pytest.raises(RuntimeError, match="Only Support 128"):
+        q.fp8_adamw_expand_step(p, p, *[st[k] for k in KEYS_EXP], 0.9, 0.95, 1e-3, 0.1, 1e-8, 1, 64, 16)
+    bad = dict(st)
+    bad["scale_exp_avg"] = torch.zeros(3, device=dev)
+    with pytest.raises(RuntimeError):
+        q.fp8_adamw_expand_step(p, p, *[bad[k] for k in KEYS_EXP], 0.9, 0.95, 1e-3, 0.1, 1e-8, 1, 128, 16)
+
+
+def test_coatadamw_trajectory_and_state_dict(dev):
+    """CoatAdamW (drop-in optimizer class) over 10 steps on a [256, 384] weight against the oracle run on
+    the CPU with the same gradients, then a state_dict round trip."""
+    from coat_amd.optimizer.fp8_adamw import CoatAdamW
+    from coat_amd.utils._fp8_quantization_config import QuantizationConfig
+    torch.manual_seed(0)
+    w0 = torch.randn(256, 384) * 0.02
+    for expansion in ("true", "false"):
+        w = torch.nn.Parameter(w0.clone().to(dev))
+        opt = CoatAdamW([w], lr=3e-4, betas=(0.9, 0.95), weight_decay=0.1, eps=1e-8,
+                        qargs=QuantizationConfig(first_order_expansion=expansion, second_order_expansion=expansion))
+        p = w0.clone().flatten()
+        st = A.fresh_state(p, expansion == "true")
+        for step in range(1, 11):
+            g = grads(p.numel(), 100 + step)
+            w.grad = g.reshape(256, 384).to(dev)
+            opt.step()
+            cpu_step(p, g, st, step, expansion == "true")
+        dp = (w.detach().cpu().flatten() - p).abs()
+        if expansion == "false":
+            assert dp.max().item() == 0.0  # the plain step is bit-exact, so is its trajectory
+        else:
+            # a moment that lands one e4m3 code away (about 1e-5 of them per step) moves that element's update by
+            # at most one fp8 step of m/denom ~ 1: lr * 2^-3 per step in the worst case; everything else is ulps
+            assert dp.max().item() <= 3e-4 * 0.125 * 10 and dp.median().item() <= 1e-8 and (dp > 1e-7).float().mean().item() < 5e-3
+        s = opt.state[w]
+        assert s["exp_avg"].dtype == torch.float8_e4m3fn and s["scale_exp_avg"].dtype == torch.float32
+        assert int(s["step"].item()) == 10 and s["step"].device.type == "cpu"
+        if expansion == "false":
+            assert "expand_exp_avg" not in s
+            assert torch.equal(s["exp_avg"].cpu().view(torch.uint8), st["exp_avg"].view(torch.uint8).reshape(256, 384))
+        else:
+            m_g = A.dequantize_state(s["exp_avg"].cpu().flatten(), s["scale_exp_avg"].cpu(), s["expand_exp_avg"].cpu(), s["sqrt_minmax_exp_avg"].cpu())
+            m_c = A.dequantize_state(st["exp_avg"], st["scale_exp_avg"], st["expand_exp_avg"], st["sqrt_minmax_exp_avg"])
+            rel = (m_g - m_c).abs() / m_c.abs().clamp_min(1e-12)
+            assert rel.median() < 1e-3 and rel.quantile(0.99) < 0.2  # trajectories stay together to within fp8 steps
+        import copy
+        sd = copy.deepcopy(opt.state_dict())  # state_dict() hands out the live tensors
+        w2 = torch.nn.Parameter(w.detach().clone())
+        opt2 = CoatAdamW([w2], lr=3e-4, betas=(0.9, 0.95), weight_decay=0.1, eps=1e-8, qargs=opt.qargs)
+        opt2.load_state_dict(sd)
+        s2 = opt2.state[w2]
+        assert s2["exp_avg"].dtype == torch.float8_e4m3fn and s2["scale_exp_avg"].dtype == torch.float32
+        g = grads(p.numel(), 999).reshape(256, 384).to(dev)
+        w.grad, w2.grad = g, g.clone()
+        opt.step(); opt2.step()
+        assert torch.equal(w.detach(), w2.detach())
