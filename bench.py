@@ -1,0 +1,184 @@
+"""Benchmark of the FP8 hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload adamw|quantize|quantize_transpose]
+
+Default workload = BASELINE.json configs[1]: one CoatAdamW step (Dynamic Range Expansion on) on an fp32 master
+weight [11008, 4096], grads N(0, 1e-3), lr 3e-4, betas (0.9, 0.95), wd 0.1, eps 1e-8, starting at step 10 from a
+moment state produced by nine untimed steps.  A "step" is one pass of the fused kernel over the whole tensor.
+Prints ONE JSON line.  `value` is algorithmic GB/s: every distinct input read once + every output written once
+(in-place tensors count read + write) divided by the wall-clock per step with inputs resident in HBM.
+`roofline.achieved` uses the kernel's average launch duration measured with HIP events on the launch stream.
+`cpu_baseline` times the plain-C oracle (one thread) on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def adamw_bytes(numel):
+    ngroups = (numel + 127) // 128
+    # p r+w (4+4), g r (4), m8 r+w (1+1), v8 r+w (1+1) per element; 6 fp32 group vectors r+w per group
+    return numel * 16 + ngroups * 48
+
+
+def make_adamw_workload(dev, shape, torch):
+    from coat_amd.optimizer import qoptim_cuda
+
+    numel = shape[0] * shape[1]
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    p = (torch.randn(shape, generator=gen) * 0.02).to(dev)
+    ng = (numel + 127) // 128
+    st = [torch.zeros(shape, dtype=torch.float8_e4m3fn, device=dev), torch.zeros(ng, device=dev),
+          torch.ones(ng, device=dev), torch.ones(ng, device=dev),
+          torch.zeros(shape, dtype=torch.float8_e4m3fn, device=dev), torch.zeros(ng, device=dev),
+          torch.ones(ng, device=dev), torch.ones(ng, device=dev)]
+    hp = (0.9, 0.95, 3e-4, 0.1, 1e-8)
+    grads = []
+    for seed in range(1, 5):  # a few distinct gradient tensors, cycled
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        grads.append((torch.randn(shape, generator=g) * 1e-3).to(dev))
+
+    state = {"step": 0}
+
+    def step():
+        state["step"] += 1
+        qoptim_cuda.fp8_adamw_expand_step(p, grads[state["step"] % len(grads)], *st, *hp, state["step"], 128, 16)
+
+    for _ in range(9):  # steps 1..9: builds a realistic moment state (k, c per group), untimed
+        step()
+    return step, adamw_bytes(numel), {"workload": "CoatAdamW.step fp32 [11008,4096], DRE on, step 10+, qgroup 128",
+                                      "numel": numel, "kernel": "k_fp8_adamw<f32,expand>"}
+
+
+def make_quantize_workload(dev, torch, transpose):
+    from coat_amd.activation.real_quantization import fp8_quantize
+    from coat_amd.activation.real_quantization._quantize_transpose import fp8_quantize_transpose
+
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn(4096, 4096, generator=gen)
+    x[torch.rand(4096, 4096, generator=gen) < 0.001] *= 100
+    # rotate over buffer sets so that > 512 MB is touched between reuses (the 256 MB Infinity Cache stays cold)
+    nset = 12
+    xs = [x.bfloat16().to(dev).clone() for _ in range(nset)]
+    state = {"i": 0}
+    fn = fp8_quantize_transpose if transpose else fp8_quantize
+
+    def step():
+        state["i"] += 1
+        fn(xs[state["i"] % nset], 16, "E4M3")
+
+    nbytes = 4096 * 4096 * 2 + (2 if transpose else 1) * (4096 * 4096 + 4096 * 256 * 2)
+    name = "fp8_quantize_transpose" if transpose else "fp8_quantize"
+    return step, nbytes, {"workload": f"{name} bf16 [4096,4096] QB16 e4m3, {nset} rotating inputs", "numel": 4096 * 4096,
+                          "kernel": "k_quantize_transpose" if transpose else "k_quantize_pg"}
+
+
+def cpu_baseline_adamw(torch):
+    """The plain-C oracle (one thread) on a bounded sample: same hyper-parameters, step 10 state built by the
+    oracle itself, sample sized for roughly 10-20 s."""
+    from oracle import adamw_ref as A
+
+    hp = (0.9, 0.95, 3e-4, 0.1, 1e-8)
+    n = 128 * 4096  # 0.5 M elements of the [11008, 4096] tensor
+    gen = torch.Generator().manual_seed(0)
+    p = torch.randn(n, generator=gen) * 0.02
+    st = A.fresh_state(p, True)
+    keys = ("exp_avg", "scale_exp_avg", "expand_exp_avg", "sqrt_minmax_exp_avg", "exp_avg_sq", "scale_exp_avg_sq",
+            "expand_exp_avg_sq", "sqrt_minmax_exp_avg_sq")
+    grads = [torch.randn(n, generator=gen) * 1e-3 for _ in range(4)]
+    step = 0
+    for _ in range(3):
+        step += 1
+        A.adamw_expand_step(p, grads[step % 4], *[st[k] for k in keys], *hp, step, 128, 16)
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 10.0:
+        step += 1
+        A.adamw_expand_step(p, grads[step % 4], *[st[k] for k in keys], *hp, step, 128, 16)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(adamw_bytes(n) / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} steps over the first {n} elements (4096 groups) of the tensor, oracle/adamw_ref.c, 1 thread"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times (known traffic, to scale rocprofv3 counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported "
+              "(every kernel on the path is independent per row / per 128-element group, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from coat_amd import _hip
+
+    _hip.lib()  # fail loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    if args.workload == "adamw":
+        step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch)
+    else:
+        step, nbytes, cfg = make_quantize_workload(dev, torch, args.workload == "quantize_transpose")
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # HIP events around every launch, on the stream the kernels are launched on (torch's current stream)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = sorted(a.elapsed_time(b) for a, b in evs)
+    avg_ms = sum(kern_ms) / len(kern_ms)
+    ms_per_step = wall * 1e3 / args.steps
+    value = nbytes / (ms_per_step * 1e-3) / 1e9
+    achieved = nbytes / (avg_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic", "config": cfg,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": nbytes, "kernel_ms_avg": round(avg_ms, 5),
+                     "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5)},
+    }
+    if args.workload == "adamw" and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_adamw(torch)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

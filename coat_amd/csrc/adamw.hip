@@ -10,10 +10,10 @@
 // maxima / minima are 15 in-lane operations plus a 3-step DPP reduction over 8 lanes, and the group
 // constants (centre c, exponent k, new scale) are computed once per lane for 16 elements.
 //
-// Numerics: + - * / sqrt are the IEEE fp32 operations of the reference source in the same order without
-// FMA contraction, so the plain (non-expand) step is bit-exact against the CPU restatement.  The x^y of
-// the expand step is exp2(y * log2(x)) on the hardware v_log_f32 / v_exp_f32 (about 1e-6 relative),
-// with the IEEE special cases of powf (y = 0, y = inf, x = 0, x = 1) reproduced explicitly.
+// Numerics: in the plain (non-expand) step + - * / sqrt are the IEEE fp32 operations of the reference source
+// in the same order without FMA contraction, so it is bit-exact against the CPU restatement.  The x^y of the
+// expand step is exp2(y * log2(x)) on the hardware v_log_f32 / v_exp_f32 (about 1e-6 relative), with the IEEE
+// special cases of powf (y = 0, y = inf, x = 0, x = 1) reproduced explicitly; see k_fp8_adamw_expand.
 // The reference's order-dependent zero-skipping minimum is reproduced exactly: when a group holds an
 // exact zero the kernel walks the reference's 32-lane shuffle tree, otherwise that tree equals a plain min.
 #include <math.h>
@@ -126,24 +126,23 @@ __device__ __forceinline__ void store_codes4(uint8_t* base, int64_t e, int64_t n
     }
 }
 
-template <int PDT, bool EXPAND>
-__global__ __launch_bounds__(256) void k_fp8_adamw(void* __restrict__ params, const void* __restrict__ grads,
-                                                    uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
-                                                    float* __restrict__ expand_m, float* __restrict__ sqrtmm_m,
-                                                    uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
-                                                    float* __restrict__ expand_v, float* __restrict__ sqrtmm_v,
-                                                    AdamArgs A, int64_t numel, int64_t ngroups) {
+// ------------------------------------------------------------------------------------------------
+// Plain (no expansion) step: every operation is the IEEE operation of the reference, bit-exact.
+template <int PDT>
+__global__ __launch_bounds__(256) void k_fp8_adamw_plain(void* __restrict__ params, const void* __restrict__ grads,
+                                                          uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
+                                                          uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
+                                                          AdamArgs A, int64_t numel, int64_t ngroups) {
     enable_fp8_saturation();
     const int lane = threadIdx.x & 63, lam = lane & 7;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t wave = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t gi = wave * 8 + (lane >> 3);
     if (wave * 8 >= ngroups) return;  // whole wave out of range (wave-uniform)
     const bool gvalid = gi < ngroups;
-    const int64_t gidx = gvalid ? gi : ngroups - 1;  // clamp: lanes of absent groups redo the last group, stores masked
+    const int64_t gidx = gvalid ? gi : ngroups - 1;  // lanes of absent groups redo the last group, stores masked
     const int64_t e0 = gidx * kGroup + lam * 4;
-    const int64_t lim = gvalid ? numel : 0;  // element validity bound for this lane
+    const int64_t lim = gvalid ? numel : 0;
 
-    // ---- loads
     float p[4][4], g[4][4];
     uint32_t cm[4], cv[4];
 #pragma unroll
@@ -154,22 +153,8 @@ __global__ __launch_bounds__(256) void k_fp8_adamw(void* __restrict__ params, co
         cv[j] = load_codes4(exp_avg_sq, e0 + 32 * j, numel);
     }
     const float sm = scale_m[gidx], sv = scale_v[gidx];
-    float invk_m = 1.0f, invk_v = 1.0f, c_m = 1.0f, c_v = 1.0f;
-    bool odd_pow = false;
-    if (EXPAND) {
-        invk_m = 1 / expand_m[gidx];
-        invk_v = 1 / expand_v[gidx];
-        c_m = sqrtmm_m[gidx];
-        c_v = sqrtmm_v[gidx];
-        // exponents outside (0, inf) need the special cases of powf; decide once per wave
-        bool odd = !(invk_m > 0.0f && invk_m < INFINITY) || !(invk_v > 0.0f && invk_v < INFINITY);
-        odd_pow = __builtin_amdgcn_ballot_w64(odd) != 0;
-    }
-
-    // ---- dequantize, Adam update
     float m[4][4], v[4][4];
-    float mx_m = 0.0f, mx_v = 0.0f, mn_m = kFltMax, mn_v = kFltMax;
-    bool has_zero = false;
+    float mx_m = 0.0f, mx_v = 0.0f;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         float fm[4], fv[4];
@@ -179,12 +164,6 @@ __global__ __launch_bounds__(256) void k_fp8_adamw(void* __restrict__ params, co
         for (int i = 0; i < 4; i++) {
             const bool ok = e0 + 32 * j + i < lim;
             float em = fm[i] * sm, ev = fv[i] * sv;
-            if (EXPAND) {
-                float pm = odd_pow ? pow_full(fabsf(em), invk_m) : pow_fast(fabsf(em), invk_m);
-                float pv = odd_pow ? pow_full(ev, invk_v) : pow_fast(ev, invk_v);
-                em = copysignf(pm * c_m, em);
-                ev = pv * c_v;
-            }
             const float gr = g[j][i], pr = p[j][i];
             em = A.beta1 * em + A.one_minus_beta1 * gr;
             ev = A.beta2 * ev + (A.one_minus_beta2 * gr) * gr;
@@ -193,62 +172,157 @@ __global__ __launch_bounds__(256) void k_fp8_adamw(void* __restrict__ params, co
             p[j][i] = pr - (A.lr * update);
             m[j][i] = em;
             v[j][i] = ev;
-            float am = ok ? fabsf(em) : 0.0f, av = ok ? fabsf(ev) : 0.0f;
-            mx_m = fmaxf(mx_m, am);
-            mx_v = fmaxf(mx_v, av);
-            if (EXPAND) {
-                mn_m = fminf(mn_m, ok ? am : kFltMax);
-                mn_v = fminf(mn_v, ok ? av : kFltMax);
-                has_zero |= ok && !(am > 0.0f && av > 0.0f);
-            }
+            mx_m = fmaxf(mx_m, ok ? fabsf(em) : 0.0f);
+            mx_v = fmaxf(mx_v, ok ? fabsf(ev) : 0.0f);
         }
     }
 #pragma unroll
     for (int j = 0; j < 4; j++) store4<PDT>(params, e0 + 32 * j, lim, p[j]);
+    mx_m = cluster_max<8>(mx_m);
+    mx_v = cluster_max<8>(mx_v);
+    // "+ 1e-20" is a double-precision add narrowed to float in the reference
+    const float snew_m = (float)((double)mx_m + 1e-20) / 448.0f;
+    const float snew_v = (float)((double)mx_v + 1e-20) / 448.0f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        store_codes4(exp_avg, e0 + 32 * j, lim,
+                     cvt4_fp8<kE4M3>(m[j][0] / snew_m, m[j][1] / snew_m, m[j][2] / snew_m, m[j][3] / snew_m));
+        store_codes4(exp_avg_sq, e0 + 32 * j, lim,
+                     cvt4_fp8<kE4M3>(v[j][0] / snew_v, v[j][1] / snew_v, v[j][2] / snew_v, v[j][3] / snew_v));
+    }
+    if (gvalid && lam == 0) {
+        scale_m[gi] = snew_m;
+        scale_v[gi] = snew_v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Expand step.  x^y is exp2(y * log2 x) on the hardware units; the arguments of log2 are kept close to 1
+// (code*s and |m|/c', both within [1/317, 317]) so that the absolute error of y*log2(x) stays ~1e-6 whatever
+// the exponent, and the division by the new scale is folded into the exponent:
+//   dequantize   m = sign * exp2(log2|code * s| * (1/k)) * c
+//   requantize   m'/s' = sign * exp2(log2(|m| * (1/c')) * k' - log2(s'))
+// sqrt and the reciprocal of the Adam denominator are the hardware approximations (1 ulp), FMAs are used
+// freely; none of this is visible next to the 1e-6 of the hardware log2 / exp2.  Groups whose exponent is 0 or inf (all values
+// equal, or an infinite max/min ratio) take the step-by-step path with the IEEE special cases of powf.
+struct GroupIn {  // per-group constants of the incoming state
+    float sm, sv, invk_m, invk_v, c_m, c_v;
+};
+
+template <int PDT, bool FULL>
+__device__ __forceinline__ void adamw_expand_wave(void* __restrict__ params, const void* __restrict__ grads,
+                                                  uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
+                                                  float* __restrict__ expand_m, float* __restrict__ sqrtmm_m,
+                                                  uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
+                                                  float* __restrict__ expand_v, float* __restrict__ sqrtmm_v,
+                                                  const AdamArgs& A, int64_t numel, int64_t ngroups, int64_t wave,
+                                                  int lane) {
+    const int lam = lane & 7;
+    const int64_t gi = wave * 8 + (lane >> 3);
+    const bool gvalid = FULL || gi < ngroups;
+    const int64_t gidx = gvalid ? gi : ngroups - 1;
+    const int64_t e0 = gidx * kGroup + lam * 4;
+    const int64_t lim = gvalid ? numel : 0;
+
+    float p[4][4], g[4][4];
+    uint32_t cm[4], cv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        load4<PDT>(params, e0 + 32 * j, FULL ? (int64_t)1 << 62 : numel, p[j]);
+        load4<PDT>(grads, e0 + 32 * j, FULL ? (int64_t)1 << 62 : numel, g[j]);
+        cm[j] = load_codes4(exp_avg, e0 + 32 * j, FULL ? (int64_t)1 << 62 : numel);
+        cv[j] = load_codes4(exp_avg_sq, e0 + 32 * j, FULL ? (int64_t)1 << 62 : numel);
+    }
+    GroupIn G;
+    G.sm = scale_m[gidx];
+    G.sv = scale_v[gidx];
+    G.invk_m = 1 / expand_m[gidx];
+    G.invk_v = 1 / expand_v[gidx];
+    G.c_m = sqrtmm_m[gidx];
+    G.c_v = sqrtmm_v[gidx];
+    // exponents outside (0, inf) need the special cases of powf; decided once per wave
+    const bool odd_in = __builtin_amdgcn_ballot_w64(!(G.invk_m > 0.0f && G.invk_m < INFINITY) ||
+                                                    !(G.invk_v > 0.0f && G.invk_v < INFINITY)) != 0;
+    const float inv_c2 = 1.0f / A.correction2_sqrt;
+
+    float m[4][4], v[4][4];
+    float mx_m = 0.0f, mx_v = 0.0f, mn_m = kFltMax, mn_v = kFltMax;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float fm[4], fv[4];
+        fp8x4_to_f32<kE4M3>(cm[j], fm);
+        fp8x4_to_f32<kE4M3>(cv[j], fv);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const bool ok = FULL || (e0 + 32 * j + i < lim);
+            float em, ev;
+            if (!odd_in) {
+                em = copysignf(exp2_hw(log2_hw(fabsf(fm[i] * G.sm)) * G.invk_m) * G.c_m, fm[i]);
+                ev = exp2_hw(log2_hw(fv[i] * G.sv) * G.invk_v) * G.c_v;
+            } else {
+                em = fm[i] * G.sm;
+                ev = fv[i] * G.sv;
+                em = copysignf(pow_full(fabsf(em), G.invk_m) * G.c_m, em);
+                ev = pow_full(ev, G.invk_v) * G.c_v;
+            }
+            const float gr = g[j][i], pr = p[j][i];
+            em = fmaf(A.beta1, em, A.one_minus_beta1 * gr);
+            ev = fmaf(A.beta2, ev, (A.one_minus_beta2 * gr) * gr);
+            const float denom = fmaf(__builtin_amdgcn_sqrtf(ev), inv_c2, A.eps) * A.correction1;
+            const float update = fmaf(em, __builtin_amdgcn_rcpf(denom), A.wd * pr);
+            p[j][i] = fmaf(-A.lr, update, pr);
+            m[j][i] = em;
+            v[j][i] = ev;
+            const float am = fabsf(em), av = fabsf(ev);
+            mx_m = fmaxf(mx_m, ok ? am : 0.0f);
+            mx_v = fmaxf(mx_v, ok ? av : 0.0f);
+            mn_m = fminf(mn_m, ok ? am : kFltMax);
+            mn_v = fminf(mn_v, ok ? av : kFltMax);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) store4<PDT>(params, e0 + 32 * j, FULL ? (int64_t)1 << 62 : lim, p[j]);
 
     // ---- group statistics (8 lanes per group)
     mx_m = cluster_max<8>(mx_m);
     mx_v = cluster_max<8>(mx_v);
-    float snew_m, snew_v, k_m = 1.0f, k_v = 1.0f, cn_m = 1.0f, cn_v = 1.0f;
-    bool odd_k = false;
-    if (EXPAND) {
-        if (__builtin_amdgcn_ballot_w64(has_zero) != 0) {
-            // some moment is exactly zero (or NaN): walk the reference's shuffle tree
-            float a[4][4], b[4][4];
+    mn_m = -cluster_max<8>(-mn_m);
+    mn_v = -cluster_max<8>(-mn_v);
+    // an exact zero (or a NaN, which fmin drops) anywhere in the wave: walk the reference's shuffle tree
+    bool suspicious = !(mn_m > 0.0f) || !(mn_v > 0.0f) || !(mx_m == mx_m) || !(mx_v == mx_v);
+    if (__builtin_amdgcn_ballot_w64(suspicious) != 0) {
+        float a[4][4], b[4][4];
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+        for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const bool ok = e0 + 32 * j + i < lim;
-                    a[j][i] = ok ? fabsf(m[j][i]) : kFltMax;
-                    b[j][i] = ok ? fabsf(v[j][i]) : kFltMax;
-                }
-            mn_m = reference_tree_min(a);
-            mn_v = reference_tree_min(b);
-            // broadcast from the lam == 0 lane of each group
-            mn_m = u2f((uint32_t)__builtin_amdgcn_ds_bpermute((lane & ~7) << 2, (int)f2u(mn_m)));
-            mn_v = u2f((uint32_t)__builtin_amdgcn_ds_bpermute((lane & ~7) << 2, (int)f2u(mn_v)));
-        } else {
-            // all values positive: the tree is a plain minimum, capped by the 1e9 filler of the block level
-            mn_m = fminf(-cluster_max<8>(-mn_m), 1e9f);
-            mn_v = fminf(-cluster_max<8>(-mn_v), 1e9f);
-        }
-        // "+ 1e-30" is a double-precision add narrowed to float in the reference
-        const float Mx_m = (float)((double)mx_m + 1e-30), Mn_m = (float)((double)mn_m + 1e-30);
-        const float Mx_v = (float)((double)mx_v + 1e-30), Mn_v = (float)((double)mn_v + 1e-30);
-        const float ratio_m = Mx_m / Mn_m, ratio_v = Mx_v / Mn_v;
-        cn_m = sqrtf(Mx_m) * sqrtf(Mn_m);
-        cn_v = sqrtf(Mx_v) * sqrtf(Mn_v);
-        k_m = floorf((kLog2RatioUpperBound / log2_hw(ratio_m)) * A.expand_min) / A.expand_min;
-        k_v = floorf((kLog2RatioUpperBound / log2_hw(ratio_v)) * A.expand_min) / A.expand_min;
-        snew_m = pow_full(Mx_m / cn_m, k_m) / 448.0f;
-        snew_v = pow_full(Mx_v / cn_v, k_v) / 448.0f;
-        bool odd = !(k_m > 0.0f && k_m < INFINITY) || !(k_v > 0.0f && k_v < INFINITY);
-        odd_k = __builtin_amdgcn_ballot_w64(odd) != 0;
+            for (int i = 0; i < 4; i++) {
+                const bool ok = FULL || (e0 + 32 * j + i < lim);
+                a[j][i] = ok ? fabsf(m[j][i]) : kFltMax;
+                b[j][i] = ok ? fabsf(v[j][i]) : kFltMax;
+            }
+        mn_m = reference_tree_min(a);
+        mn_v = reference_tree_min(b);
+        mn_m = u2f((uint32_t)__builtin_amdgcn_ds_bpermute((lane & ~7) << 2, (int)f2u(mn_m)));
+        mn_v = u2f((uint32_t)__builtin_amdgcn_ds_bpermute((lane & ~7) << 2, (int)f2u(mn_v)));
     } else {
-        snew_m = (float)((double)mx_m + 1e-20) / 448.0f;
-        snew_v = (float)((double)mx_v + 1e-20) / 448.0f;
+        // all values positive: the tree is a plain minimum, capped by the 1e9 filler of its block level
+        mn_m = fminf(mn_m, 1e9f);
+        mn_v = fminf(mn_v, 1e9f);
     }
+    // "+ 1e-30" is a double-precision add narrowed to float in the reference
+    const float Mx_m = (float)((double)mx_m + 1e-30), Mn_m = (float)((double)mn_m + 1e-30);
+    const float Mx_v = (float)((double)mx_v + 1e-30), Mn_v = (float)((double)mn_v + 1e-30);
+    const float ratio_m = Mx_m / Mn_m, ratio_v = Mx_v / Mn_v;
+    const float cn_m = sqrtf(Mx_m) * sqrtf(Mn_m), cn_v = sqrtf(Mx_v) * sqrtf(Mn_v);
+    const float k_m = floorf((kLog2RatioUpperBound / log2_hw(ratio_m)) * A.expand_min) / A.expand_min;
+    const float k_v = floorf((kLog2RatioUpperBound / log2_hw(ratio_v)) * A.expand_min) / A.expand_min;
+    const float snew_m = pow_full(Mx_m / cn_m, k_m) / 448.0f;
+    const float snew_v = pow_full(Mx_v / cn_v, k_v) / 448.0f;
+    const bool odd_out = __builtin_amdgcn_ballot_w64(!(k_m > 0.0f && k_m < INFINITY) || !(k_v > 0.0f && k_v < INFINITY) ||
+                                                     !(snew_m > 0.0f && snew_m < INFINITY) ||
+                                                     !(snew_v > 0.0f && snew_v < INFINITY)) != 0;
+    const float rcn_m = 1.0f / cn_m, rcn_v = 1.0f / cn_v;
+    const float qoff_m = -log2_hw(snew_m), qoff_v = -log2_hw(snew_v);
 
     // ---- requantize
 #pragma unroll
@@ -256,30 +330,45 @@ __global__ __launch_bounds__(256) void k_fp8_adamw(void* __restrict__ params, co
         float qm[4], qv[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            float em = m[j][i], ev = v[j][i];
-            if (EXPAND) {
-                float xm = fabsf(em) / cn_m, xv = ev / cn_v;
-                float pm = odd_k ? pow_full(xm, k_m) : pow_fast(xm, k_m);
-                float pv = odd_k ? pow_full(xv, k_v) : pow_fast(xv, k_v);
-                em = copysignf(pm, em);
-                ev = pv;
+            const float em = m[j][i], ev = v[j][i];
+            if (!odd_out) {
+                qm[i] = copysignf(exp2_hw(fmaf(log2_hw(fabsf(em) * rcn_m), k_m, qoff_m)), em);
+                qv[i] = exp2_hw(fmaf(log2_hw(ev * rcn_v), k_v, qoff_v));
+            } else {
+                qm[i] = copysignf(pow_full(fabsf(em) / cn_m, k_m), em) / snew_m;
+                qv[i] = pow_full(ev / cn_v, k_v) / snew_v;
             }
-            qm[i] = em / snew_m;
-            qv[i] = ev / snew_v;
         }
-        store_codes4(exp_avg, e0 + 32 * j, lim, cvt4_fp8<kE4M3>(qm[0], qm[1], qm[2], qm[3]));
-        store_codes4(exp_avg_sq, e0 + 32 * j, lim, cvt4_fp8<kE4M3>(qv[0], qv[1], qv[2], qv[3]));
+        store_codes4(exp_avg, e0 + 32 * j, FULL ? (int64_t)1 << 62 : lim, cvt4_fp8<kE4M3>(qm[0], qm[1], qm[2], qm[3]));
+        store_codes4(exp_avg_sq, e0 + 32 * j, FULL ? (int64_t)1 << 62 : lim, cvt4_fp8<kE4M3>(qv[0], qv[1], qv[2], qv[3]));
     }
     if (gvalid && lam == 0) {
         scale_m[gi] = snew_m;
         scale_v[gi] = snew_v;
-        if (EXPAND) {
-            expand_m[gi] = k_m;
-            expand_v[gi] = k_v;
-            sqrtmm_m[gi] = cn_m;
-            sqrtmm_v[gi] = cn_v;
-        }
+        expand_m[gi] = k_m;
+        expand_v[gi] = k_v;
+        sqrtmm_m[gi] = cn_m;
+        sqrtmm_v[gi] = cn_v;
     }
+}
+
+template <int PDT>
+__global__ __launch_bounds__(256) void k_fp8_adamw_expand(void* __restrict__ params, const void* __restrict__ grads,
+                                                           uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
+                                                           float* __restrict__ expand_m, float* __restrict__ sqrtmm_m,
+                                                           uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
+                                                           float* __restrict__ expand_v, float* __restrict__ sqrtmm_v,
+                                                           AdamArgs A, int64_t numel, int64_t ngroups) {
+    enable_fp8_saturation();
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (wave * 8 >= ngroups) return;  // whole wave out of range (wave-uniform)
+    if ((wave * 8 + 8) * kGroup <= numel)
+        adamw_expand_wave<PDT, true>(params, grads, exp_avg, scale_m, expand_m, sqrtmm_m, exp_avg_sq, scale_v, expand_v,
+                                     sqrtmm_v, A, numel, ngroups, wave, lane);
+    else
+        adamw_expand_wave<PDT, false>(params, grads, exp_avg, scale_m, expand_m, sqrtmm_m, exp_avg_sq, scale_v, expand_v,
+                                      sqrtmm_v, A, numel, ngroups, wave, lane);
 }
 
 }  // namespace coat
@@ -312,13 +401,12 @@ static int adamw_common(void* params, const void* grads, int p_dtype, void* exp_
     hipStream_t st = (hipStream_t)stream;
 #define LAUNCH(PDT)                                                                                                   \
     if (expand)                                                                                                       \
-        hipLaunchKernelGGL((k_fp8_adamw<PDT, true>), dim3((unsigned)blocks), dim3(256), 0, st, params, grads,         \
+        hipLaunchKernelGGL((k_fp8_adamw_expand<PDT>), dim3((unsigned)blocks), dim3(256), 0, st, params, grads,        \
                            (uint8_t*)exp_avg, scale_m, expand_m, sqrtmm_m, (uint8_t*)exp_avg_sq, scale_v, expand_v,   \
                            sqrtmm_v, A, numel, ngroups);                                                              \
     else                                                                                                              \
-        hipLaunchKernelGGL((k_fp8_adamw<PDT, false>), dim3((unsigned)blocks), dim3(256), 0, st, params, grads,        \
-                           (uint8_t*)exp_avg, scale_m, nullptr, nullptr, (uint8_t*)exp_avg_sq, scale_v, nullptr,      \
-                           nullptr, A, numel, ngroups);
+        hipLaunchKernelGGL((k_fp8_adamw_plain<PDT>), dim3((unsigned)blocks), dim3(256), 0, st, params, grads,         \
+                           (uint8_t*)exp_avg, scale_m, (uint8_t*)exp_avg_sq, scale_v, A, numel, ngroups);
     switch (p_dtype) {
         case COAT_F32: LAUNCH(kF32); break;
         case COAT_BF16: LAUNCH(kBF16); break;
