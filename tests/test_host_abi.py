@@ -1,0 +1,94 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares; host-side mirrors of
+the reference interface validate their arguments the way the reference does.  No compute calls (no GPU here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from coat_amd import _hip
+
+    header = open(os.path.join(ROOT, "include", "coat_hip.h")).read()
+    declared = set(re.findall(r"\b(coat_[a-z0-9_]+)\s*\(", header))
+    declared -= {"coat_status", "coat_dtype", "coat_fp8"}
+    assert len(declared) >= 11
+    L = _hip.lib()
+    for name in sorted(declared):
+        assert hasattr(L, name), f"{name} declared in include/coat_hip.h but not exported"
+    assert set(_hip.SIGNATURES) <= declared
+    assert b"gfx950" in L.coat_version()
+    assert b"128 per-group" in L.coat_status_string(-4)
+
+
+def test_argument_validation_without_gpu():
+    """Rejected arguments return before any launch, so these run without a GPU."""
+    from coat_amd import _hip
+
+    L = _hip.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.c_void_p(ctypes.addressof(buf) & ~15)
+    assert L.coat_fp8_quantize(p, 1, p, p, 1, 4, 40, 16, 0, None) == -2  # N % QB
+    assert L.coat_fp8_quantize(p, 7, p, p, 1, 4, 64, 16, 0, None) == -3  # dtype
+    assert L.coat_fp8_quantize(None, 1, p, p, 1, 4, 64, 16, 0, None) == -1
+    assert L.coat_fp8_quantize(p, 1, p, p, 1, 0, 64, 16, 0, None) == 0  # empty
+    assert L.coat_fp8_quantize(ctypes.c_void_p(p.value + 2), 1, p, p, 1, 4, 64, 16, 0, None) == -5
+    assert L.coat_fp8_quantize_transpose(p, 1, p, p, p, p, 1, 24, 64, 16, 0, None) == -2  # M % QB
+    assert L.coat_fp8_transpose(p, p, 8, 64, None) == -2
+    assert L.coat_fp8_adamw_step(p, p, 0, p, p, p, p, 0.9, 0.95, 1e-3, 0.1, 1e-8, 1, 64, 256, 2, None) == -4
+    assert L.coat_fp8_adamw_step(p, p, 0, p, p, p, p, 0.9, 0.95, 1e-3, 0.1, 1e-8, 1, 128, 256, 3, None) == -2
+    with pytest.raises(RuntimeError, match="128 per-group"):
+        _hip.check(-4, "x")
+    with pytest.raises(ValueError):
+        _hip.check(-2, "x")
+
+
+def test_quantization_config_defaults():
+    from coat_amd.utils._fp8_quantization_config import QuantizationConfig
+
+    q = QuantizationConfig()
+    assert (q.fabit, q.fwbit, q.fobit, q.babit, q.bwbit, q.bobit) == ("E4M3",) * 3 + ("E5M2",) * 3
+    assert q.group_size == 16 and q.qgroup_size == 128 and q.expand_min == 16 and q.weight_memory_efficient is True
+    assert q.first_order_expansion == "true" and q.epsilon == 1e-10
+    q2 = QuantizationConfig(group_size=32, unknown_flag=1)  # unknown keywords are swallowed, as in the reference
+    assert q2.group_size == 32 and not hasattr(q2, "unknown_flag")
+
+
+def test_coatadamw_constructor_and_expansion_switch():
+    from coat_amd.optimizer.fp8_adamw import CoatAdamW
+    from coat_amd.utils._fp8_quantization_config import QuantizationConfig
+
+    w = torch.nn.Parameter(torch.zeros(4, 4))
+    for bad in (dict(lr=-1.0), dict(eps=-1.0), dict(betas=(1.0, 0.9)), dict(betas=(0.9, 1.0)), dict(weight_decay=-0.1)):
+        with pytest.raises(ValueError):
+            CoatAdamW([w], **bad)
+    with pytest.raises(AssertionError):
+        CoatAdamW([w], qargs=QuantizationConfig(first_order_expansion="true", second_order_expansion="false"))
+    assert CoatAdamW([w]).use_expansion
+    assert CoatAdamW([w], qargs=QuantizationConfig(first_order_expansion="expansion", second_order_expansion="expansion")).use_expansion
+    # the OLMo YAMLs' spelling "expand" silently selects the plain kernel in the reference too (fp8_adamw.py:293)
+    assert not CoatAdamW([w], qargs=QuantizationConfig(first_order_expansion="expand", second_order_expansion="expand")).use_expansion
+    opt = CoatAdamW([w])
+    w.grad = torch.zeros(4, 4)
+    with pytest.raises(RuntimeError):  # CPU tensors are refused loudly, there is no fallback
+        opt.step()
+
+
+def test_dropin_aliases():
+    import coat_amd.dropin  # noqa: F401
+    import qoptim_cuda
+    from coat.activation.real_quantization import fp8_quantize
+    from coat.optimizer.fp8_adamw import CoatAdamW
+
+    assert hasattr(qoptim_cuda, "fp8_adamw_expand_step") and callable(fp8_quantize) and CoatAdamW.__name__ == "CoatAdamW"
+
+
+def test_entry_points_refuse_cpu_tensors():
+    from coat_amd.activation.real_quantization import fp8_quantize
+
+    with pytest.raises(RuntimeError, match="GPU"):
+        fp8_quantize(torch.zeros(4, 64, dtype=torch.bfloat16), 16, "E4M3")
