@@ -28,6 +28,16 @@ SIGNATURES = {
     "coat_fp8_division": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_transpose": [_vp, _vp, _i64, _i64, _vp],
     "coat_fp8_dequantize": [_vp, _i, _vp, _i, _vp, _i64, _i64, _i, _vp],
+    "coat_fp8_silu_forward": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],
+    "coat_fp8_silu_backward": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
+    "coat_fp8_mul_forward": [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp],
+    "coat_fp8_mul_backward": [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
+    "coat_fp8_gelu_forward": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp],
+    "coat_fp8_gelu_backward": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
+    "coat_fp8_add_fwd": [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
+    "coat_fp8_add_bwd": [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
+    "coat_fp8_rmsnorm_forward": [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i64, _i64, _i, _f, _vp],
+    "coat_fp8_rmsnorm_backward": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
     "coat_fp8_adamw_expand_step": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _i,
                                    _i64, _i64, _vp],
     "coat_fp8_adamw_step": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _i64, _i64, _vp],

@@ -1,0 +1,24 @@
+"""Shared marshalling of the fused element-wise entry points (SiLU / GELU / mul / add)."""
+import torch
+
+from ... import _hip
+from .common import flatten_2d
+
+
+def prep_pg(x, s_x):
+    """Flatten a per-group FP8 tensor and its scales to 2-D dense GPU tensors; returns (x2d, s2d, batch)."""
+    x, batch = flatten_2d(x)
+    s_x, _ = flatten_2d(s_x)
+    return _hip.dense(x), _hip.dense(s_x), batch
+
+
+def prep_bf16(g):
+    g, _ = flatten_2d(g)
+    if g.dtype != torch.bfloat16:
+        g = g.to(torch.bfloat16)
+    return _hip.dense(g)
+
+
+def new_max(device):
+    """Zero-initialised fp32 device scalar for the order-independent atomic maximum of the group scales."""
+    return torch.zeros((), dtype=torch.float32, device=device)

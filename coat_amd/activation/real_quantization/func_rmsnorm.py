@@ -1,0 +1,46 @@
+"""FP8 RMSNorm forward / backward.
+Reference: coat/activation/real_quantization/func_rmsnorm.py:223-335."""
+import torch
+
+from ... import _hip
+from ._division import _division
+from ._fused import new_max, prep_bf16, prep_pg
+from .common import restore
+
+_DW_PARTIALS = 512  # blocks of the dx kernel; each contributes one fp32 partial row of dw
+
+
+def fp8_rmsnorm_forward(x, s_x, w, QB, eps, transpose_output_2d=False):
+    """Returns (qy, s_y_max, qy_t, (w, rstd, num_warps)); qy is per-tensor FP8 in x's dtype."""
+    x, s_x, batch = prep_pg(x, s_x)
+    M, N = x.shape
+    w = _hip.dense(w)
+    y = torch.empty_like(x, dtype=torch.bfloat16)
+    s_row = torch.empty((M,), dtype=torch.bfloat16, device=x.device)
+    rstd = torch.empty((M,), dtype=torch.float32, device=x.device)
+    s_max = new_max(x.device)
+    _hip.check(_hip.lib().coat_fp8_rmsnorm_forward(
+        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.dt(w), _hip.ptr(y), _hip.ptr(s_row),
+        _hip.ptr(rstd), _hip.ptr(s_max), M, N, QB, float(eps), _hip.stream(x.device)), "fp8_rmsnorm_forward")
+    qy, s_y_max, qy_t = _division(y, x.dtype, s_max.to(torch.bfloat16), True, True, "fp8_rmsnorm_forward")
+    if batch is not None and not transpose_output_2d:
+        qy_t = qy_t.reshape(batch, -1, N)
+    num_warps = 8  # kept in the tuple for signature compatibility; the HIP kernels do not use it
+    return restore(qy, batch), s_y_max, qy_t, (w, rstd, num_warps)
+
+
+def fp8_rmsnorm_backward(x, s_x, g, w, v, QB, num_warps):
+    """Returns (dx bf16, dw in w's dtype); ``v`` is the rstd saved by the forward."""
+    x, s_x, batch = prep_pg(x, s_x)
+    g = prep_bf16(g)
+    M, N = g.shape
+    w = _hip.dense(w)
+    rstd = _hip.dense(v.to(torch.float32))
+    dx = torch.empty_like(g, dtype=torch.bfloat16)
+    dw = torch.empty((N,), dtype=w.dtype, device=w.device)
+    nparts = min(_DW_PARTIALS, M)
+    partial = torch.empty((nparts, N), dtype=torch.float32, device=w.device)
+    _hip.check(_hip.lib().coat_fp8_rmsnorm_backward(
+        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(g), _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd),
+        _hip.ptr(dx), _hip.ptr(dw), _hip.ptr(partial), nparts, M, N, QB, _hip.stream(x.device)), "fp8_rmsnorm_backward")
+    return restore(dx, batch), dw

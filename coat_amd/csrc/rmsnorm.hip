@@ -1,0 +1,267 @@
+// FP8 RMSNorm forward / backward for gfx950.
+//
+// Reference: coat/activation/real_quantization/func_rmsnorm.py (_rms_norm_fwd_fused :54-111,
+// _rms_norm_bwd_dx_fused :121-196, _rms_norm_bwd_dwdb :200-220).
+//
+// One 256-thread block per row; a lane owns 16-element chunks `lane + 256*it` of the row (16 B of FP8 codes,
+// 2 x 16 B of bf16 per chunk), so a row of up to 16384 columns lives in registers for the two passes over it
+// (statistic, then normalise).  Row sums are reduced in a fixed order (in-lane, DPP butterfly per wave, then
+// the four wave partials in index order), so results are deterministic, unlike the reference's lock-ordered dw.
+// dw is a two-stage reduction: every block accumulates the rows it owns into fp32 registers and writes one
+// partial row; a second kernel sums the partials in block order.
+#include <math.h>
+
+#include "coat_device.h"
+#include "coat_host.h"
+
+namespace coat {
+
+__device__ __forceinline__ float block_sum_256(float v, float* smem) {
+    v = cluster_sum<64>(v);
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();  // smem may still be read from a previous call
+    if ((threadIdx.x & 63) == 0) smem[wave] = v;
+    __syncthreads();
+    return ((smem[0] + smem[1]) + smem[2]) + smem[3];
+}
+__device__ __forceinline__ float block_max_256(float v, float* smem) {
+    v = cluster_max<64>(v);
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) smem[wave] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(smem[0], smem[1]), fmaxf(smem[2], smem[3]));
+}
+
+template <int KIND> __device__ __forceinline__ void dequant16(const uint8_t* q, const void* s, int s_dt, int64_t row_off,
+                                                             int64_t srow_off, int col, int qb, float* v) {
+    uint4 c = *(const uint4*)(q + row_off + col);
+    float sc;
+    const int64_t si = srow_off + col / qb;
+    if (s_dt == kBF16) sc = u2f((uint32_t)((const uint16_t*)s)[si] << 16);
+    else if (s_dt == kF32) sc = ((const float*)s)[si];
+    else sc = f16lo(((const uint16_t*)s)[si]);
+    uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float f[4];
+        fp8x4_to_f32<KIND>(w[k], f);
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[4 * k + i] = f[i] * sc;
+    }
+}
+template <int WDT> __device__ __forceinline__ void load_w16(const void* w, int col, float* o) {
+    if (WDT == kF32) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float4 t = ((const float4*)((const float*)w + col))[i];
+            o[4 * i] = t.x; o[4 * i + 1] = t.y; o[4 * i + 2] = t.z; o[4 * i + 3] = t.w;
+        }
+    } else {
+        const uint4* src = (const uint4*)((const uint16_t*)w + col);
+        uint4 a = src[0], b = src[1];
+        uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            o[2 * k] = WDT == kBF16 ? bf16lo(u[k]) : f16lo(u[k]);
+            o[2 * k + 1] = WDT == kBF16 ? bf16hi(u[k]) : f16hi(u[k]);
+        }
+    }
+}
+__device__ __forceinline__ void store_bf16_16(void* p, int64_t off, const float* v) {
+    uint32_t w[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) w[k] = pack_bf16x2(v[2 * k], v[2 * k + 1]);
+    uint4* dst = (uint4*)((uint16_t*)p + off);
+    dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+    dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+}
+
+// Forward: y = bf16(x * rstd * w), rstd[row], row scale (max|y| + 1e-10)/fp8max (bf16), tensor max of the row scales.
+template <int KIND, int WDT, int ITERS>
+__global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                      const void* __restrict__ w, void* __restrict__ y,
+                                                      void* __restrict__ s_row, float* __restrict__ rstd_out,
+                                                      float* __restrict__ s_max, int N, int qb, float eps) {
+    __shared__ float smem[4];
+    const int64_t row = blockIdx.x;
+    const int64_t row_off = row * N, srow_off = row * (N / qb);
+    float x[ITERS][16];
+    float ss = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int col = (threadIdx.x + it * 256) * 16;
+        if (col < N) {
+            dequant16<KIND>(q, s, s_dt, row_off, srow_off, col, qb, x[it]);
+#pragma unroll
+            for (int i = 0; i < 16; i++) ss += x[it][i] * x[it][i];
+        }
+    }
+    const float var = block_sum_256(ss, smem) / (float)N;
+    const float rstd = 1 / sqrtf(var + eps);
+    float amax = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int col = (threadIdx.x + it * 256) * 16;
+        if (col < N) {
+            float wv[16], yv[16];
+            load_w16<WDT>(w, col, wv);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                yv[i] = (x[it][i] * rstd) * wv[i];
+                amax = fmaxf(amax, fabsf(yv[i]));
+            }
+            store_bf16_16(y, row_off + col, yv);
+        }
+    }
+    amax = block_max_256(amax, smem);
+    if (threadIdx.x == 0) {
+        const float sr = group_scale<KIND>(amax);
+        ((uint16_t*)s_row)[row] = (uint16_t)f2bf16(sr);
+        rstd_out[row] = rstd;
+        atomic_max_nonneg(s_max, sr);
+    }
+}
+
+// Backward: dx = bf16((w*dy - xhat * mean(xhat*w*dy)) * rstd); per-block partial of dw = sum_rows dy * xhat.
+template <int KIND, int WDT, int ITERS>
+__global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                      const void* __restrict__ dy, const void* __restrict__ w,
+                                                      const float* __restrict__ rstd_in, void* __restrict__ dx,
+                                                      float* __restrict__ dw_partial, int64_t M, int N, int qb) {
+    __shared__ float smem[4];
+    float acc[ITERS][16];
+#pragma unroll
+    for (int it = 0; it < ITERS; it++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[it][i] = 0.0f;
+    for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+        const int64_t row_off = row * N, srow_off = row * (N / qb);
+        const float rstd = rstd_in[row];
+        float xhat[ITERS][16], wdy[ITERS][16];
+        float dot = 0.0f;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+            const int col = (threadIdx.x + it * 256) * 16;
+            if (col < N) {
+                float xv[16], wv[16], gv[16];
+                dequant16<KIND>(q, s, s_dt, row_off, srow_off, col, qb, xv);
+                load_w16<WDT>(w, col, wv);
+                {
+                    const uint4* src = (const uint4*)((const uint16_t*)dy + row_off + col);
+                    uint4 a = src[0], b = src[1];
+                    uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        gv[2 * k] = bf16lo(u[k]);
+                        gv[2 * k + 1] = bf16hi(u[k]);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    xhat[it][i] = xv[i] * rstd;
+                    wdy[it][i] = wv[i] * gv[i];
+                    dot += xhat[it][i] * wdy[it][i];
+                    acc[it][i] += gv[i] * xhat[it][i];
+                }
+            }
+        }
+        const float c1 = block_sum_256(dot, smem) / (float)N;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+            const int col = (threadIdx.x + it * 256) * 16;
+            if (col < N) {
+                float o[16];
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[i] = (wdy[it][i] - (xhat[it][i] * c1)) * rstd;
+                store_bf16_16(dx, row_off + col, o);
+            }
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int col = (threadIdx.x + it * 256) * 16;
+        if (col < N) {
+            float4* dst = (float4*)(dw_partial + (int64_t)blockIdx.x * N + col);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[i] = make_float4(acc[it][4 * i], acc[it][4 * i + 1], acc[it][4 * i + 2], acc[it][4 * i + 3]);
+        }
+    }
+}
+
+// dw[col] = sum over blocks (in block order) of the partials, stored in the weight's dtype.
+template <int WDT>
+__global__ __launch_bounds__(256) void k_rmsnorm_dw(const float* __restrict__ partial, void* __restrict__ dw, int nblocks,
+                                                     int N) {
+    const int col = blockIdx.x * 256 + threadIdx.x;
+    if (col >= N) return;
+    float s = 0.0f;
+    for (int b = 0; b < nblocks; b++) s += partial[(int64_t)b * N + col];
+    store_from_f32<WDT>(dw, col, s);
+}
+
+}  // namespace coat
+
+using namespace coat;
+
+static int rms_check(int64_t M, int64_t N, int QB) {
+    if (M < 0 || N < 0) return COAT_EINVAL;
+    if (QB < 16 || (QB & (QB - 1)) || N % QB != 0 || N % 16 != 0) return COAT_ESHAPE;
+    if (N > 16384) return COAT_ESHAPE;  // a row is held in registers: 4 chunks of 16 per lane at most
+    return COAT_OK;
+}
+
+#define RMS_DISPATCH(KERNEL, GRID, ...)                                                                                \
+    {                                                                                                                  \
+        const int iters = N <= 4096 ? 1 : (N <= 8192 ? 2 : 4);                                                         \
+        if (fp8 != COAT_E4M3 && fp8 != COAT_E5M2) return COAT_EINVAL;                                                  \
+        if (w_dtype != COAT_BF16 && w_dtype != COAT_F32 && w_dtype != COAT_F16) return COAT_EDTYPE;                    \
+        switch ((fp8 * 3 + w_dtype) * 3 + (iters == 1 ? 0 : (iters == 2 ? 1 : 2))) {                                   \
+            RMS_CASES(KERNEL, GRID, __VA_ARGS__)                                                                       \
+            default: return COAT_EINVAL;                                                                               \
+        }                                                                                                              \
+    }
+#define RMS_CASE(KERNEL, GRID, K, W, I, ...)                                                                           \
+    case ((K * 3 + W) * 3 + (I == 1 ? 0 : (I == 2 ? 1 : 2))):                                                          \
+        hipLaunchKernelGGL((KERNEL<K, W, I>), dim3((unsigned)(GRID)), dim3(256), 0, st, __VA_ARGS__);                  \
+        break;
+#define RMS_CASES(KERNEL, GRID, ...)                                                                                   \
+    RMS_CASE(KERNEL, GRID, 0, 0, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 0, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 0, 4, __VA_ARGS__) \
+    RMS_CASE(KERNEL, GRID, 0, 1, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 1, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 1, 4, __VA_ARGS__) \
+    RMS_CASE(KERNEL, GRID, 0, 2, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 2, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 2, 4, __VA_ARGS__) \
+    RMS_CASE(KERNEL, GRID, 1, 0, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 0, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 0, 4, __VA_ARGS__) \
+    RMS_CASE(KERNEL, GRID, 1, 1, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 1, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 1, 4, __VA_ARGS__) \
+    RMS_CASE(KERNEL, GRID, 1, 2, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 2, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 2, 4, __VA_ARGS__)
+
+extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype,
+                                        void* y, void* s_row, float* rstd, float* s_max, int64_t M, int64_t N, int QB,
+                                        float eps, void* stream) {
+    if (int e = rms_check(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !s_x || !w || !y || !s_row || !rstd || !s_max) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(y)) return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    RMS_DISPATCH(k_rmsnorm_fwd, M, (const uint8_t*)x, s_x, s_dtype, w, y, s_row, rstd, s_max, (int)N, QB, eps)
+    return coat_launch_status();
+}
+
+extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
+                                         const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
+                                         float* dw_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream) {
+    if (int e = rms_check(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !s_x || !dy || !w || !rstd || !dx || !dw || !dw_partial || n_partial <= 0) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(dy) || !coat_aligned16(dx) || !coat_aligned16(dw_partial))
+        return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t grid = n_partial < M ? n_partial : M;
+    RMS_DISPATCH(k_rmsnorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, rstd, dx, dw_partial, M, (int)N, QB)
+    if (int e = coat_launch_status()) return e;
+    const int cols_blocks = (int)((N + 255) / 256);
+    switch (w_dtype) {
+        case COAT_F32: hipLaunchKernelGGL((k_rmsnorm_dw<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        case COAT_BF16: hipLaunchKernelGGL((k_rmsnorm_dw<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        default: hipLaunchKernelGGL((k_rmsnorm_dw<kF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+    }
+    return coat_launch_status();
+}

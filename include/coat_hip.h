@@ -73,6 +73,51 @@ int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, void* strea
 int coat_fp8_dequantize(const void* q, int fp8, const void* s, int s_dtype, void* y, int64_t M, int64_t N, int QB,
                         void* stream);
 
+/* ---- fused element-wise kernels -----------------------------------------------------------------
+ * Inputs x* are per-group FP8 ([M,N] codes + [M,N/QB] scales of s_dtype); g is a bf16 gradient.
+ * "value" outputs y are bf16 [M,N]; s_y (optional, may be NULL) receives the bf16 per-group scales
+ * (amax_g + 1e-10) / fp8max(fp8_out) of the fp32 value; s_max (optional) is a zero-initialised fp32 device
+ * scalar that receives their maximum (the per-tensor scale of the division that follows in the reference). */
+
+/* rq/silu_fwd.py:152 fp8_silu_forward (kernel :47-149): y = per-group fp8(silu(x)), same fp8 type as x. */
+int coat_fp8_silu_forward(const void* x, int fp8, const void* s_x, int s_dtype, void* y, void* s_y, int64_t M,
+                          int64_t N, int QB, void* stream);
+/* rq/silu_bwd.py:170 fp8_silu_backward (kernel :47-167): y = bf16((sig + x*sig*(1-sig)) * g). */
+int coat_fp8_silu_backward(const void* x, int fp8_in, const void* s_x, int s_dtype, const void* g, void* y, void* s_y,
+                           float* s_max, int fp8_out, int64_t M, int64_t N, int QB, void* stream);
+/* rq/mul_fwd.py:191 fp8_mul_forward (kernel :51-188): y = bf16(x1 * x2). */
+int coat_fp8_mul_forward(const void* x1, const void* s_x1, const void* x2, const void* s_x2, int fp8_in, int s_dtype,
+                         void* y, void* s_y, float* s_max, int64_t M, int64_t N, int QB, void* stream);
+/* rq/mul_bwd.py:221 fp8_mul_backward (kernel :49-218): y1 = bf16(g * x2); y2 = bf16(g * x1) with scales. */
+int coat_fp8_mul_backward(const void* x1, const void* s_x1, const void* x2, const void* s_x2, int fp8_in, int s_dtype,
+                          const void* g, void* y1, void* y2, void* s_y2, float* s_max, int fp8_out, int64_t M,
+                          int64_t N, int QB, void* stream);
+/* rq/gelu_fwd.py:152 fp8_gelu_forward (kernel :47-149): y = bf16(x * (1 + erf(x / sqrt 2)) / 2). */
+int coat_fp8_gelu_forward(const void* x, int fp8, const void* s_x, int s_dtype, void* y, void* s_y, float* s_max,
+                          int64_t M, int64_t N, int QB, void* stream);
+/* rq/gelu_bwd.py:173 fp8_gelu_backward (kernel :47-170): y = bf16((cdf + x * exp(-x^2/2) / sqrt(2 pi)) * g). */
+int coat_fp8_gelu_backward(const void* x, int fp8_in, const void* s_x, int s_dtype, const void* g, void* y, void* s_y,
+                           float* s_max, int fp8_out, int64_t M, int64_t N, int QB, void* stream);
+/* rq/add_fwd.py:162 fp8_add_Ifp_Ifp_Ofp_Og16 (kernel :46-159): bf16 x1, x2 -> y = bf16(x1 + x2) and the
+ * per-group FP8 (q, s_q) of the fp32 sum. */
+int coat_fp8_add_fwd(const void* x1, const void* x2, void* y, void* q, void* s_q, int fp8_out, int64_t M, int64_t N,
+                     int QB, void* stream);
+/* rq/add_bwd.py:147 fp8_add_Ifp_Ifp_Ofp_Opt (kernel :48-144): y = bf16(x1 + x2), scales of the fp32 sum. */
+int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s_y, float* s_max, int fp8_out, int64_t M,
+                     int64_t N, int QB, void* stream);
+
+/* rq/func_rmsnorm.py:223 fp8_rmsnorm_forward (kernel :54-111): y = bf16(x * rstd * w); s_row [M] bf16 row scales
+ * (max|y| + 1e-10) / fp8max; rstd [M] fp32; s_max as above.  N <= 16384, N % 16 == 0. */
+int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype, void* y,
+                             void* s_row, float* rstd, float* s_max, int64_t M, int64_t N, int QB, float eps,
+                             void* stream);
+/* rq/func_rmsnorm.py:281 fp8_rmsnorm_backward (kernels :121-196, :200-220): dx bf16 [M,N], dw [N] in w's dtype.
+ * dw_partial: caller-provided fp32 workspace [n_partial, N]; the kernel uses min(n_partial, M) blocks and sums their
+ * partial rows in block order (deterministic, unlike the reference's lock-ordered accumulation). */
+int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* w,
+                              int w_dtype, const float* rstd, void* dx, void* dw, float* dw_partial, int n_partial,
+                              int64_t M, int64_t N, int QB, void* stream);
+
 /* ---- optimizer -------------------------------------------------------------------------------- */
 
 /* qoptim_cuda.fp8_adamw_expand_step (coat/optimizer/kernels/bindings.cpp:7,
