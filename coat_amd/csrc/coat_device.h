@@ -55,6 +55,12 @@ template <int DT> __device__ __forceinline__ void store_from_f32(void* p, int64_
     else if (DT == kBF16) ((uint16_t*)p)[i] = (uint16_t)f2bf16(v);
     else ((uint16_t*)p)[i] = (uint16_t)f2f16(v);
 }
+// Scalar load with a run-time dtype (scales, bias): wave-uniform branch.
+__device__ __forceinline__ float load_rt_f32(const void* p, int64_t i, int dt) {
+    if (dt == kBF16) return u2f((uint32_t)((const uint16_t*)p)[i] << 16);
+    if (dt == kF32) return ((const float*)p)[i];
+    return f16lo(((const uint16_t*)p)[i]);
+}
 // Round an fp32 value to dtype DT and back (what storing and re-loading would give).
 template <int DT> __device__ __forceinline__ float round_to(float v) {
     if (DT == kF32) return v;

@@ -118,6 +118,17 @@ int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dty
                               int w_dtype, const float* rstd, void* dx, void* dw, float* dw_partial, int n_partial,
                               int64_t M, int64_t N, int QB, void* stream);
 
+/* ---- GEMM -------------------------------------------------------------------------------------------
+ * rq/linear.py:172 fp8matmul (kernel :61-169): C[M,N] = (A[M,K] . B[N,K]^T) * (float(*scale_a) * float(*scale_b))
+ * (+ bias[N]), fp32 accumulation on FP8 MFMA.  A and B are row-major with K contiguous (the reference passes B as
+ * the .t() view of such a matrix, linear.py:253-302); fmt_a / fmt_b are coat_fp8 values and may differ.
+ * out_kind 0: C is bf16 [M,N] (:166-169).  out_kind 1 / 2: C is e4m3 / e5m2 [M,N], quantized per 1 x QB group along
+ * N with scale (amax + 1e-10) / fp8max, and c_scale is bf16 [M, N/QB] (:139-164); QB must be 16.
+ * scale_a / scale_b: one element each of s_dtype in device memory.  K % 16 == 0. */
+int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
+                  const void* scale_a, const void* scale_b, int s_dtype, const void* bias, int bias_dtype, int64_t M,
+                  int64_t N, int64_t K, int QB, void* stream);
+
 /* ---- optimizer -------------------------------------------------------------------------------- */
 
 /* qoptim_cuda.fp8_adamw_expand_step (coat/optimizer/kernels/bindings.cpp:7,
