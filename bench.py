@@ -80,6 +80,33 @@ def make_quantize_workload(dev, torch, transpose):
                           "kernel": "k_quantize_transpose" if transpose else "k_quantize_pg"}
 
 
+def make_gemm_workload(dev, torch, which):
+    """BASELINE configs[2]: X [8192,4096] x W [11008,4096]; which = fwd | dgrad | wgrad (the three GEMMs of FP8Linear)."""
+    from coat_amd.activation.real_quantization.linear import fp8matmul
+
+    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+    T, K, N = 8192, 4096, 11008
+    gen = torch.Generator(device="cpu").manual_seed(0)
+
+    def rnd(shape, dtype, std):
+        return (torch.randn(shape, generator=gen) * std).to(dtype).to(dev)
+
+    one = torch.tensor(0.01, dtype=torch.bfloat16, device=dev)
+    if which == "fwd":      # Y[T,N] = X[T,K] W[N,K]^T
+        a, b, (M_, N_, K_) = rnd((T, K), E4, 1.0), rnd((N, K), E4, 1.0), (T, N, K)
+    elif which == "dgrad":  # dX[T,K] = G[T,N] Wt[K,N]^T, G is e5m2
+        a, b, (M_, N_, K_) = rnd((T, N), E5, 1.0), rnd((K, N), E4, 1.0), (T, K, N)
+    else:                   # dW[N,K] = Gt[N,T] Xt[K,T]^T
+        a, b, (M_, N_, K_) = rnd((N, T), E5, 1.0), rnd((K, T), E4, 1.0), (N, K, T)
+
+    def step():
+        fp8matmul(a, b.t(), False, one, one, 16)
+
+    flops = 2 * M_ * N_ * K_
+    return step, flops, {"workload": f"fp8matmul {which}: [{M_},{K_}] x [{N_},{K_}]^T -> bf16, per-tensor scales",
+                         "M": M_, "N": N_, "K": K_, "kernel": "k_fp8_gemm"}
+
+
 def cpu_baseline_adamw(torch):
     """The plain-C oracle (one thread) on a bounded sample: same hyper-parameters, step 10 state built by the
     oracle itself, sample sized for roughly 10-20 s."""
@@ -113,7 +140,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose"])
+    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (known traffic, to scale rocprofv3 counters)")
@@ -134,8 +161,11 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    is_gemm = args.workload.startswith("gemm")
     if args.workload == "adamw":
         step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch)
+    elif is_gemm:
+        step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1])
     else:
         step, nbytes, cfg = make_quantize_workload(dev, torch, args.workload == "quantize_transpose")
 
@@ -163,14 +193,17 @@ def main():
     value = nbytes / (ms_per_step * 1e-3) / 1e9
     achieved = nbytes / (avg_ms * 1e-3) / 1e9
 
+    unit, peak, bound = ("TFLOP/s", 5000.0, "mfma") if is_gemm else ("GB/s", HBM_PEAK_GBS, "hbm")
+    if is_gemm:  # nbytes holds FLOPs for the GEMM workloads; report TFLOP/s
+        value, achieved = value / 1e3, achieved / 1e3
     out = {
         "metric": "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms",
-        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic", "config": cfg,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "algorithmic_bytes_per_launch": nbytes, "kernel_ms_avg": round(avg_ms, 5),
+        "dtype": "fp8" if is_gemm else "f32", "data": "synthetic", "config": cfg,
+        "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     ("algorithmic_flops_per_launch" if is_gemm else "algorithmic_bytes_per_launch"): nbytes, "kernel_ms_avg": round(avg_ms, 5),
                      "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5)},
     }
     if args.workload == "adamw" and not args.no_cpu_baseline:
