@@ -17,3 +17,4 @@ from .mul_fwd import fp8_mul_forward
 from .silu_bwd import fp8_silu_backward
 from .silu_fwd import fp8_silu_forward
 from .linear import fp8_linear_backward, fp8_linear_forward
+from .func_quantize import Coat_quantize_bgn, Coat_quantize_end
