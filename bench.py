@@ -107,6 +107,75 @@ def make_gemm_workload(dev, torch, which):
                          "M": M_, "N": N_, "K": K_, "kernel": "k_fp8_gemm"}
 
 
+class Bf16DecoderLayer:
+    """The same Llama decoder layer in plain bf16 torch (F.linear / F.rms_norm / F.silu / SDPA): the baseline the FP8
+    layer has to beat (benchmark/benchmark_llamalayer.py of the reference times HF's LlamaDecoderLayer the same way)."""
+
+    def __init__(self, torch, coat_layer):
+        self.torch = torch
+        self.p = {n: p.detach().clone().requires_grad_(True) for n, p in coat_layer.named_parameters()}
+        self.nh = coat_layer.self_attn.num_heads
+
+    def __call__(self, x):
+        import torch.nn.functional as F
+        from coat_amd.models.coat_llama import apply_rotary_pos_emb, rotary_cos_sin
+        p, torch = self.p, self.torch
+        B, S, H = x.shape
+        hd = H // self.nh
+        h = F.rms_norm(x, (H,), p["input_layernorm.weight"], 1e-5)
+        q = F.linear(h, p["BeforeAttention.q_proj.weight"]).view(B, S, self.nh, hd).transpose(1, 2)
+        k = F.linear(h, p["BeforeAttention.k_proj.weight"]).view(B, S, self.nh, hd).transpose(1, 2)
+        v = F.linear(h, p["BeforeAttention.v_proj.weight"]).view(B, S, self.nh, hd).transpose(1, 2)
+        pos = torch.arange(S, device=x.device).unsqueeze(0).expand(B, -1)
+        cos, sin = rotary_cos_sin(pos, hd, 10000.0, x.dtype)
+        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, H)
+        x1 = x + F.linear(a, p["AfterAttention.o_proj.weight"])
+        h2 = F.rms_norm(x1, (H,), p["post_attention_layernorm.weight"], 1e-5)
+        m = F.silu(F.linear(h2, p["MLPResidual.gate_proj.weight"])) * F.linear(h2, p["MLPResidual.up_proj.weight"])
+        return x1 + F.linear(m, p["MLPResidual.down_proj.weight"])
+
+
+def make_layer_workload(dev, torch, size):
+    """BASELINE configs[4]: COAT Llama decoder layer fwd+bwd, batch 4 x seq 2048, random init N(0, 0.02)."""
+    from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
+    from coat_amd.models.coat_llama import CoatLlamaConfig, CoatLlamaDecoderLayer
+    from coat_amd.utils._fp8manager import FP8Manager
+
+    H, heads, I = (4096, 32, 11008) if size == "7b" else (5120, 40, 13824)
+    B, S = 4, 2048
+    torch.manual_seed(0)
+    cfg = CoatLlamaConfig(hidden_size=H, intermediate_size=I, num_attention_heads=heads)
+    layer = CoatLlamaDecoderLayer(cfg, 0)
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+    layer = layer.to(dev).to(torch.bfloat16).train()
+    bgn, end = Coat_quantize_bgn(layer.qargs), Coat_quantize_end(layer.qargs)
+    x = torch.randn(B, S, H, device=dev, dtype=torch.bfloat16)
+    gy = torch.randn(B, S, H, device=dev, dtype=torch.bfloat16) * 1e-2
+    ref = Bf16DecoderLayer(torch, layer)
+    state = {"first": True}
+
+    def step_fp8():
+        FP8Manager.is_first_microbatch = state["first"]  # True once, then False (benchmark_llamalayer.py:185-191)
+        state["first"] = False
+        xin = x.detach().requires_grad_(True)
+        h, q, s = bgn(xin)
+        (h, q, s), = layer(h, q, s)
+        end(h, q, s).backward(gy)
+
+    def step_bf16():
+        xin = x.detach().requires_grad_(True)
+        ref(xin).backward(gy)
+
+    gemm_flops = 3 * 2 * B * S * (4 * H * H + 3 * H * I)
+    return step_fp8, step_bf16, gemm_flops, {
+        "workload": f"CoatLlamaDecoderLayer fwd+bwd, Llama-2-{size.upper()} shape (H {H}, heads {heads}, I {I}), "
+                    f"batch {B} x seq {S}, FP8 linears/activations/norms, bf16 SDPA attention",
+        "tokens": B * S, "gemm_flops": gemm_flops}
+
+
 def cpu_baseline_adamw(torch):
     """The plain-C oracle (one thread) on a bounded sample: same hyper-parameters, step 10 state built by the
     oracle itself, sample sized for roughly 10-20 s."""
@@ -135,12 +204,49 @@ def cpu_baseline_adamw(torch):
             "sample": f"{reps} steps over the first {n} elements (4096 groups) of the tensor, oracle/adamw_ref.c, 1 thread"}
 
 
+def bench_layer(args, dev, torch):
+    step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1])
+
+    def time_it(fn):
+        for _ in range(max(2, args.warmup // 2)):
+            fn()
+        torch.cuda.synchronize()
+        evs = []
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / args.steps
+        ms = sorted(a.elapsed_time(b) for a, b in evs)
+        return wall, ms[len(ms) // 2]
+
+    wall8, med8 = time_it(step_fp8)
+    wall16, med16 = time_it(step_bf16)
+    out = {
+        "metric": "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms",
+        "value": round(wall8, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall8, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8", "data": "synthetic", "config": cfg,
+        "layer": {"fp8_ms_median": round(med8, 4), "bf16_ms_median": round(med16, 4), "bf16_ms_per_step": round(wall16, 4),
+                  "speedup_vs_bf16": round(med16 / med8, 4),
+                  "fp8_gemm_tflops_equiv": round(gemm_flops / (med8 * 1e-3) / 1e12, 1)},
+        "roofline": {"bound": "mfma", "achieved": round(gemm_flops / (med8 * 1e-3) / 1e12, 2), "peak": 5000.0,
+                     "unit": "TFLOP/s", "frac": round(gemm_flops / (med8 * 1e-3) / 1e12 / 5000.0, 4), "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad"])
+    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (known traffic, to scale rocprofv3 counters)")
@@ -162,6 +268,8 @@ def main():
     torch.cuda.set_device(dev)
 
     is_gemm = args.workload.startswith("gemm")
+    if args.workload.startswith("layer"):
+        return bench_layer(args, dev, torch)
     if args.workload == "adamw":
         step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch)
     elif is_gemm:

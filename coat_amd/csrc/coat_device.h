@@ -160,6 +160,12 @@ template <int LANES> __device__ __forceinline__ float cluster_sum(float v) {
 }
 
 // Order-independent device-wide maximum of non-negative floats (bit pattern order == value order).
-__device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) { atomicMax((unsigned int*)addr, f2u(v)); }
+// Atomics on one address serialise in L2 (~10 ns each), so callers reduce over a wave (or more) first, and the
+// atomic is skipped when a device-coherent read already shows a value that is not smaller: the stored maximum only
+// grows, so a stale reading can only cause a redundant atomic, never a lost update.
+__device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
+    const float cur = *(volatile float*)addr;
+    if (!(v <= cur)) atomicMax((unsigned int*)addr, f2u(v));
+}
 
 }  // namespace coat

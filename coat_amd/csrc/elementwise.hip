@@ -81,10 +81,13 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
     constexpr bool kQuantPg = (OP == kSiluFwd || OP == kAddFwd);         // emit per-group FP8 + scales
     constexpr bool kWriteY = !(OP == kSiluFwd);                          // emit the bf16 value
     enable_fp8_saturation();
-    const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int lpg = A.qb >> 4;  // lanes per group
+    float tensor_max = 0.0f;
+    // grid-stride over 256-chunk slabs: the trip count is block-uniform, so the lanes of a group stay together
+    for (int64_t base = (int64_t)blockIdx.x * 256; base < A.nchunk; base += (int64_t)gridDim.x * 256) {
+    const int64_t chunk = base + threadIdx.x;
     const bool ok = chunk < A.nchunk;
     const int64_t c = ok ? chunk : 0;
-    const int lpg = A.qb >> 4;  // lanes per group
 
     float a[16], b[16], g[16], v[16];
     if (kBf16In) {
@@ -141,8 +144,10 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
         if (ok) *(uint4*)((uint8_t*)A.q + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
     }
     if (A.s_out && ok && (threadIdx.x % lpg) == 0) ((uint16_t*)A.s_out)[(c * 16) / A.qb] = (uint16_t)f2bf16(s);
+    if (A.s_max) tensor_max = fmaxf(tensor_max, ok ? s : 0.0f);
+    }
     if (A.s_max) {
-        float wmax = cluster_max<64>(ok ? s : 0.0f);
+        const float wmax = cluster_max<64>(tensor_max);
         if ((threadIdx.x & 63) == 0) atomic_max_nonneg(A.s_max, wmax);
     }
 }
@@ -152,7 +157,8 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
 using namespace coat;
 
 template <int OP> static int launch_ew(const EwArgs& A, int kind_in, int kind_out, hipStream_t st) {
-    const int64_t blocks = (A.nchunk + 255) / 256;
+    int64_t blocks = (A.nchunk + 255) / 256;
+    if (blocks > 8192) blocks = 8192;  // 32 blocks per CU; the kernel strides over the rest
 #define EW_LAUNCH(KI, KO)                                                                                   \
     hipLaunchKernelGGL((k_elementwise<OP, KI, KO>), dim3((unsigned)blocks), dim3(256), 0, st, A); \
     return coat_launch_status();

@@ -66,7 +66,9 @@ __global__ __launch_bounds__(256) void k_quantize_pg(const void* __restrict__ x,
     constexpr int VEC = VecOf<XDT>::kVec;
     const int LPG = (QB ? QB : qb_rt) / VEC;  // lanes per group (QB == 0: group size given at run time)
     enable_fp8_saturation();
-    const int64_t base = ((int64_t)blockIdx.x * UNROLL) * 256 + threadIdx.x;
+    float wmax = 0.0f;
+    for (int64_t blk = blockIdx.x; blk * (UNROLL * 256) < nvec; blk += gridDim.x) {
+    const int64_t base = (blk * UNROLL) * 256 + threadIdx.x;
     float v[UNROLL][VEC];
     bool ok[UNROLL];
 #pragma unroll
@@ -79,7 +81,6 @@ __global__ __launch_bounds__(256) void k_quantize_pg(const void* __restrict__ x,
             for (int k = 0; k < VEC; k++) v[u][k] = 0.0f;
         }
     }
-    float wmax = 0.0f;
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
         int64_t i = base + (int64_t)u * 256;
@@ -94,6 +95,7 @@ __global__ __launch_bounds__(256) void k_quantize_pg(const void* __restrict__ x,
         }
         if (WRITE_S && ok[u] && (threadIdx.x % LPG) == 0) store_from_f32<SDT>(s_out, i / LPG, s);
     }
+    }
     if (WITH_MAX) {
         wmax = cluster_max<64>(wmax);
         if ((threadIdx.x & 63) == 0) atomic_max_nonneg(s_max, wmax);
@@ -106,15 +108,17 @@ template <int XDT, int UNROLL>
 __global__ __launch_bounds__(256) void k_absmax(const void* __restrict__ x, float* __restrict__ amax, int64_t nvec,
                                                  int64_t numel) {
     constexpr int VEC = VecOf<XDT>::kVec;
-    const int64_t base = ((int64_t)blockIdx.x * UNROLL) * 256 + threadIdx.x;
     float m = 0.0f;
+    for (int64_t blk = blockIdx.x; blk * (UNROLL * 256) < nvec; blk += gridDim.x) {
+        const int64_t base = (blk * UNROLL) * 256 + threadIdx.x;
 #pragma unroll
-    for (int u = 0; u < UNROLL; u++) {
-        int64_t i = base + (int64_t)u * 256;
-        if (i < nvec) {
-            float v[VEC];
-            load_vec<XDT>(x, i * VEC, v);
-            m = fmaxf(m, vec_amax<VEC>(v));
+        for (int u = 0; u < UNROLL; u++) {
+            int64_t i = base + (int64_t)u * 256;
+            if (i < nvec) {
+                float v[VEC];
+                load_vec<XDT>(x, i * VEC, v);
+                m = fmaxf(m, vec_amax<VEC>(v));
+            }
         }
     }
     // ragged tail (numel % VEC elements), handled by the first threads of block 0
@@ -391,9 +395,11 @@ static int launch_quantize_pg(const void* x, void* q, void* s, float* s_max, int
     // small problems: one vector per lane to spread over the chip; large ones: 4 independent loads per lane
     if (nvec >= (int64_t)256 * 4 * 2048) {
         int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
+        if (WMAX && blocks > 4096) blocks = 4096;  // fewer, longer blocks: one atomic per wave
         hipLaunchKernelGGL((k_quantize_pg<XDT, SDT, KIND, QB, WQ, WS, WMAX, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, q, s, s_max, nvec, qb);
     } else {
         int64_t blocks = (nvec + 256 * 2 - 1) / (256 * 2);
+        if (WMAX && blocks > 4096) blocks = 4096;
         hipLaunchKernelGGL((k_quantize_pg<XDT, SDT, KIND, QB, WQ, WS, WMAX, 2>), dim3((unsigned)blocks), dim3(256), 0, st, x, q, s, s_max, nvec, qb);
     }
     return coat_launch_status();
@@ -439,6 +445,7 @@ extern "C" int coat_absmax(const void* x, int x_dtype, float* amax, int64_t nume
         int64_t nvec = numel / VEC;
         int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
         if (blocks == 0) blocks = 1;
+        if (blocks > 4096) blocks = 4096;
         hipLaunchKernelGGL((k_absmax<XDT, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, amax, nvec, numel);
         return coat_launch_status();
     });
