@@ -168,4 +168,12 @@ __device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
     if (!(v <= cur)) atomicMax((unsigned int*)addr, f2u(v));
 }
 
+// Block-wide (256 threads) version: one lazy atomic per block.  `smem` holds 4 floats; every thread must call.
+__device__ __forceinline__ void block_atomic_max_nonneg(float* addr, float v, float* smem) {
+    v = cluster_max<64>(v);
+    if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) atomic_max_nonneg(addr, fmaxf(fmaxf(smem[0], smem[1]), fmaxf(smem[2], smem[3])));
+}
+
 }  // namespace coat

@@ -80,6 +80,7 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
     constexpr bool kHasG = (OP == kSiluBwd || OP == kMulBwd || OP == kGeluBwd);
     constexpr bool kQuantPg = (OP == kSiluFwd || OP == kAddFwd);         // emit per-group FP8 + scales
     constexpr bool kWriteY = !(OP == kSiluFwd);                          // emit the bf16 value
+    __shared__ float smem_max[4];
     enable_fp8_saturation();
     const int lpg = A.qb >> 4;  // lanes per group
     float tensor_max = 0.0f;
@@ -146,10 +147,7 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
     if (A.s_out && ok && (threadIdx.x % lpg) == 0) ((uint16_t*)A.s_out)[(c * 16) / A.qb] = (uint16_t)f2bf16(s);
     if (A.s_max) tensor_max = fmaxf(tensor_max, ok ? s : 0.0f);
     }
-    if (A.s_max) {
-        const float wmax = cluster_max<64>(tensor_max);
-        if ((threadIdx.x & 63) == 0) atomic_max_nonneg(A.s_max, wmax);
-    }
+    if (A.s_max) block_atomic_max_nonneg(A.s_max, tensor_max, smem_max);
 }
 
 }  // namespace coat
@@ -158,7 +156,7 @@ using namespace coat;
 
 template <int OP> static int launch_ew(const EwArgs& A, int kind_in, int kind_out, hipStream_t st) {
     int64_t blocks = (A.nchunk + 255) / 256;
-    if (blocks > 8192) blocks = 8192;  // 32 blocks per CU; the kernel strides over the rest
+    if (blocks > 2048) blocks = 2048;  // 8 blocks per CU; the kernel strides over the rest
 #define EW_LAUNCH(KI, KO)                                                                                   \
     hipLaunchKernelGGL((k_elementwise<OP, KI, KO>), dim3((unsigned)blocks), dim3(256), 0, st, A); \
     return coat_launch_status();

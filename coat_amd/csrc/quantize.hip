@@ -65,6 +65,7 @@ __global__ __launch_bounds__(256) void k_quantize_pg(const void* __restrict__ x,
                                                       int64_t nvec, int qb_rt) {
     constexpr int VEC = VecOf<XDT>::kVec;
     const int LPG = (QB ? QB : qb_rt) / VEC;  // lanes per group (QB == 0: group size given at run time)
+    __shared__ float smem_max[4];
     enable_fp8_saturation();
     float wmax = 0.0f;
     for (int64_t blk = blockIdx.x; blk * (UNROLL * 256) < nvec; blk += gridDim.x) {
@@ -96,10 +97,7 @@ __global__ __launch_bounds__(256) void k_quantize_pg(const void* __restrict__ x,
         if (WRITE_S && ok[u] && (threadIdx.x % LPG) == 0) store_from_f32<SDT>(s_out, i / LPG, s);
     }
     }
-    if (WITH_MAX) {
-        wmax = cluster_max<64>(wmax);
-        if ((threadIdx.x & 63) == 0) atomic_max_nonneg(s_max, wmax);
-    }
+    if (WITH_MAX) block_atomic_max_nonneg(s_max, wmax, smem_max);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -108,6 +106,7 @@ template <int XDT, int UNROLL>
 __global__ __launch_bounds__(256) void k_absmax(const void* __restrict__ x, float* __restrict__ amax, int64_t nvec,
                                                  int64_t numel) {
     constexpr int VEC = VecOf<XDT>::kVec;
+    __shared__ float smem_max[4];
     float m = 0.0f;
     for (int64_t blk = blockIdx.x; blk * (UNROLL * 256) < nvec; blk += gridDim.x) {
         const int64_t base = (blk * UNROLL) * 256 + threadIdx.x;
@@ -123,8 +122,7 @@ __global__ __launch_bounds__(256) void k_absmax(const void* __restrict__ x, floa
     }
     // ragged tail (numel % VEC elements), handled by the first threads of block 0
     if (blockIdx.x == 0 && threadIdx.x < numel - nvec * VEC) m = fmaxf(m, fabsf(load_as_f32<XDT>(x, nvec * VEC + threadIdx.x)));
-    m = cluster_max<64>(m);
-    if ((threadIdx.x & 63) == 0) atomic_max_nonneg(amax, m);
+    block_atomic_max_nonneg(amax, m, smem_max);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -395,11 +393,11 @@ static int launch_quantize_pg(const void* x, void* q, void* s, float* s_max, int
     // small problems: one vector per lane to spread over the chip; large ones: 4 independent loads per lane
     if (nvec >= (int64_t)256 * 4 * 2048) {
         int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
-        if (WMAX && blocks > 4096) blocks = 4096;  // fewer, longer blocks: one atomic per wave
+        if (WMAX && blocks > 2048) blocks = 2048;  // fewer, longer blocks: one atomic per block
         hipLaunchKernelGGL((k_quantize_pg<XDT, SDT, KIND, QB, WQ, WS, WMAX, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, q, s, s_max, nvec, qb);
     } else {
         int64_t blocks = (nvec + 256 * 2 - 1) / (256 * 2);
-        if (WMAX && blocks > 4096) blocks = 4096;
+        if (WMAX && blocks > 2048) blocks = 2048;
         hipLaunchKernelGGL((k_quantize_pg<XDT, SDT, KIND, QB, WQ, WS, WMAX, 2>), dim3((unsigned)blocks), dim3(256), 0, st, x, q, s, s_max, nvec, qb);
     }
     return coat_launch_status();
@@ -445,7 +443,7 @@ extern "C" int coat_absmax(const void* x, int x_dtype, float* amax, int64_t nume
         int64_t nvec = numel / VEC;
         int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
         if (blocks == 0) blocks = 1;
-        if (blocks > 4096) blocks = 4096;
+        if (blocks > 2048) blocks = 2048;
         hipLaunchKernelGGL((k_absmax<XDT, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, amax, nvec, numel);
         return coat_launch_status();
     });
