@@ -15,8 +15,6 @@
 // is two quads in each of the lanes l and l^32.
 // Block ids are remapped so that the 8 XCDs (round-robin block dispatch) each work on a contiguous band of
 // tiles, ordered in panels of 8 tile-rows, which keeps A / B slabs hot in that XCD's L2.
-#include <stdlib.h>
-
 #include "coat_device.h"
 #include "coat_host.h"
 
@@ -44,7 +42,6 @@ struct GemmArgs {
     int s_dt, bias_dt;
     int M, N, K;
     int tiles_m, tiles_n;
-    int remap;  // 1: XCD-aware block -> tile mapping
 };
 
 // A slab row is 64 bytes = four 16-byte chunks.  A 16-byte-per-lane LDS read is served 16 lanes (256 bytes, 64
@@ -55,11 +52,29 @@ struct GemmArgs {
 __device__ __forceinline__ int swz_chunk(int row, int chunk) { return chunk ^ ((row >> 2) & 3); }
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+// buffer_load_dwordx4 ... lds: every lane fetches 16 bytes at byte offset `voff` of the buffer and the wave's 1 KiB
+// lands in LDS at lds_addr + 16 * lane without passing through registers; offsets beyond the buffer's extent fill
+// zeros.  Issued as inline assembly so that the compiler does not order later LDS reads behind it with a full
+// vmcnt(0) wait (it cannot tell which ring stage a read touches); completion is tracked by hand with s_waitcnt vmcnt.
+__device__ __forceinline__ void lds_dma16(v4i rsrc, uint32_t lds_addr, int voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
+    const uint64_t a = (uint64_t)p;
+    return (v4i){(int)(uint32_t)a, (int)(uint32_t)(a >> 32) & 0xFFFF, (int)bytes, 0x00020000};
+}
 
 // s_waitcnt vmcnt(N) only (expcnt / lgkmcnt left at their maxima), gfx9 encoding.
 #define COAT_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (0x7 << 4) | (0xF << 8) | ((((N) >> 4) & 0x3) << 14))
 
 // NWN = waves along N (2: four waves of 128 x 128, one per SIMD; 4: eight waves of 128 x 64, two per SIMD).
+// Persistent: the grid is one block per CU; a block walks its share of the output tiles and the LDS ring runs straight
+// across tile boundaries, so the first slabs of the next tile are already in flight while the epilogue stores drain.
 template <int FMT_A, int FMT_B, int EPI, int NWN>
 __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
     constexpr int NW = 2 * NWN;               // waves per block
@@ -72,46 +87,69 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / NWN, wn = wave % NWN;
 
-    // ---- XCD-aware tile mapping
+    // ---- XCD-aware tile schedule.  Blocks are dispatched round-robin over the 8 XCDs, so block b runs on XCD b % 8.
+    // XCD x owns the contiguous band [x * per_xcd, (x + 1) * per_xcd) of the tile order below, and its blocks take the
+    // band's tiles in rounds of gridDim.x / 8: at any time one XCD works on neighbouring tiles, whose A / B slabs are
+    // shared through that XCD's L2.  The tile order runs down panels of GROUP_M tile-rows.
     const int ntiles = G.tiles_m * G.tiles_n;
     const int per_xcd = (ntiles + 7) / 8;
-    int tile = G.remap ? (blockIdx.x % 8) * per_xcd + blockIdx.x / 8 : blockIdx.x;
-    if (tile >= ntiles) return;
+    const int xcd = blockIdx.x & 7, my = blockIdx.x >> 3, stride = gridDim.x >> 3;
+    const int band = min(max(ntiles - xcd * per_xcd, 0), per_xcd);
+    const int my_ntiles = my < band ? (band - my + stride - 1) / stride : 0;
+    if (my_ntiles == 0) return;
     constexpr int GROUP_M = 8;
-    const int width = GROUP_M * G.tiles_n;
-    const int group = tile / width;
-    const int gsize = min(G.tiles_m - group * GROUP_M, GROUP_M);
-    const int tm = group * GROUP_M + (tile % width) % gsize;
-    const int tn = (tile % width) / gsize;
-    const int m0 = tm * BM, n0 = tn * BN;
+    auto tile_origin = [&](int it, int& m0, int& n0) {
+        const int tile = xcd * per_xcd + my + it * stride;
+        const int width = GROUP_M * G.tiles_n;
+        const int group = tile / width;
+        const int gsize = min(G.tiles_m - group * GROUP_M, GROUP_M);
+        m0 = (group * GROUP_M + (tile % width) % gsize) * BM;
+        n0 = ((tile % width) / gsize) * BN;
+    };
 
     // ---- global -> LDS without passing through registers: buffer_load_dwordx4 ... lds.
     // One wave instruction fills 1 KiB of LDS contiguously (lane i at +16 i) = 16 slab rows; the lane picks the global
     // chunk that belongs at its position under the swizzle.  Out-of-range rows / K-tail chunks use an offset beyond
     // num_records, for which the buffer load returns zeros.
-    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)G.A, 0, G.M * G.K, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)G.B, 0, G.N * G.K, 0x00020000);
+    const v4i rsrcA = make_rsrc(G.A, (uint32_t)(G.M * G.K));
+    const v4i rsrcB = make_rsrc(G.B, (uint32_t)(G.N * G.K));
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+    // K is walked in an even number of slabs (the register ping-pong below alternates per slab); a padding slab is all
+    // zero fills.
+    const int nslab = (((G.K + BK - 1) / BK) + 1) & ~1;
+    // load cursor: tile iteration lt, slab lkt, ring stage st_load; runs PREFETCH slabs ahead of the multiply cursor
     int offA[LI], offB[LI], kc[LI];
+    int lt = 0, lkt = 0, st_load = 0;
+    auto set_load_tile = [&](int it) {
+        int m0 = 0, n0 = 0;
+        const bool live = it < my_ntiles;
+        if (live) tile_origin(it, m0, n0);
 #pragma unroll
-    for (int i = 0; i < LI; i++) {
-        const int row = wave * LROWS + i * 16 + (lane >> 2);
-        const int c = swz_chunk(row, lane & 3);
-        kc[i] = c * 16;
-        offA[i] = (m0 + row < G.M) ? (m0 + row) * G.K + c * 16 : -1;
-        offB[i] = (n0 + row < G.N) ? (n0 + row) * G.K + c * 16 : -1;
-    }
-    auto issue_slab = [&](int kt) {
-        const int stage = kt % NSTAGE;
-        const int k0 = kt * BK;
-        uint8_t* sA = lds + stage * kStageBytes + wave * LROWS * BK;
-        uint8_t* sB = sA + BM * BK;
+        for (int i = 0; i < LI; i++) {
+            const int row = wave * LROWS + i * 16 + (lane >> 2);
+            const int c = swz_chunk(row, lane & 3);
+            kc[i] = c * 16;
+            offA[i] = (live && m0 + row < G.M) ? (m0 + row) * G.K + c * 16 : -1;
+            offB[i] = (live && n0 + row < G.N) ? (n0 + row) * G.K + c * 16 : -1;
+        }
+    };
+    set_load_tile(0);
+    auto issue_next = [&]() {
+        const int k0 = lkt * BK;
+        const uint32_t sA = lds_base + st_load * kStageBytes + wave * LROWS * BK;
+        const uint32_t sB = sA + BM * BK;
 #pragma unroll
         for (int i = 0; i < LI; i++) {
             const bool kin = k0 + kc[i] < G.K;
             const int oa = (kin && offA[i] >= 0) ? offA[i] + k0 : 0x7FFFFFFF;
             const int ob = (kin && offB[i] >= 0) ? offB[i] + k0 : 0x7FFFFFFF;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_ptr_t)(sA + i * 16 * BK), 16, oa, 0, 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(sB + i * 16 * BK), 16, ob, 0, 0, 0);
+            lds_dma16(rsrcA, sA + i * 16 * BK, oa);
+            lds_dma16(rsrcB, sB + i * 16 * BK, ob);
+        }
+        st_load = st_load + 1 == NSTAGE ? 0 : st_load + 1;
+        if (++lkt == nslab) {
+            lkt = 0;
+            set_load_tile(++lt);  // past the last tile: zero fills, which keep the outstanding-load counts uniform
         }
     };
     // fragment addresses (bytes inside a stage) for this lane: row = tile base + lane%32, 32-byte half = lane/32
@@ -130,18 +168,10 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
             fb_off[t][h] = BM * BK + rowb * BK + (swz_chunk(rowb, c) << 4);
         }
     }
-
-    v16f acc[TJ][4];  // [n-tile j][m-tile i]
-#pragma unroll
-    for (int j = 0; j < TJ; j++)
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
-
-    const int nslab = (G.K + BK - 1) / BK;
-    auto load_frags = [&](int kt, v8i* fa, v8i* fb) {
-        const uint8_t* st = lds + (kt % NSTAGE) * kStageBytes;
+    int st_frag = 0;  // ring stage of the next slab whose fragments are to be read
+    auto load_frags = [&](v8i* fa, v8i* fb) {
+        const uint8_t* st = lds + st_frag * kStageBytes;
+        st_frag = st_frag + 1 == NSTAGE ? 0 : st_frag + 1;
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const uint4 a0 = *(const uint4*)(st + fa_off[t][0]), a1 = *(const uint4*)(st + fa_off[t][1]);
@@ -153,39 +183,53 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
             fb[t] = (v8i){(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
         }
     };
-    // prologue: PREFETCH slabs in flight (slabs past the end are all-zero fills, which keeps the counts uniform)
+
+    v16f acc[TJ][4];  // [n-tile j][m-tile i]
+    // prologue: PREFETCH slabs in flight
 #pragma unroll
-    for (int p = 0; p < PREFETCH; p++) issue_slab(p);
+    for (int p = 0; p < PREFETCH; p++) issue_next();
     COAT_WAIT_VMCNT(LOADS * (PREFETCH - 1));  // slab 0 has landed (this wave's part)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     v8i fa0[4], fb0[TJ], fa1[4], fb1[TJ];
-    load_frags(0, fa0, fb0);
-    // One step: wait for this wave's part of slab kt+1, barrier (slab kt+1 is now complete and visible, and every wave
-    // has issued the MFMAs of slab kt-1, i.e. finished reading that stage), refill that stage with slab kt+PREFETCH,
-    // fetch the fragments of slab kt+1 and issue the MFMAs of slab kt while they arrive.
-    auto step = [&](int kt, v8i* fc_a, v8i* fc_b, v8i* fn_a, v8i* fn_b) {
+    load_frags(fa0, fb0);
+    // One step on slab g of this block's slab sequence: wait for this wave's part of slab g+1, barrier (slab g+1 is now
+    // complete and visible, and every wave has issued the MFMAs of slab g-1, i.e. finished reading that stage), refill
+    // that stage with slab g+PREFETCH, fetch the fragments of slab g+1 and issue the MFMAs of slab g while they arrive.
+    // Loads return in order, so "at most LOADS * (PREFETCH - 2) vector-memory operations outstanding" implies slab g+1
+    // has landed also when epilogue stores of the previous tile are still in that count (the wait is then merely
+    // conservative).
+    auto step = [&](v8i* fc_a, v8i* fc_b, v8i* fn_a, v8i* fn_b) {
         COAT_WAIT_VMCNT(LOADS * (PREFETCH - 2));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        issue_slab(kt + PREFETCH);
-        load_frags(kt + 1, fn_a, fn_b);
+        issue_next();
+        load_frags(fn_a, fn_b);
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
                 acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fc_b[j], fc_a[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
     };
-    for (int kt = 0; kt < nslab; kt += 2) {
-        step(kt, fa0, fb0, fa1, fb1);
-        if (kt + 1 < nslab) step(kt + 1, fa1, fb1, fa0, fb0);
-    }
-    COAT_WAIT_VMCNT(0);  // drain the zero-fill slabs before the block may exit
-
-    // ---- epilogue
     const float scale = load_rt_f32(G.sa, 0, G.s_dt) * load_rt_f32(G.sb, 0, G.s_dt);
     if (EPI != kEpiBf16) enable_fp8_saturation();
     const int half = lane >> 5;
+
+    for (int it = 0; it < my_ntiles; it++) {
+#pragma unroll
+    for (int j = 0; j < TJ; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
+    for (int kt = 0; kt < nslab; kt += 2) {
+        step(fa0, fb0, fa1, fb1);
+        step(fa1, fb1, fa0, fb0);
+    }
+    int m0, n0;
+    tile_origin(it, m0, n0);
+
+    // ---- epilogue (stores are not waited for: they drain while the next tile is multiplied)
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int m = m0 + wm * 128 + i * 32 + (lane & 31);
@@ -244,6 +288,8 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
             }
         }
     }
+    }  // tiles
+    COAT_WAIT_VMCNT(0);  // drain the trailing zero-fill slabs before the block may exit
 }
 
 }  // namespace coat
@@ -274,9 +320,15 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     G.M = (int)M; G.N = (int)N; G.K = (int)K;
     G.tiles_m = (int)((M + BM - 1) / BM);
     G.tiles_n = (int)((N + BN - 1) / BN);
-    G.remap = getenv("COAT_GEMM_NOREMAP") ? 0 : 1;
     const int ntiles = G.tiles_m * G.tiles_n;
-    const int grid = ((ntiles + 7) / 8) * 8;
+    static int n_cu = 0;  // persistent grid: one block per CU (the block's LDS ring takes a whole CU's LDS)
+    if (n_cu == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 8)
+            return COAT_EINVAL;
+        n_cu = v & ~7;
+    }
+    const int grid = min(((ntiles + 7) / 8) * 8, n_cu);
     const size_t lds_bytes = kLdsBytes;
     hipStream_t st = (hipStream_t)stream;
 #define GEMM_LAUNCH(FA, FB, EP)                                                                                    \
