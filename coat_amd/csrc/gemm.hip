@@ -23,11 +23,11 @@ namespace coat {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int NSTAGE = 5;                      // LDS ring of K-slabs (5 x 32 KiB = the whole 160 KiB LDS)
-constexpr int PREFETCH = 4;                    // slabs in flight ahead of the one being multiplied
-constexpr int kStageBytes = (BM + BN) * BK;    // 32 KiB
-constexpr int kLdsBytes = NSTAGE * kStageBytes;
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int NUNIT = 5;                       // LDS ring of slabs (5 x 32 KiB = the whole 160 KiB LDS)
+constexpr int kUnitBytes = BM * BK;            // one matrix's 256 rows x 128 bytes of K = 32 KiB
+constexpr int kLdsBytes = NUNIT * kUnitBytes;
+static_assert(BM == BN, "A and B slabs share one unit size");
 
 enum Epilogue { kEpiBf16 = 0, kEpiQuantE4M3 = 1, kEpiQuantE5M2 = 2 };
 
@@ -44,12 +44,12 @@ struct GemmArgs {
     int tiles_m, tiles_n;
 };
 
-// A slab row is 64 bytes = four 16-byte chunks.  A 16-byte-per-lane LDS read is served 16 lanes (256 bytes, 64
-// banks) per cycle, so 16 consecutive rows reading the same chunk must land in 16 different 16-byte slots modulo 256:
-// row & 3 already selects the 64-byte quarter, and placing chunk c of row r at position c ^ ((r >> 2) & 3) makes the
-// four rows that share a quarter use four different slots.  (SQ_LDS_BANK_CONFLICT: 0 with this layout, 50 % of the
-// LDS cycles with c ^ ((r >> 1) & 3), 75 % with c ^ (r & 3).)
-__device__ __forceinline__ int swz_chunk(int row, int chunk) { return chunk ^ ((row >> 2) & 3); }
+// A slab row is 128 bytes = eight 16-byte chunks (one full cache line per row and load instruction: fetching rows as
+// two 64-byte halves was measured at 0.6 x the LDS-DMA throughput).  A 16-byte-per-lane LDS read is served 16 lanes
+// (256 bytes, 64 banks) per cycle, so 16 consecutive rows reading the same chunk must land in 16 different 16-byte
+// slots modulo 256: row & 1 selects the 128-byte half, and placing chunk c of row r at position c ^ ((r >> 1) & 7)
+// spreads the eight row pairs over the eight slots of a half.
+__device__ __forceinline__ int swz_chunk(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -72,16 +72,15 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 // s_waitcnt vmcnt(N) only (expcnt / lgkmcnt left at their maxima), gfx9 encoding.
 #define COAT_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (0x7 << 4) | (0xF << 8) | ((((N) >> 4) & 0x3) << 14))
 
-// NWN = waves along N (2: four waves of 128 x 128, one per SIMD; 4: eight waves of 128 x 64, two per SIMD).
+// Eight waves (2 along M x 4 along N), each 128 x 64 of the 256 x 256 tile as 4 x 2 tiles of
+// v_mfma_f32_32x32x64_f8f6f4, two waves per SIMD.
 // Persistent: the grid is one block per CU; a block walks its share of the output tiles and the LDS ring runs straight
 // across tile boundaries, so the first slabs of the next tile are already in flight while the epilogue stores drain.
-template <int FMT_A, int FMT_B, int EPI, int NWN>
-__global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
-    constexpr int NW = 2 * NWN;               // waves per block
-    constexpr int TJ = BN / (NWN * 32);       // n-tiles per wave (4 or 2); m-tiles per wave is always 4
-    constexpr int LROWS = BM / NW;            // slab rows each wave fetches per matrix (64 or 32)
-    constexpr int LI = LROWS / 16;            // load instructions per wave per matrix per slab
-    constexpr int LOADS = 2 * LI;             // buffer loads per wave per slab
+template <int FMT_A, int FMT_B, int EPI>
+__global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
+    constexpr int NWN = 4, NW = 8;
+    constexpr int TJ = 2;                     // n-tiles per wave; m-tiles per wave is 4
+    constexpr int LI = BM / (NW * 8);         // load instructions per wave per slab (each covers 8 rows) = 4
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -107,109 +106,106 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
         n0 = ((tile % width) / gsize) * BN;
     };
 
-    // ---- global -> LDS without passing through registers: buffer_load_dwordx4 ... lds.
-    // One wave instruction fills 1 KiB of LDS contiguously (lane i at +16 i) = 16 slab rows; the lane picks the global
-    // chunk that belongs at its position under the swizzle.  Out-of-range rows / K-tail chunks use an offset beyond
-    // num_records, for which the buffer load returns zeros.
+    // ---- global -> LDS without passing through registers.  The ring holds 5 slabs; slab u of a tile is the A slab
+    // (u even) or the B slab (u odd) of K-step u / 2.  One wave instruction fills 1 KiB of LDS contiguously (lane i at
+    // +16 i) = 8 slab rows; the lane picks the global chunk that belongs at its position under the swizzle.
+    // Out-of-range rows / K-tail chunks use an offset beyond the buffer's extent, which fills zeros.
     const v4i rsrcA = make_rsrc(G.A, (uint32_t)(G.M * G.K));
     const v4i rsrcB = make_rsrc(G.B, (uint32_t)(G.N * G.K));
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
-    // K is walked in an even number of slabs (the register ping-pong below alternates per slab); a padding slab is all
-    // zero fills.
-    const int nslab = (((G.K + BK - 1) / BK) + 1) & ~1;
-    // load cursor: tile iteration lt, slab lkt, ring stage st_load; runs PREFETCH slabs ahead of the multiply cursor
+    const int nstep = (G.K + BK - 1) / BK;
+    // load cursor: tile iteration lt, K-step lstep of that tile, ring slot sl_load; slabs go A, B, A, B, ...
     int offA[LI], offB[LI], kc[LI];
-    int lt = 0, lkt = 0, st_load = 0;
+    const int lrow = wave * (LI * 8) + (lane >> 3);  // + 8 i
+#pragma unroll
+    for (int i = 0; i < LI; i++) kc[i] = swz_chunk(lrow + 8 * i, lane & 7) * 16;
+    int lt = 0, lstep = 0, sl_load = 0;
     auto set_load_tile = [&](int it) {
         int m0 = 0, n0 = 0;
         const bool live = it < my_ntiles;
         if (live) tile_origin(it, m0, n0);
 #pragma unroll
         for (int i = 0; i < LI; i++) {
-            const int row = wave * LROWS + i * 16 + (lane >> 2);
-            const int c = swz_chunk(row, lane & 3);
-            kc[i] = c * 16;
-            offA[i] = (live && m0 + row < G.M) ? (m0 + row) * G.K + c * 16 : -1;
-            offB[i] = (live && n0 + row < G.N) ? (n0 + row) * G.K + c * 16 : -1;
+            const int row = lrow + 8 * i;
+            offA[i] = (live && m0 + row < G.M) ? (m0 + row) * G.K + kc[i] : -1;
+            offB[i] = (live && n0 + row < G.N) ? (n0 + row) * G.K + kc[i] : -1;
         }
     };
     set_load_tile(0);
-    auto issue_next = [&]() {
-        const int k0 = lkt * BK;
-        const uint32_t sA = lds_base + st_load * kStageBytes + wave * LROWS * BK;
-        const uint32_t sB = sA + BM * BK;
+    auto issue_A = [&]() {
+        const int k0 = lstep * BK;
+        const uint32_t dst = lds_base + sl_load * kUnitBytes + wave * (LI * 8 * BK);
 #pragma unroll
-        for (int i = 0; i < LI; i++) {
-            const bool kin = k0 + kc[i] < G.K;
-            const int oa = (kin && offA[i] >= 0) ? offA[i] + k0 : 0x7FFFFFFF;
-            const int ob = (kin && offB[i] >= 0) ? offB[i] + k0 : 0x7FFFFFFF;
-            lds_dma16(rsrcA, sA + i * 16 * BK, oa);
-            lds_dma16(rsrcB, sB + i * 16 * BK, ob);
-        }
-        st_load = st_load + 1 == NSTAGE ? 0 : st_load + 1;
-        if (++lkt == nslab) {
-            lkt = 0;
+        for (int i = 0; i < LI; i++) lds_dma16(rsrcA, dst + i * 8 * BK, (k0 + kc[i] < G.K && offA[i] >= 0) ? offA[i] + k0 : 0x7FFFFFFF);
+        sl_load = sl_load + 1 == NUNIT ? 0 : sl_load + 1;
+    };
+    auto issue_B = [&]() {
+        const int k0 = lstep * BK;
+        const uint32_t dst = lds_base + sl_load * kUnitBytes + wave * (LI * 8 * BK);
+#pragma unroll
+        for (int i = 0; i < LI; i++) lds_dma16(rsrcB, dst + i * 8 * BK, (k0 + kc[i] < G.K && offB[i] >= 0) ? offB[i] + k0 : 0x7FFFFFFF);
+        sl_load = sl_load + 1 == NUNIT ? 0 : sl_load + 1;
+        if (++lstep == nstep) {
+            lstep = 0;
             set_load_tile(++lt);  // past the last tile: zero fills, which keep the outstanding-load counts uniform
         }
     };
-    // fragment addresses (bytes inside a stage) for this lane: row = tile base + lane%32, 32-byte half = lane/32
-    int fa_off[4][2], fb_off[TJ][2];
+    // fragment addresses (bytes inside a slab) for this lane and K-substep 0: row = tile base + lane % 32, 16-byte
+    // chunks 2 * (lane / 32) + h; the chunks of substep 1 are those + 4, i.e. the address with bit 6 flipped.
+    int fa_off[2], fb_off[2];  // + t * 32 * BK per 32-row tile
 #pragma unroll
     for (int h = 0; h < 2; h++) {
         const int c = 2 * (lane >> 5) + h;
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const int rowa = wm * 128 + t * 32 + (lane & 31);
-            fa_off[t][h] = rowa * BK + (swz_chunk(rowa, c) << 4);
-        }
-#pragma unroll
-        for (int t = 0; t < TJ; t++) {
-            const int rowb = wn * (TJ * 32) + t * 32 + (lane & 31);
-            fb_off[t][h] = BM * BK + rowb * BK + (swz_chunk(rowb, c) << 4);
-        }
+        const int rowa = wm * 128 + (lane & 31), rowb = wn * (TJ * 32) + (lane & 31);
+        fa_off[h] = rowa * BK + (swz_chunk(rowa, c) << 4);
+        fb_off[h] = rowb * BK + (swz_chunk(rowb, c) << 4);
     }
-    int st_frag = 0;  // ring stage of the next slab whose fragments are to be read
-    auto load_frags = [&](v8i* fa, v8i* fb) {
-        const uint8_t* st = lds + st_frag * kStageBytes;
-        st_frag = st_frag + 1 == NSTAGE ? 0 : st_frag + 1;
+    int sl_frag = 0;  // ring slot of the A slab of the next K-step to be multiplied (its B slab is in the next slot)
+    auto load_frags = [&](int sub, v8i* fa, v8i* fb) {
+        const uint8_t* sa = lds + sl_frag * kUnitBytes;
+        const uint8_t* sb = lds + (sl_frag + 1 == NUNIT ? 0 : sl_frag + 1) * kUnitBytes;
+        const int x = sub * 64;
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const uint4 a0 = *(const uint4*)(st + fa_off[t][0]), a1 = *(const uint4*)(st + fa_off[t][1]);
+            const uint4 a0 = *(const uint4*)(sa + ((fa_off[0] ^ x) + t * 32 * BK)), a1 = *(const uint4*)(sa + ((fa_off[1] ^ x) + t * 32 * BK));
             fa[t] = (v8i){(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
         }
 #pragma unroll
         for (int t = 0; t < TJ; t++) {
-            const uint4 b0 = *(const uint4*)(st + fb_off[t][0]), b1 = *(const uint4*)(st + fb_off[t][1]);
+            const uint4 b0 = *(const uint4*)(sb + ((fb_off[0] ^ x) + t * 32 * BK)), b1 = *(const uint4*)(sb + ((fb_off[1] ^ x) + t * 32 * BK));
             fb[t] = (v8i){(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
         }
     };
 
     v16f acc[TJ][4];  // [n-tile j][m-tile i]
-    // prologue: PREFETCH slabs in flight
-#pragma unroll
-    for (int p = 0; p < PREFETCH; p++) issue_next();
-    COAT_WAIT_VMCNT(LOADS * (PREFETCH - 1));  // slab 0 has landed (this wave's part)
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    v8i fa0[4], fb0[TJ], fa1[4], fb1[TJ];
-    load_frags(fa0, fb0);
-    // One step on slab g of this block's slab sequence: wait for this wave's part of slab g+1, barrier (slab g+1 is now
-    // complete and visible, and every wave has issued the MFMAs of slab g-1, i.e. finished reading that stage), refill
-    // that stage with slab g+PREFETCH, fetch the fragments of slab g+1 and issue the MFMAs of slab g while they arrive.
-    // Loads return in order, so "at most LOADS * (PREFETCH - 2) vector-memory operations outstanding" implies slab g+1
-    // has landed also when epilogue stores of the previous tile are still in that count (the wait is then merely
-    // conservative).
-    auto step = [&](v8i* fc_a, v8i* fc_b, v8i* fn_a, v8i* fn_b) {
-        COAT_WAIT_VMCNT(LOADS * (PREFETCH - 2));
+    // prologue: three slabs in flight (A0, B0, A1)
+    issue_A();
+    issue_B();
+    issue_A();
+    // One K-step of 128: wait until at most the newest slab is outstanding (loads return in order, so the two slabs of
+    // this step have landed also when epilogue stores of the previous tile are still in that count), barrier (they
+    // are now complete and visible from every wave, and every wave has issued the MFMAs of the previous step, i.e.
+    // finished reading its two slabs), refill those two slots, and multiply: 2 substeps x 8 MFMAs per wave.
+    auto step = [&]() {
+        COAT_WAIT_VMCNT(LI);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        issue_next();
-        load_frags(fn_a, fn_b);
+        v8i fa0[4], fb0[TJ], fa1[4], fb1[TJ];
+        load_frags(0, fa0, fb0);
+        issue_B();
+        issue_A();
+        load_frags(1, fa1, fb1);
+        sl_frag = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fc_b[j], fc_a[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
+                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
     };
     const float scale = load_rt_f32(G.sa, 0, G.s_dt) * load_rt_f32(G.sb, 0, G.s_dt);
     if (EPI != kEpiBf16) enable_fp8_saturation();
@@ -222,10 +218,7 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
-    for (int kt = 0; kt < nslab; kt += 2) {
-        step(fa0, fb0, fa1, fb1);
-        step(fa1, fb1, fa0, fb0);
-    }
+    for (int ks = 0; ks < nstep; ks++) step();
     int m0, n0;
     tile_origin(it, m0, n0);
 
@@ -296,10 +289,6 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
 
 using namespace coat;
 
-#ifndef COAT_GEMM_NWN
-#define COAT_GEMM_NWN 4
-#endif
-
 extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
                              const void* scale_a, const void* scale_b, int s_dtype, const void* bias, int bias_dtype,
                              int64_t M, int64_t N, int64_t K, int QB, void* stream) {
@@ -335,12 +324,12 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     {                                                                                                              \
         static bool attr_set = false;                                                                              \
         if (!attr_set) {                                                                                           \
-            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP, COAT_GEMM_NWN>,                 \
+            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP>,                 \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);        \
             if (e != hipSuccess) return (int)e;                                                                    \
             attr_set = true;                                                                                       \
         }                                                                                                          \
-        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, COAT_GEMM_NWN>), dim3(grid), dim3(128 * COAT_GEMM_NWN), lds_bytes, st, G); \
+        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP>), dim3(grid), dim3(512), lds_bytes, st, G); \
         return coat_launch_status();                                                                               \
     }
 #define GEMM_FMT(EP)                                                             \
