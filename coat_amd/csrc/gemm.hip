@@ -71,6 +71,8 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 
 // s_waitcnt vmcnt(N) only (expcnt / lgkmcnt left at their maxima), gfx9 encoding.
 #define COAT_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (0x7 << 4) | (0xF << 8) | ((((N) >> 4) & 0x3) << 14))
+// the same with lgkmcnt(0): all LDS reads issued so far have returned
+#define COAT_WAIT_VMCNT_LGKM0(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (0x7 << 4) | (0x0 << 8) | ((((N) >> 4) & 0x3) << 14))
 
 // Eight waves (2 along M x 4 along N), each 128 x 64 of the 256 x 256 tile as 4 x 2 tiles of
 // v_mfma_f32_32x32x64_f8f6f4, two waves per SIMD.
@@ -160,10 +162,10 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
         fa_off[h] = rowa * BK + (swz_chunk(rowa, c) << 4);
         fb_off[h] = rowb * BK + (swz_chunk(rowb, c) << 4);
     }
-    int sl_frag = 0;  // ring slot of the A slab of the next K-step to be multiplied (its B slab is in the next slot)
-    auto load_frags = [&](int sub, v8i* fa, v8i* fb) {
-        const uint8_t* sa = lds + sl_frag * kUnitBytes;
-        const uint8_t* sb = lds + (sl_frag + 1 == NUNIT ? 0 : sl_frag + 1) * kUnitBytes;
+    int sl_frag = 0;  // ring slot of the A slab of the K-step being multiplied (its B slab is in the next slot)
+    auto load_frags = [&](int slot_a, int sub, v8i* fa, v8i* fb) {
+        const uint8_t* sa = lds + slot_a * kUnitBytes;
+        const uint8_t* sb = lds + (slot_a + 1 == NUNIT ? 0 : slot_a + 1) * kUnitBytes;
         const int x = sub * 64;
 #pragma unroll
         for (int t = 0; t < 4; t++) {
@@ -178,34 +180,42 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     };
 
     v16f acc[TJ][4];  // [n-tile j][m-tile i]
-    // prologue: three slabs in flight (A0, B0, A1)
+    v8i fax[4], fbx[TJ], fay[4], fby[TJ];  // fragments of K-substep 0 (x) and 1 (y)
+    // prologue: fill the ring (A0 B0 A1 B1 A2), wait for the first step's two slabs, fetch its substep-0 fragments
     issue_A();
     issue_B();
     issue_A();
-    // One K-step of 128: wait until at most the newest slab is outstanding (loads return in order, so the two slabs of
-    // this step have landed also when epilogue stores of the previous tile are still in that count), barrier (they
-    // are now complete and visible from every wave, and every wave has issued the MFMAs of the previous step, i.e.
-    // finished reading its two slabs), refill those two slots, and multiply: 2 substeps x 8 MFMAs per wave.
+    issue_B();
+    issue_A();
+    COAT_WAIT_VMCNT(3 * LI);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    load_frags(sl_frag, 0, fax, fbx);
+    // One K-step of 128 = 2 substeps x 8 MFMAs per wave, with one barrier in the middle:
+    //   read the substep-1 fragments, multiply substep 0;
+    //   wait until those reads have returned and at most the newest slab is outstanding, barrier: every wave now holds
+    //   all it needs from this step's two slabs in registers, and the next step's slabs have landed and are visible
+    //   (loads return in order, so this holds also when epilogue stores of the previous tile are still in the count);
+    //   refill this step's two slots, read the next step's substep-0 fragments, multiply substep 1.
     auto step = [&]() {
-        COAT_WAIT_VMCNT(LI);
+        load_frags(sl_frag, 1, fay, fby);
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fbx[j], fax[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
+        COAT_WAIT_VMCNT_LGKM0(LI);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        v8i fa0[4], fb0[TJ], fa1[4], fb1[TJ];
-        load_frags(0, fa0, fb0);
         issue_B();
         issue_A();
-        load_frags(1, fa1, fb1);
         sl_frag = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
+        load_frags(sl_frag, 0, fax, fbx);
 #pragma unroll
         for (int j = 0; j < TJ; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
+                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fby[j], fay[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
     };
     const float scale = load_rt_f32(G.sa, 0, G.s_dt) * load_rt_f32(G.sb, 0, G.s_dt);
     if (EPI != kEpiBf16) enable_fp8_saturation();
