@@ -204,10 +204,22 @@ def cpu_baseline_adamw(torch):
             "sample": f"{reps} steps over the first {n} elements (4096 groups) of the tensor, oracle/adamw_ref.c, 1 thread"}
 
 
+def ramp_clocks(step, seconds, torch):
+    """Keep the GPU continuously busy with `step` for `seconds` (untimed) so that the timed region runs at the sustained clock."""
+    if seconds <= 0:
+        return
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+
+
 def bench_layer(args, dev, torch):
     step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1])
 
     def time_it(fn):
+        ramp_clocks(fn, args.ramp_seconds, torch)
         for _ in range(max(2, args.warmup // 2)):
             fn()
         torch.cuda.synchronize()
@@ -248,6 +260,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ramp-seconds", type=float, default=1.5,
+                    help="untimed continuous run of the step before the W warmup steps: an idle MI355X sits at ~100 MHz and "
+                         "takes several hundred ms of load to reach its sustained shader clock, so a few ms of warmup would "
+                         "time the kernel on a ramping clock (0 disables)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (known traffic, to scale rocprofv3 counters)")
     args = ap.parse_args()
@@ -283,6 +299,7 @@ def main():
         for _ in range(5):
             dst.copy_(src)  # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
+    ramp_clocks(step, args.ramp_seconds, torch)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

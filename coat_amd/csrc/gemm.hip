@@ -78,11 +78,11 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 // v_mfma_f32_32x32x64_f8f6f4, two waves per SIMD.
 // Persistent: the grid is one block per CU; a block walks its share of the output tiles and the LDS ring runs straight
 // across tile boundaries, so the first slabs of the next tile are already in flight while the epilogue stores drain.
-template <int FMT_A, int FMT_B, int EPI>
-__global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
-    constexpr int NWN = 4, NW = 8;
-    constexpr int TJ = 2;                     // n-tiles per wave; m-tiles per wave is 4
-    constexpr int LI = BM / (NW * 8);         // load instructions per wave per slab (each covers 8 rows) = 4
+template <int FMT_A, int FMT_B, int EPI, int NWN>
+__global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
+    constexpr int NW = 2 * NWN;
+    constexpr int TJ = BN / (NWN * 32);       // n-tiles per wave; m-tiles per wave is 4
+    constexpr int LI = BM / (NW * 8);         // load instructions per wave per slab (each covers 8 rows)
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -299,6 +299,10 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
 
 using namespace coat;
 
+#ifndef COAT_GEMM_NWN
+#define COAT_GEMM_NWN 4
+#endif
+
 extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
                              const void* scale_a, const void* scale_b, int s_dtype, const void* bias, int bias_dtype,
                              int64_t M, int64_t N, int64_t K, int QB, void* stream) {
@@ -334,12 +338,12 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     {                                                                                                              \
         static bool attr_set = false;                                                                              \
         if (!attr_set) {                                                                                           \
-            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP>,                 \
+            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP, COAT_GEMM_NWN>,                 \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);        \
             if (e != hipSuccess) return (int)e;                                                                    \
             attr_set = true;                                                                                       \
         }                                                                                                          \
-        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP>), dim3(grid), dim3(512), lds_bytes, st, G); \
+        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, COAT_GEMM_NWN>), dim3(grid), dim3(128 * COAT_GEMM_NWN), lds_bytes, st, G); \
         return coat_launch_status();                                                                               \
     }
 #define GEMM_FMT(EP)                                                             \
