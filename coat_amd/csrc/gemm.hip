@@ -5,16 +5,19 @@
 // every tensor is kept in both orientations so that forward, dgrad and wgrad are all of this form
 // (linear.py:253-302).  Operand formats are independent (e4m3 or e5m2 each: gradients are e5m2).
 //
-// Tiling: 256 x 256 per 256-thread block, 2 x 2 waves, each wave 128 x 128 as 4 x 4 tiles of
-// v_mfma_f32_32x32x64_f8f6f4; K advances in 64-byte slabs (one MFMA K-step).  LDS is a ring of four slabs
-// (4 x 32 KiB) filled straight from global memory (buffer_load ... lds, no register staging) three slabs ahead of
-// the one being multiplied; 16-byte chunks are XOR-swizzled with the row so that the 32-byte-per-lane fragment reads
-// are conflict-free.  Fragments are double-buffered in registers: those of slab k+1 are read while the 16 MFMAs of
-// slab k issue.  One barrier per slab.  The MFMA takes the B tile as its first operand, so a lane ends up holding
-// 4 consecutive n for one m per accumulator quad: bf16 rows are packed 4 at a time, and a 1 x 16 quantization group
-// is two quads in each of the lanes l and l^32.
-// Block ids are remapped so that the 8 XCDs (round-robin block dispatch) each work on a contiguous band of
-// tiles, ordered in panels of 8 tile-rows, which keeps A / B slabs hot in that XCD's L2.
+// Tiling: one 256 x 256 output tile per 512-thread block at a time, 2 x 4 waves, each wave 128 x 64 as 4 x 2 tiles of
+// v_mfma_f32_32x32x64_f8f6f4 (two waves per SIMD).  The grid is persistent, one block per CU (the LDS ring takes the
+// whole 160 KiB), and every block walks its share of the tiles; block ids map to tiles so that the 8 XCDs
+// (round-robin block dispatch) each work on a contiguous band of tiles, ordered in panels of 8 tile-rows, which keeps
+// A / B slabs hot in that XCD's L2.
+// K advances in steps of 128 bytes (two MFMA K-substeps).  LDS is a ring of five 32 KiB slabs (256 rows x 128 bytes of
+// one matrix), alternately A and B, filled straight from global memory (buffer_load_dwordx4 ... lds, no register
+// staging); the ring runs across tile boundaries, so the next tile's first slabs are in flight during the epilogue.
+// 16-byte chunks are XOR-swizzled with the row so that the 32-byte-per-lane fragment reads are conflict-free.
+// Fragments of both substeps are double-buffered in registers; there is one barrier per K-step, placed where every
+// wave holds the rest of the step in registers, which frees the step's two slabs for refilling.
+// The MFMA takes the B tile as its first operand, so a lane ends up holding 4 consecutive n for one m per accumulator
+// quad: bf16 rows are packed 4 at a time, and a 1 x 16 quantization group is two quads in each of the lanes l, l^32.
 #include "coat_device.h"
 #include "coat_host.h"
 
@@ -58,10 +61,12 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 // lands in LDS at lds_addr + 16 * lane without passing through registers; offsets beyond the buffer's extent fill
 // zeros.  Issued as inline assembly so that the compiler does not order later LDS reads behind it with a full
 // vmcnt(0) wait (it cannot tell which ring stage a read touches); completion is tracked by hand with s_waitcnt vmcnt.
-__device__ __forceinline__ void lds_dma16(v4i rsrc, uint32_t lds_addr, int voff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+// `soff` is a wave-uniform byte offset added to every lane's address; it takes no part in the range check, which is on
+// `voff` alone.
+__device__ __forceinline__ void lds_dma16(v4i rsrc, uint32_t lds_addr, int voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
-                 : "s"(lds_addr), "v"(voff), "s"(rsrc)
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                  : "memory", "m0");
 }
 __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
@@ -78,10 +83,10 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 // v_mfma_f32_32x32x64_f8f6f4, two waves per SIMD.
 // Persistent: the grid is one block per CU; a block walks its share of the output tiles and the LDS ring runs straight
 // across tile boundaries, so the first slabs of the next tile are already in flight while the epilogue stores drain.
-template <int FMT_A, int FMT_B, int EPI, int NWN>
-__global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
-    constexpr int NW = 2 * NWN;
-    constexpr int TJ = BN / (NWN * 32);       // n-tiles per wave; m-tiles per wave is 4
+template <int FMT_A, int FMT_B, int EPI>
+__global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
+    constexpr int NWN = 4, NW = 2 * NWN;      // waves along N, waves per block
+    constexpr int TJ = BN / (NWN * 32);       // n-tiles per wave (2); m-tiles per wave is 4
     constexpr int LI = BM / (NW * 8);         // load instructions per wave per slab (each covers 8 rows)
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -117,7 +122,8 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
     const int nstep = (G.K + BK - 1) / BK;
     // load cursor: tile iteration lt, K-step lstep of that tile, ring slot sl_load; slabs go A, B, A, B, ...
-    int offA[LI], offB[LI], kc[LI];
+    constexpr int kOob = 0x7FFFFFFF;
+    int offA[LI], offB[LI], kc[LI];  // per-lane byte offsets of K-step 0 (kOob for rows outside the matrix)
     const int lrow = wave * (LI * 8) + (lane >> 3);  // + 8 i
 #pragma unroll
     for (int i = 0; i < LI; i++) kc[i] = swz_chunk(lrow + 8 * i, lane & 7) * 16;
@@ -129,28 +135,39 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
 #pragma unroll
         for (int i = 0; i < LI; i++) {
             const int row = lrow + 8 * i;
-            offA[i] = (live && m0 + row < G.M) ? (m0 + row) * G.K + kc[i] : -1;
-            offB[i] = (live && n0 + row < G.N) ? (n0 + row) * G.K + kc[i] : -1;
+            offA[i] = (live && m0 + row < G.M) ? (m0 + row) * G.K + kc[i] : kOob;
+            offB[i] = (live && n0 + row < G.N) ? (n0 + row) * G.K + kc[i] : kOob;
         }
     };
     set_load_tile(0);
-    auto issue_A = [&]() {
+    // one load instruction (8 slab rows) of the A / B slab at the cursor.  Interior K-steps add the step's K offset
+    // as the instruction's scalar offset (no per-lane arithmetic); only a last, partial K-step masks lanes past K.
+    auto dma_row = [&](const v4i& rsrc, int off, int kci, int i) {
         const int k0 = lstep * BK;
-        const uint32_t dst = lds_base + sl_load * kUnitBytes + wave * (LI * 8 * BK);
-#pragma unroll
-        for (int i = 0; i < LI; i++) lds_dma16(rsrcA, dst + i * 8 * BK, (k0 + kc[i] < G.K && offA[i] >= 0) ? offA[i] + k0 : 0x7FFFFFFF);
-        sl_load = sl_load + 1 == NUNIT ? 0 : sl_load + 1;
+        const uint32_t dst = lds_base + sl_load * kUnitBytes + (wave * LI + i) * (8 * BK);
+        int v = off;
+        if (k0 + BK > G.K && k0 + kci >= G.K) v = kOob;
+        lds_dma16(rsrc, dst, v, k0);
     };
-    auto issue_B = [&]() {
-        const int k0 = lstep * BK;
-        const uint32_t dst = lds_base + sl_load * kUnitBytes + wave * (LI * 8 * BK);
-#pragma unroll
-        for (int i = 0; i < LI; i++) lds_dma16(rsrcB, dst + i * 8 * BK, (k0 + kc[i] < G.K && offB[i] >= 0) ? offB[i] + k0 : 0x7FFFFFFF);
+    auto dma_A = [&](int i) { dma_row(rsrcA, offA[i], kc[i], i); };
+    auto dma_B = [&](int i) { dma_row(rsrcB, offB[i], kc[i], i); };
+    auto next_A = [&]() { sl_load = sl_load + 1 == NUNIT ? 0 : sl_load + 1; };
+    auto next_B = [&]() {
         sl_load = sl_load + 1 == NUNIT ? 0 : sl_load + 1;
         if (++lstep == nstep) {
             lstep = 0;
             set_load_tile(++lt);  // past the last tile: zero fills, which keep the outstanding-load counts uniform
         }
+    };
+    auto issue_A = [&]() {
+#pragma unroll
+        for (int i = 0; i < LI; i++) dma_A(i);
+        next_A();
+    };
+    auto issue_B = [&]() {
+#pragma unroll
+        for (int i = 0; i < LI; i++) dma_B(i);
+        next_B();
     };
     // fragment addresses (bytes inside a slab) for this lane and K-substep 0: row = tile base + lane % 32, 16-byte
     // chunks 2 * (lane / 32) + h; the chunks of substep 1 are those + 4, i.e. the address with bit 6 flipped.
@@ -163,59 +180,84 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
         fb_off[h] = rowb * BK + (swz_chunk(rowb, c) << 4);
     }
     int sl_frag = 0;  // ring slot of the A slab of the K-step being multiplied (its B slab is in the next slot)
-    auto load_frags = [&](int slot_a, int sub, v8i* fa, v8i* fb) {
-        const uint8_t* sa = lds + slot_a * kUnitBytes;
-        const uint8_t* sb = lds + (slot_a + 1 == NUNIT ? 0 : slot_a + 1) * kUnitBytes;
+    auto load_fa = [&](int slot_a, int sub, int t) -> v8i {
+        const uint8_t* sa = lds + slot_a * kUnitBytes + t * 32 * BK;
         const int x = sub * 64;
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const uint4 a0 = *(const uint4*)(sa + ((fa_off[0] ^ x) + t * 32 * BK)), a1 = *(const uint4*)(sa + ((fa_off[1] ^ x) + t * 32 * BK));
-            fa[t] = (v8i){(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
-        }
-#pragma unroll
-        for (int t = 0; t < TJ; t++) {
-            const uint4 b0 = *(const uint4*)(sb + ((fb_off[0] ^ x) + t * 32 * BK)), b1 = *(const uint4*)(sb + ((fb_off[1] ^ x) + t * 32 * BK));
-            fb[t] = (v8i){(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
-        }
+        const uint4 a0 = *(const uint4*)(sa + (fa_off[0] ^ x)), a1 = *(const uint4*)(sa + (fa_off[1] ^ x));
+        return (v8i){(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+    };
+    auto load_fb = [&](int slot_a, int sub, int t) -> v8i {
+        const uint8_t* sb = lds + (slot_a + 1 == NUNIT ? 0 : slot_a + 1) * kUnitBytes + t * 32 * BK;
+        const int x = sub * 64;
+        const uint4 b0 = *(const uint4*)(sb + (fb_off[0] ^ x)), b1 = *(const uint4*)(sb + (fb_off[1] ^ x));
+        return (v8i){(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
     };
 
     v16f acc[TJ][4];  // [n-tile j][m-tile i]
     v8i fax[4], fbx[TJ], fay[4], fby[TJ];  // fragments of K-substep 0 (x) and 1 (y)
-    // prologue: fill the ring (A0 B0 A1 B1 A2), wait for the first step's two slabs, fetch its substep-0 fragments
+    // prologue: two K-steps in flight (A0 B0 A1 B1), wait for the first step's two slabs, fetch its substep-0 fragments
     issue_A();
     issue_B();
     issue_A();
     issue_B();
-    issue_A();
-    COAT_WAIT_VMCNT(3 * LI);
+    COAT_WAIT_VMCNT(2 * LI);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    load_frags(sl_frag, 0, fax, fbx);
+#pragma unroll
+    for (int t = 0; t < 4; t++) fax[t] = load_fa(sl_frag, 0, t);
+#pragma unroll
+    for (int t = 0; t < TJ; t++) fbx[t] = load_fb(sl_frag, 0, t);
+#define COAT_MFMA(FB_, FA_, J, I) \
+    acc[J][I] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FB_[J], FA_[I], acc[J][I], FMT_B, FMT_A, 0, 0, 0, 0)
+#define COAT_PIN() __builtin_amdgcn_sched_barrier(0)
     // One K-step of 128 = 2 substeps x 8 MFMAs per wave, with one barrier in the middle:
-    //   read the substep-1 fragments, multiply substep 0;
+    //   multiply substep 0 while reading the substep-1 fragments;
     //   wait until those reads have returned and at most the newest slab is outstanding, barrier: every wave now holds
     //   all it needs from this step's two slabs in registers, and the next step's slabs have landed and are visible
     //   (loads return in order, so this holds also when epilogue stores of the previous tile are still in the count);
-    //   refill this step's two slots, read the next step's substep-0 fragments, multiply substep 1.
+    //   multiply substep 1 while refilling this step's two slots and reading the next step's substep-0 fragments.
+    // Loads and LDS reads are spread between the MFMAs by hand (and pinned) so that the matrix pipe never waits for a
+    // burst of address arithmetic after the barrier.
+    static_assert(TJ == 2 && LI == 4 && NW == 8, "the interleaving below is written for eight waves of 128 x 64");
     auto step = [&]() {
-        load_frags(sl_frag, 1, fay, fby);
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fbx[j], fax[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
+        // substep 0: 8 MFMAs; between them the substep-1 fragment reads and the four loads of the A slab two steps ahead
+        COAT_MFMA(fbx, fax, 0, 0); COAT_PIN();
+        fay[0] = load_fa(sl_frag, 1, 0); fby[0] = load_fb(sl_frag, 1, 0); COAT_PIN();
+        COAT_MFMA(fbx, fax, 0, 1); COAT_PIN();
+        dma_A(0); COAT_PIN();
+        COAT_MFMA(fbx, fax, 0, 2); COAT_PIN();
+        fay[1] = load_fa(sl_frag, 1, 1); fby[1] = load_fb(sl_frag, 1, 1); COAT_PIN();
+        COAT_MFMA(fbx, fax, 0, 3); COAT_PIN();
+        dma_A(1); COAT_PIN();
+        COAT_MFMA(fbx, fax, 1, 0); COAT_PIN();
+        fay[2] = load_fa(sl_frag, 1, 2); fay[3] = load_fa(sl_frag, 1, 3); COAT_PIN();
+        COAT_MFMA(fbx, fax, 1, 1); COAT_PIN();
+        dma_A(2); COAT_PIN();
+        COAT_MFMA(fbx, fax, 1, 2); COAT_PIN();
+        dma_A(3); next_A(); COAT_PIN();
+        COAT_MFMA(fbx, fax, 1, 3); COAT_PIN();
         COAT_WAIT_VMCNT_LGKM0(LI);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        issue_B();
-        issue_A();
-        sl_frag = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
-        load_frags(sl_frag, 0, fax, fbx);
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fby[j], fay[i], acc[j][i], FMT_B, FMT_A, 0, 0, 0, 0);
+        const int sl_next = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
+        // substep 1: 8 MFMAs; between them the next step's substep-0 fragment reads and the four loads of its
+        // successor's B slab
+        COAT_MFMA(fby, fay, 0, 0); COAT_PIN();
+        fax[0] = load_fa(sl_next, 0, 0); fbx[0] = load_fb(sl_next, 0, 0); COAT_PIN();
+        COAT_MFMA(fby, fay, 0, 1); COAT_PIN();
+        dma_B(0); COAT_PIN();
+        COAT_MFMA(fby, fay, 0, 2); COAT_PIN();
+        fax[1] = load_fa(sl_next, 0, 1); fbx[1] = load_fb(sl_next, 0, 1); COAT_PIN();
+        COAT_MFMA(fby, fay, 0, 3); COAT_PIN();
+        dma_B(1); COAT_PIN();
+        COAT_MFMA(fby, fay, 1, 0); COAT_PIN();
+        fax[2] = load_fa(sl_next, 0, 2); fax[3] = load_fa(sl_next, 0, 3); COAT_PIN();
+        COAT_MFMA(fby, fay, 1, 1); COAT_PIN();
+        dma_B(2); COAT_PIN();
+        COAT_MFMA(fby, fay, 1, 2); COAT_PIN();
+        dma_B(3); next_B(); COAT_PIN();
+        COAT_MFMA(fby, fay, 1, 3); COAT_PIN();
+        sl_frag = sl_next;
     };
     const float scale = load_rt_f32(G.sa, 0, G.s_dt) * load_rt_f32(G.sb, 0, G.s_dt);
     if (EPI != kEpiBf16) enable_fp8_saturation();
@@ -299,10 +341,6 @@ __global__ __launch_bounds__(128 * NWN) void k_fp8_gemm(GemmArgs G) {
 
 using namespace coat;
 
-#ifndef COAT_GEMM_NWN
-#define COAT_GEMM_NWN 4
-#endif
-
 extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
                              const void* scale_a, const void* scale_b, int s_dtype, const void* bias, int bias_dtype,
                              int64_t M, int64_t N, int64_t K, int QB, void* stream) {
@@ -338,12 +376,12 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     {                                                                                                              \
         static bool attr_set = false;                                                                              \
         if (!attr_set) {                                                                                           \
-            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP, COAT_GEMM_NWN>,                 \
+            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP>,                 \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);        \
             if (e != hipSuccess) return (int)e;                                                                    \
             attr_set = true;                                                                                       \
         }                                                                                                          \
-        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, COAT_GEMM_NWN>), dim3(grid), dim3(128 * COAT_GEMM_NWN), lds_bytes, st, G); \
+        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP>), dim3(grid), dim3(512), lds_bytes, st, G); \
         return coat_launch_status();                                                                               \
     }
 #define GEMM_FMT(EP)                                                             \
