@@ -204,6 +204,17 @@ def cpu_baseline_adamw(torch):
             "sample": f"{reps} steps over the first {n} elements (4096 groups) of the tensor, oracle/adamw_ref.c, 1 thread"}
 
 
+# HBM / fabric bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled by what the same
+# counters read for a 256 MiB copy); the runs are recorded under profiles/.  They cannot be taken inside this process.
+MEASURED_TRAFFIC = {
+    "adamw": 739.1e6,               # profiles/k_fp8_adamw_expand__adamw_11008x4096.txt
+    "quantize": 52.5e6,             # profiles/k_quantize_pg__quantize_4096x4096_bf16.txt
+    "quantize_transpose": 78.8e6,   # profiles/k_quantize_transpose__quantize_transpose_4096x4096_bf16.txt
+    "gemm_fwd": 809.2e6,            # profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt
+    "gemm_dgrad": 617.0e6,
+}
+
+
 def ramp_clocks(step, seconds, torch):
     """Keep the GPU continuously busy with `step` for `seconds` (untimed) so that the timed region runs at the sustained clock."""
     if seconds <= 0:
@@ -327,7 +338,7 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8" if is_gemm else "f32", "data": "synthetic", "config": cfg,
         "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
                      ("algorithmic_flops_per_launch" if is_gemm else "algorithmic_bytes_per_launch"): nbytes, "kernel_ms_avg": round(avg_ms, 5),
                      "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5)},
     }
