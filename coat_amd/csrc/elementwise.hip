@@ -71,7 +71,16 @@ __device__ __forceinline__ void store_bf16x16(void* p, int64_t chunk, const floa
     dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
 }
 
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+// 1 / (1 + exp(-x)) on the hardware transcendental units: exp(-x) = 2^n * v_exp_f32(f) with t = -x log2(e) split into
+// n = rint(t) and f = fma(x, -log2(e), -n) (so the exponent argument keeps full precision for large |x|), then
+// v_rcp_f32.  About 2 ulp against the correctly rounded value; overflow of 2^t gives 1 / inf = 0 like the libm form.
+__device__ __forceinline__ float sigmoid_f32(float x) {
+    constexpr float kNegLog2e = -1.44269504088896340736f;
+    const float n = __builtin_rintf(fminf(fmaxf(x * kNegLog2e, -150.0f), 150.0f));
+    const float f = fmaf(x, kNegLog2e, -n);
+    const float e = __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(f), (int)n);
+    return __builtin_amdgcn_rcpf(1.0f + e);
+}
 
 template <int OP, int KIND_IN, int KIND_OUT>
 __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {

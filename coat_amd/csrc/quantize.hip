@@ -30,6 +30,20 @@ template <int XDT> __device__ __forceinline__ void load_vec(const void* x, int64
     }
 }
 
+// the same conversion for 16 bytes already in registers
+template <int XDT> __device__ __forceinline__ void unpack_vec(const uint4& t, float* v) {
+    if (XDT == kF32) {
+        v[0] = u2f(t.x); v[1] = u2f(t.y); v[2] = u2f(t.z); v[3] = u2f(t.w);
+    } else {
+        uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = XDT == kBF16 ? bf16lo(w[i]) : f16lo(w[i]);
+            v[2 * i + 1] = XDT == kBF16 ? bf16hi(w[i]) : f16hi(w[i]);
+        }
+    }
+}
+
 template <int VEC> __device__ __forceinline__ float vec_amax(const float* v) {
     float a = fmaxf(fabsf(v[0]), fabsf(v[1]));
 #pragma unroll
@@ -282,67 +296,88 @@ __global__ __launch_bounds__(256) void k_division_transpose(const void* __restri
 template <int XDT, int SDT, int KIND, int QB, int TM>
 __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restrict__ x, void* __restrict__ q,
                                                              void* __restrict__ s_out, void* __restrict__ qt,
-                                                             void* __restrict__ st_out, int64_t M, int64_t N) {
+                                                             void* __restrict__ st_out, int64_t M, int64_t N,
+                                                             int tiles_per_block) {
     constexpr int VEC = VecOf<XDT>::kVec;
+    constexpr int ESIZE = 16 / VEC;
     constexpr int LPG = QB / VEC;
     constexpr int PITCH = kTileN + 1;
     static_assert(QB <= kTileN && TM % QB == 0, "tile must hold whole groups in both directions");
     __shared__ float tile[TM * PITCH];
     enable_fp8_saturation();
-    const int64_t tiles_n = (N + kTileN - 1) / kTileN;
-    const int64_t m0 = (blockIdx.x / tiles_n) * TM, n0 = (blockIdx.x % tiles_n) * kTileN;
+    const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = (N + kTileN - 1) / kTileN;
     const int64_t SN = N / QB, SM = M / QB;
+    // A block walks a contiguous range of tile ids; ids run down a 64-column strip (m fastest), so the 8-byte pieces
+    // of transposed scales and the 64-byte pieces of transposed codes that consecutive tiles write are neighbours and
+    // merge in L2.  The next tile's input is fetched into registers before the barrier and lands during phase 2.
+    const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_block;
+    const int64_t t_end = min(t_begin + tiles_per_block, tiles_m * tiles_n);
 
-    // phase 1: jobs of VEC consecutive elements; a row of the tile is 64/VEC jobs (a multiple of LPG)
+    // phase-1 jobs: VEC consecutive elements (16 bytes); a row of the tile is 64/VEC jobs (a multiple of LPG)
     constexpr int JPR = kTileN / VEC;
     constexpr int JOBS = TM * JPR;
     static_assert(JOBS % 256 == 0, "phase 1 keeps all lanes of a group in the same iteration");
-    for (int job = threadIdx.x; job < JOBS; job += 256) {
-        int row = job / JPR, cv = job % JPR;
-        int64_t m = m0 + row, n = n0 + cv * VEC;
-        bool ok = m < M && n < N;  // N % QB == 0: a group is inside or outside as a whole
-        float v[VEC];
-        if (ok) load_vec<XDT>(x, m * N + n, v);
-        else {
+    constexpr int NIT = JOBS / 256;
+    uint4 raw[NIT];
+    auto fetch = [&](int64_t t) {
+        const int64_t m0 = (t % tiles_m) * TM, n0 = (t / tiles_m) * kTileN;
 #pragma unroll
-            for (int k = 0; k < VEC; k++) v[k] = 0.0f;
+        for (int it = 0; it < NIT; it++) {
+            const int job = threadIdx.x + it * 256;
+            const int64_t m = m0 + job / JPR, n = n0 + (job % JPR) * VEC;
+            raw[it] = (m < M && n < N) ? *(const uint4*)((const uint8_t*)x + (m * N + n) * ESIZE) : make_uint4(0, 0, 0, 0);
         }
-        float amax = cluster_max<LPG>(vec_amax<VEC>(v));
-        float s = group_scale<KIND>(amax);
-        float r = 1.0f / s;
-        uint32_t c[VEC / 4];
-        quantize_vec<KIND, VEC>(v, s, r, c);
-        if (ok) {
-            store_codes<VEC>(q, m * N + n, c);
-            if ((threadIdx.x % LPG) == 0) store_from_f32<SDT>(s_out, m * SN + n / QB, s);
-        }
+    };
+    if (t_begin < t_end) fetch(t_begin);
+    for (int64_t t = t_begin; t < t_end; t++) {
+        const int64_t m0 = (t % tiles_m) * TM, n0 = (t / tiles_m) * kTileN;
 #pragma unroll
-        for (int k = 0; k < VEC; k++) tile[row * PITCH + cv * VEC + k] = v[k];
-    }
-    __syncthreads();
+        for (int it = 0; it < NIT; it++) {
+            const int job = threadIdx.x + it * 256;
+            const int row = job / JPR, cv = job % JPR;
+            const int64_t m = m0 + row, n = n0 + cv * VEC;
+            const bool ok = m < M && n < N;  // N % QB == 0: a group is inside or outside as a whole
+            float v[VEC];
+            unpack_vec<XDT>(raw[it], v);
+            float amax = cluster_max<LPG>(vec_amax<VEC>(v));
+            float s = group_scale<KIND>(amax);
+            float r = 1.0f / s;
+            uint32_t c[VEC / 4];
+            quantize_vec<KIND, VEC>(v, s, r, c);
+            if (ok) {
+                store_codes<VEC>(q, m * N + n, c);
+                if ((threadIdx.x % LPG) == 0) store_from_f32<SDT>(s_out, m * SN + n / QB, s);
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; k++) tile[row * PITCH + cv * VEC + k] = v[k];
+        }
+        if (t + 1 < t_end) fetch(t + 1);
+        __syncthreads();
 
-    // phase 2: job = (column n, 16-row chunk mc), mc fastest so that neighbouring lanes write
-    // neighbouring 16-byte pieces of one qt row; groups of QB rows are QB/16 neighbouring lanes.
-    constexpr int MC = TM / 16;
-    constexpr int LPG_T = QB / 16;
-    constexpr int JOBS2 = MC * kTileN;
-    static_assert(JOBS2 % 256 == 0, "phase 2 keeps all lanes of a group in the same iteration");
-    for (int job = threadIdx.x; job < JOBS2; job += 256) {
-        int mc = job % MC, col = job / MC;
-        int64_t m = m0 + mc * 16, n = n0 + col;
-        bool ok = m < M && n < N;  // M % QB == 0: whole groups again
-        float v[16];
+        // phase 2: job = (column n, 16-row chunk mc), mc fastest so that neighbouring lanes write
+        // neighbouring 16-byte pieces of one qt row; groups of QB rows are QB/16 neighbouring lanes.
+        constexpr int MC = TM / 16;
+        constexpr int LPG_T = QB / 16;
+        constexpr int JOBS2 = MC * kTileN;
+        static_assert(JOBS2 % 256 == 0, "phase 2 keeps all lanes of a group in the same iteration");
+        for (int job = threadIdx.x; job < JOBS2; job += 256) {
+            int mc = job % MC, col = job / MC;
+            int64_t m = m0 + mc * 16, n = n0 + col;
+            bool ok = m < M && n < N;  // M % QB == 0: whole groups again
+            float v[16];
 #pragma unroll
-        for (int i = 0; i < 16; i++) v[i] = tile[(mc * 16 + i) * PITCH + col];
-        float amax = cluster_max<LPG_T>(vec_amax<16>(v));
-        float s = group_scale<KIND>(amax);
-        float r = 1.0f / s;
-        uint32_t c[4];
-        quantize_vec<KIND, 16>(v, s, r, c);
-        if (ok) {
-            *(uint4*)((uint8_t*)qt + n * M + m) = make_uint4(c[0], c[1], c[2], c[3]);
-            if ((mc % LPG_T) == 0) store_from_f32<SDT>(st_out, n * SM + m / QB, s);
+            for (int i = 0; i < 16; i++) v[i] = tile[(mc * 16 + i) * PITCH + col];
+            float amax = cluster_max<LPG_T>(vec_amax<16>(v));
+            float s = group_scale<KIND>(amax);
+            float r = 1.0f / s;
+            uint32_t c[4];
+            quantize_vec<KIND, 16>(v, s, r, c);
+            if (ok) {
+                *(uint4*)((uint8_t*)qt + n * M + m) = make_uint4(c[0], c[1], c[2], c[3]);
+                if ((mc % LPG_T) == 0) store_from_f32<SDT>(st_out, n * SM + m / QB, s);
+            }
         }
+        __syncthreads();  // the tile is rewritten by the next iteration
     }
 }
 
@@ -525,11 +560,13 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
     if (QB > 64) return COAT_ESHAPE;  // column groups must fit the 64-wide tile
     hipStream_t st = (hipStream_t)stream;
     constexpr int TM = 64;
-    int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
+    const int64_t ntiles = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
+    const int tiles_per_block = (int)((ntiles + 8191) / 8192);  // one tile per block up to 32 blocks per CU (measured faster than fewer, longer blocks)
+    const int64_t blocks = (ntiles + tiles_per_block - 1) / tiles_per_block;
 #define LAUNCH_QT(QBV)                                                                                               \
     DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                 \
         hipLaunchKernelGGL((k_quantize_transpose<XDT, SDT, KIND, QBV, TM>), dim3((unsigned)blocks), dim3(256), 0, st, \
-                           x, q, s, qt, st_out, M, N);                                                               \
+                           x, q, s, qt, st_out, M, N, tiles_per_block);                                              \
         return coat_launch_status();                                                                                 \
     })))
     switch (QB) {

@@ -193,11 +193,28 @@ __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__
 template <int WDT>
 __global__ __launch_bounds__(256) void k_rmsnorm_dw(const float* __restrict__ partial, void* __restrict__ dw, int nblocks,
                                                      int N) {
-    const int col = blockIdx.x * 256 + threadIdx.x;
-    if (col >= N) return;
-    float s = 0.0f;
-    for (int b = 0; b < nblocks; b++) s += partial[(int64_t)b * N + col];
-    store_from_f32<WDT>(dw, col, s);
+    // 32 columns per block, the partial rows split over 8 thread slices (fixed order: deterministic), 8 loads in flight
+    __shared__ float red[8][32];
+    const int c = threadIdx.x & 31, slice = threadIdx.x >> 5;
+    const int col = blockIdx.x * 32 + c;
+    float acc[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) acc[u] = 0.0f;
+    if (col < N) {
+        for (int b0 = slice * 8; b0 < nblocks; b0 += 64) {
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (b0 + u < nblocks) acc[u] += partial[(int64_t)(b0 + u) * N + col];
+        }
+    }
+    red[slice][c] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+    __syncthreads();
+    if (slice == 0 && col < N) {
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) s += red[k][c];
+        store_from_f32<WDT>(dw, col, s);
+    }
 }
 
 }  // namespace coat
@@ -257,7 +274,7 @@ extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x
     const int64_t grid = n_partial < M ? n_partial : M;
     RMS_DISPATCH(k_rmsnorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, rstd, dx, dw_partial, M, (int)N, QB)
     if (int e = coat_launch_status()) return e;
-    const int cols_blocks = (int)((N + 255) / 256);
+    const int cols_blocks = (int)((N + 31) / 32);
     switch (w_dtype) {
         case COAT_F32: hipLaunchKernelGGL((k_rmsnorm_dw<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
         case COAT_BF16: hipLaunchKernelGGL((k_rmsnorm_dw<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
