@@ -43,6 +43,23 @@ def test_fp8matmul_bf16(dev, M, N, K, fa, fb):
     check_bf16(c, a, b, sa, sb)
 
 
+@pytest.mark.parametrize("M,N,K,fa", [(4352, 4112, 400, E4), (5000, 4608, 144, E5)])
+def test_fp8matmul_more_tiles_than_cus(dev, M, N, K, fa):
+    """More 256 x 256 tiles than the chip has CUs: every block walks several tiles with its LDS ring running across the
+    tile boundary; ragged last tile row / column and a partial last K-step included."""
+    lin = _lin()
+    a, b = rand_fp8((M, K), 11, fa), rand_fp8((N, K), 12, E4)
+    sa, sb = torch.tensor(0.03).bfloat16(), torch.tensor(0.011).bfloat16()
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(13)).bfloat16()
+    c = lin.fp8matmul(a.to(dev), b.to(dev).t(), False, sa.to(dev), sb.to(dev), 16, bias.to(dev))
+    check_bf16(c, a, b, sa, sb, bias)
+    # same operands through the quantizing epilogue: dequantized output within one e4m3 step of the bf16 result
+    cq, cs = lin.fp8matmul(a.to(dev), b.to(dev).t(), True, sa.to(dev), sb.to(dev), 16, bias.to(dev))
+    deq = cq.cpu().float().reshape(M, N // 16, 16) * cs.cpu().float().unsqueeze(-1)
+    gmax = c.cpu().float().reshape(M, N // 16, 16).abs().amax(dim=2, keepdim=True)
+    assert ((deq - c.cpu().float().reshape(M, N // 16, 16)).abs() <= gmax * 2.0 ** -3 + 1e-6).all()
+
+
 def test_fp8matmul_bias_batched_and_rowmajor_b(dev):
     lin = _lin()
     a, b = rand_fp8((4 * 96, 256), 3, E4).reshape(4, 96, 256), rand_fp8((160, 256), 4, E4)
