@@ -107,6 +107,81 @@ def make_gemm_workload(dev, torch, which):
                          "M": M_, "N": N_, "K": K_, "kernel": "k_fp8_gemm"}
 
 
+def make_linear_workload(dev, torch):
+    """BASELINE configs[2] end to end: FP8Linear forward + backward at the Llama-2-7B MLP shape: per-tensor quantization
+    (with transposes) of X, W and the output gradient, then the three GEMMs.  Returns (fp8 step, bf16 step, flops)."""
+    from coat_amd.activation.real_quantization.fp8linear import FP8Linear
+
+    T, K, N = 8192, 4096, 11008
+    torch.manual_seed(0)
+    lin = FP8Linear(K, N, bias=False, device=dev).to(torch.bfloat16).train()
+    torch.nn.init.normal_(lin.weight, std=0.02)
+    ref = torch.nn.Linear(K, N, bias=False, device=dev, dtype=torch.bfloat16)
+    ref.weight.data.copy_(lin.weight.data)
+    x = (torch.randn(4, 2048, K, device=dev) * 0.02).bfloat16()
+    g = (torch.randn(4, 2048, N, device=dev) * 1e-2).bfloat16()
+
+    def run(mod):
+        def step():
+            mod.weight.grad = None
+            xin = x.detach().requires_grad_(True)
+            mod(xin).backward(g)
+        return step
+
+    return run(lin), run(ref), 3 * 2 * T * K * N, {
+        "workload": f"FP8Linear fwd+bwd: X bf16 [4,2048,{K}] x W [{N},{K}], e4m3 per-tensor X/W, e5m2 grad, bf16 outputs",
+        "M": T, "N": N, "K": K}
+
+
+def make_silu_mul_workload(dev, torch):
+    """BASELINE configs[3]: SiLU(gate) * up on bf16 [8192,11008] inputs -> FP8 with 1x16 scales (and the saved FP8
+    activations), then the backward chain with a bf16 gradient, as CoatLlamaMLPResidual strings the kernels together
+    (coat/models/coat_llama.py:664-766)."""
+    import coat_amd.activation.real_quantization as rq
+
+    M, N, QB = 8192, 11008, 16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    gate = torch.randn(M, N, generator=gen, device=dev).bfloat16()
+    up = torch.randn(M, N, generator=gen, device=dev).bfloat16()
+    g = (torch.randn(M, N, generator=gen, device=dev) * 1e-2).bfloat16()
+
+    def step():
+        qg, sg = rq.fp8_quantize(gate, QB, "E4M3")
+        qu, su = rq.fp8_quantize(up, QB, "E4M3")
+        qs, ss = rq.fp8_silu_forward(qg, sg, QB)
+        rq.fp8_mul_forward(qs, ss, qu, su, QB, transpose_output_2d=True)
+        g1, _ = rq.fp8_mul_backward(qs, ss, qu, su, g, QB, "E5M2", output_quantized_transpose=True)
+        rq.fp8_silu_backward(qg, sg, g1, QB, "E5M2", output_quantized_transpose=True)
+
+    E = M * N
+    # forward: read 2 bf16 inputs (4E), write gate / up / silu codes + scales 3(E + E/8), write product q + q^T (2E);
+    # backward: read g (2E) + the three saved FP8 tensors 3(E + E/8), write two gradients as q + q^T (4E)
+    nbytes = int(4 * E + 3 * (E + E / 8) + 2 * E + 2 * E + 3 * (E + E / 8) + 4 * E)
+    return step, nbytes, {"workload": f"SiLU(gate)*up fwd + bwd chain on bf16 [{M},{N}], 1x16 e4m3 / per-tensor e5m2 outputs",
+                          "M": M, "N": N, "kernel": "k_quantize_pg, k_elementwise, k_division_transpose"}
+
+
+def make_rmsnorm_workload(dev, torch):
+    """BASELINE configs[3], second half: RMSNorm on the FP8 block input [8192,4096] -> FP8 (+ transpose), and its backward."""
+    import coat_amd.activation.real_quantization as rq
+
+    M, N, QB = 8192, 4096, 16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(M, N, generator=gen, device=dev).bfloat16()
+    w = torch.ones(N, device=dev, dtype=torch.bfloat16)
+    g = (torch.randn(M, N, generator=gen, device=dev) * 1e-2).bfloat16()
+    q, s = rq.fp8_quantize(x, QB, "E4M3")
+
+    def step():
+        qy, sy, qyt, (_, rstd, nw) = rq.fp8_rmsnorm_forward(q, s, w, QB, 1e-5, transpose_output_2d=True)
+        rq.fp8_rmsnorm_backward(q, s, g, w, rstd, QB, nw)
+
+    E = M * N
+    nbytes = int((E + E / 8) + 2 * E + (E + E / 8) + 2 * E + 2 * E)  # fwd: codes+scales in, q + q^T out; bwd: codes+scales, dy in, dx out
+    return step, nbytes, {"workload": f"RMSNorm fwd (FP8 in -> per-tensor FP8 + transpose) + bwd on [{M},{N}]",
+                          "M": M, "N": N, "kernel": "k_rmsnorm_fwd, k_division_transpose, k_rmsnorm_bwd, k_rmsnorm_dw"}
+
+
 class Bf16DecoderLayer:
     """The same Llama decoder layer in plain bf16 torch (F.linear / F.rms_norm / F.silu / SDPA): the baseline the FP8
     layer has to beat (benchmark/benchmark_llamalayer.py of the reference times HF's LlamaDecoderLayer the same way)."""
@@ -227,7 +302,10 @@ def ramp_clocks(step, seconds, torch):
 
 
 def bench_layer(args, dev, torch):
-    step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1])
+    if args.workload == "linear":
+        step_fp8, step_bf16, gemm_flops, cfg = make_linear_workload(dev, torch)
+    else:
+        step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1])
 
     def time_it(fn):
         ramp_clocks(fn, args.ramp_seconds, torch)
@@ -269,7 +347,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "layer_7b", "layer_13b"])
+    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
+                             "silu_mul", "rmsnorm", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ramp-seconds", type=float, default=1.5,
                     help="untimed continuous run of the step before the W warmup steps: an idle MI355X sits at ~100 MHz and "
@@ -295,12 +374,16 @@ def main():
     torch.cuda.set_device(dev)
 
     is_gemm = args.workload.startswith("gemm")
-    if args.workload.startswith("layer"):
+    if args.workload.startswith("layer") or args.workload == "linear":
         return bench_layer(args, dev, torch)
     if args.workload == "adamw":
         step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch)
     elif is_gemm:
         step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1])
+    elif args.workload == "silu_mul":
+        step, nbytes, cfg = make_silu_mul_workload(dev, torch)
+    elif args.workload == "rmsnorm":
+        step, nbytes, cfg = make_rmsnorm_workload(dev, torch)
     else:
         step, nbytes, cfg = make_quantize_workload(dev, torch, args.workload == "quantize_transpose")
 
