@@ -1,0 +1,48 @@
+"""FP8 LayerNorm without affine parameters, forward / backward.
+Reference: coat/activation/real_quantization/func_layernorm_noparam.py:193-297."""
+import torch
+
+from ... import _hip
+from ._division import _division
+from ._fused import new_max, prep_bf16, prep_pg
+from .common import no_stochastic, restore
+
+
+def _forward(x, s_x, w, b, QB, eps, transpose_output_2d, who):
+    x, s_x, batch = prep_pg(x, s_x)
+    M, N = x.shape
+    y = torch.empty_like(x, dtype=torch.float32)  # the reference keeps the normalised tensor in fp32 (:205)
+    s_row = torch.empty((M,), dtype=torch.bfloat16, device=x.device)
+    mean = torch.empty((M,), dtype=torch.float32, device=x.device)
+    rstd = torch.empty((M,), dtype=torch.float32, device=x.device)
+    s_max = new_max(x.device)
+    _hip.check(_hip.lib().coat_fp8_layernorm_forward(
+        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.ptr(b),
+        -1 if w is None else _hip.dt(w), _hip.ptr(y), _hip.ptr(s_row), _hip.ptr(mean), _hip.ptr(rstd), _hip.ptr(s_max),
+        M, N, QB, float(eps), _hip.stream(x.device)), who)
+    qy, s_y_max, qy_t = _division(y, x.dtype, s_max.to(torch.bfloat16), True, True, who)
+    if batch is not None and not transpose_output_2d:
+        qy_t = qy_t.reshape(batch, -1, N)
+    return restore(qy, batch), s_y_max, qy_t, mean, rstd
+
+
+def fp8_layernorm_noparam_forward(x, s_x, QB, eps, transpose_output_2d=False):
+    """Returns (qy, s_y_max, qy_t, (mean, rstd, num_warps)); qy is per-tensor FP8 in x's dtype."""
+    qy, s_y_max, qy_t, mean, rstd = _forward(x, s_x, None, None, QB, eps, transpose_output_2d,
+                                             "fp8_layernorm_noparam_forward")
+    num_warps = 8  # kept in the tuple for signature compatibility; the HIP kernels do not use it
+    return qy, s_y_max, qy_t, (mean, rstd, num_warps)
+
+
+def fp8_layernorm_noparam_backward(x, s_x, g, QB, m, v, num_warps, stochastic=False):
+    """Returns dx (bf16); ``m`` / ``v`` are the mean / rstd saved by the forward."""
+    no_stochastic(stochastic)
+    x, s_x, batch = prep_pg(x, s_x)
+    g = prep_bf16(g)
+    M, N = g.shape
+    mean, rstd = _hip.dense(m.to(torch.float32)), _hip.dense(v.to(torch.float32))
+    dx = torch.empty_like(g, dtype=torch.bfloat16)
+    _hip.check(_hip.lib().coat_fp8_layernorm_backward(
+        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(g), None, -1, _hip.ptr(mean), _hip.ptr(rstd),
+        _hip.ptr(dx), None, None, None, None, 0, M, N, QB, _hip.stream(x.device)), "fp8_layernorm_noparam_backward")
+    return restore(dx, batch)

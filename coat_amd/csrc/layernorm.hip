@@ -1,0 +1,263 @@
+// FP8 LayerNorm forward / backward for gfx950, without and with affine parameters.
+//
+// Reference: coat/activation/real_quantization/func_layernorm_noparam.py (_layer_norm_fwd_fused :53-115,
+// _layer_norm_bwd_dx_fused :125-190) and func_layernorm_param.py (_layer_norm_fwd_fused :51-125,
+// _layer_norm_bwd_dx_fused :134-226, _fp8_layer_norm_bwd_dwdb :229-255).
+//
+// Same organisation as the RMSNorm kernels: one 256-thread block per row, the dequantized row stays in registers
+// for the mean pass, the variance pass (two-pass variance, as the reference computes it) and the output pass.
+// The forward output is fp32 (the reference allocates y as float32 and lets the per-tensor division read that).
+// dw / db use per-block fp32 partial rows and a column reduction in block order instead of the reference's
+// lock-guarded accumulation in the weight dtype.
+#include <math.h>
+
+#include "coat_host.h"
+#include "norm_common.h"
+
+namespace coat {
+
+constexpr int kNoParam = 3;  // WMODE: 0..2 = dtype of w and b, 3 = no affine parameters
+
+template <int WMODE> __device__ __forceinline__ void load_wb16(const void* w, int col, float* o) {
+    if (WMODE == kNoParam) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[i] = 1.0f;
+    } else {
+        load_w16<WMODE == kNoParam ? kF32 : WMODE>(w, col, o);
+    }
+}
+__device__ __forceinline__ void load_bf16_16(const void* p, int64_t off, float* v) {
+    const uint4* src = (const uint4*)((const uint16_t*)p + off);
+    uint4 a = src[0], b = src[1];
+    uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        v[2 * k] = bf16lo(u[k]);
+        v[2 * k + 1] = bf16hi(u[k]);
+    }
+}
+
+// Forward: y = (x - mean) * rstd (* w + b) in fp32, mean[row], rstd[row], row scale (max|y| + 1e-10)/fp8max (bf16),
+// tensor max of the row scales.
+template <int KIND, int WMODE, int ITERS>
+__global__ __launch_bounds__(256) void k_layernorm_fwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                        const void* __restrict__ w, const void* __restrict__ b,
+                                                        float* __restrict__ y, void* __restrict__ s_row,
+                                                        float* __restrict__ mean_out, float* __restrict__ rstd_out,
+                                                        float* __restrict__ s_max, int N, int qb, float eps) {
+    __shared__ float smem[4];
+    const int64_t row = blockIdx.x;
+    const int64_t row_off = row * N, srow_off = row * (N / qb);
+    float x[ITERS][16];
+    float sum = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int col = (threadIdx.x + it * 256) * 16;
+        if (col < N) {
+            dequant16<KIND>(q, s, s_dt, row_off, srow_off, col, qb, x[it]);
+#pragma unroll
+            for (int i = 0; i < 16; i++) sum += x[it][i];
+        }
+    }
+    const float mean = block_sum_256(sum, smem) / (float)N;
+    float ss = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int col = (threadIdx.x + it * 256) * 16;
+        if (col < N) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float d = x[it][i] - mean;
+                ss += d * d;
+            }
+        }
+    }
+    const float var = block_sum_256(ss, smem) / (float)N;
+    const float rstd = 1 / sqrtf(var + eps);
+    float amax = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITERS; it++) {
+        const int col = (threadIdx.x + it * 256) * 16;
+        if (col < N) {
+            float wv[16], bv[16], yv[16];
+            if (WMODE != kNoParam) {
+                load_wb16<WMODE>(w, col, wv);
+                load_wb16<WMODE>(b, col, bv);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                float v = (x[it][i] - mean) * rstd;
+                if (WMODE != kNoParam) v = v * wv[i] + bv[i];
+                yv[i] = v;
+                amax = fmaxf(amax, fabsf(v));
+            }
+            float4* dst = (float4*)(y + row_off + col);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[i] = make_float4(yv[4 * i], yv[4 * i + 1], yv[4 * i + 2], yv[4 * i + 3]);
+        }
+    }
+    amax = block_max_256(amax, smem);
+    if (threadIdx.x == 0) {
+        const float sr = group_scale<KIND>(amax);
+        ((uint16_t*)s_row)[row] = (uint16_t)f2bf16(sr);
+        mean_out[row] = mean;
+        rstd_out[row] = rstd;
+        atomic_max_nonneg(s_max, sr);
+    }
+}
+
+// Backward: wdy = w * dy; dx = bf16((wdy - (xhat * mean(xhat * wdy) + mean(wdy))) * rstd);
+// per-block partials of dw = sum_rows dy * xhat and db = sum_rows dy (affine variant only).
+template <int KIND, int WMODE, int ITERS>
+__global__ __launch_bounds__(256) void k_layernorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                        const void* __restrict__ dy, const void* __restrict__ w,
+                                                        const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+                                                        void* __restrict__ dx, float* __restrict__ dw_partial,
+                                                        float* __restrict__ db_partial, int64_t M, int N, int qb) {
+    __shared__ float smem[4];
+    constexpr bool kAffine = WMODE != kNoParam;
+    float accw[kAffine ? ITERS : 1][16], accb[kAffine ? ITERS : 1][16];
+    if (kAffine) {
+#pragma unroll
+        for (int it = 0; it < ITERS; it++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) accw[it][i] = accb[it][i] = 0.0f;
+    }
+    for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+        const int64_t row_off = row * N, srow_off = row * (N / qb);
+        const float mean = mean_in[row], rstd = rstd_in[row];
+        float xhat[ITERS][16], wdy[ITERS][16];
+        float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+            const int col = (threadIdx.x + it * 256) * 16;
+            if (col < N) {
+                float xv[16], wv[16], gv[16];
+                dequant16<KIND>(q, s, s_dt, row_off, srow_off, col, qb, xv);
+                load_wb16<WMODE>(w, col, wv);
+                load_bf16_16(dy, row_off + col, gv);
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    xhat[it][i] = (xv[i] - mean) * rstd;
+                    wdy[it][i] = kAffine ? wv[i] * gv[i] : gv[i];
+                    dot += xhat[it][i] * wdy[it][i];
+                    sum += wdy[it][i];
+                    if (kAffine) {
+                        accw[it][i] += gv[i] * xhat[it][i];
+                        accb[it][i] += gv[i];
+                    }
+                }
+            }
+        }
+        const float c1 = block_sum_256(dot, smem) / (float)N;
+        const float c2 = block_sum_256(sum, smem) / (float)N;
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+            const int col = (threadIdx.x + it * 256) * 16;
+            if (col < N) {
+                float o[16];
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[i] = (wdy[it][i] - (xhat[it][i] * c1 + c2)) * rstd;
+                store_bf16_16(dx, row_off + col, o);
+            }
+        }
+    }
+    if (kAffine) {
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+            const int col = (threadIdx.x + it * 256) * 16;
+            if (col < N) {
+                float4* dw = (float4*)(dw_partial + (int64_t)blockIdx.x * N + col);
+                float4* db = (float4*)(db_partial + (int64_t)blockIdx.x * N + col);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    dw[i] = make_float4(accw[it][4 * i], accw[it][4 * i + 1], accw[it][4 * i + 2], accw[it][4 * i + 3]);
+                    db[i] = make_float4(accb[it][4 * i], accb[it][4 * i + 1], accb[it][4 * i + 2], accb[it][4 * i + 3]);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace coat
+
+using namespace coat;
+
+static int ln_check(int64_t M, int64_t N, int QB) {
+    if (M < 0 || N < 0) return COAT_EINVAL;
+    if (QB < 16 || (QB & (QB - 1)) || N % QB != 0 || N % 16 != 0) return COAT_ESHAPE;
+    if (N > 16384) return COAT_ESHAPE;  // a row is held in registers: 4 chunks of 16 per lane at most
+    return COAT_OK;
+}
+
+// w_dtype < 0: no affine parameters
+#define LN_CASE(KERNEL, GRID, K, W, I, ...)                                                           \
+    case ((K * 4 + W) * 3 + (I == 1 ? 0 : (I == 2 ? 1 : 2))):                                          \
+        hipLaunchKernelGGL((KERNEL<K, W, I>), dim3((unsigned)(GRID)), dim3(256), 0, st, __VA_ARGS__);  \
+        break;
+#define LN_CASES_W(KERNEL, GRID, K, W, ...) \
+    LN_CASE(KERNEL, GRID, K, W, 1, __VA_ARGS__) LN_CASE(KERNEL, GRID, K, W, 2, __VA_ARGS__) LN_CASE(KERNEL, GRID, K, W, 4, __VA_ARGS__)
+#define LN_CASES_K(KERNEL, GRID, K, ...)                                                          \
+    LN_CASES_W(KERNEL, GRID, K, 0, __VA_ARGS__) LN_CASES_W(KERNEL, GRID, K, 1, __VA_ARGS__)       \
+    LN_CASES_W(KERNEL, GRID, K, 2, __VA_ARGS__) LN_CASES_W(KERNEL, GRID, K, 3, __VA_ARGS__)
+#define LN_DISPATCH(KERNEL, GRID, ...)                                                            \
+    {                                                                                             \
+        const int iters = N <= 4096 ? 1 : (N <= 8192 ? 2 : 4);                                    \
+        const int wmode = w_dtype < 0 ? kNoParam : w_dtype;                                       \
+        if (fp8 != COAT_E4M3 && fp8 != COAT_E5M2) return COAT_EINVAL;                             \
+        if (wmode > kNoParam) return COAT_EDTYPE;                                                 \
+        switch ((fp8 * 4 + wmode) * 3 + (iters == 1 ? 0 : (iters == 2 ? 1 : 2))) {                \
+            LN_CASES_K(KERNEL, GRID, 0, __VA_ARGS__)                                              \
+            LN_CASES_K(KERNEL, GRID, 1, __VA_ARGS__)                                              \
+            default: return COAT_EINVAL;                                                          \
+        }                                                                                         \
+    }
+
+extern "C" int coat_fp8_layernorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w,
+                                          const void* b, int w_dtype, float* y, void* s_row, float* mean, float* rstd,
+                                          float* s_max, int64_t M, int64_t N, int QB, float eps, void* stream) {
+    if (int e = ln_check(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !s_x || !y || !s_row || !mean || !rstd || !s_max) return COAT_EINVAL;
+    if (w_dtype >= 0 && (!w || !b)) return COAT_EINVAL;
+    if (s_dtype < 0 || s_dtype > 2) return COAT_EDTYPE;
+    if (!coat_aligned16(x) || !coat_aligned16(y) || !coat_aligned16(w) || !coat_aligned16(b)) return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    LN_DISPATCH(k_layernorm_fwd, M, (const uint8_t*)x, s_x, s_dtype, w, b, y, s_row, mean, rstd, s_max, (int)N, QB, eps)
+    return coat_launch_status();
+}
+
+extern "C" int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
+                                           const void* w, int w_dtype, const float* mean, const float* rstd, void* dx,
+                                           void* dw, void* db, float* dw_partial, float* db_partial, int n_partial,
+                                           int64_t M, int64_t N, int QB, void* stream) {
+    if (int e = ln_check(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (!x || !s_x || !dy || !mean || !rstd || !dx) return COAT_EINVAL;
+    if (w_dtype >= 0 && (!w || !dw || !db || !dw_partial || !db_partial || n_partial <= 0)) return COAT_EINVAL;
+    if (s_dtype < 0 || s_dtype > 2) return COAT_EDTYPE;
+    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(dy) || !coat_aligned16(dx) ||
+        !coat_aligned16(dw_partial) || !coat_aligned16(db_partial))
+        return COAT_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    int64_t grid = w_dtype >= 0 ? (n_partial < M ? n_partial : M) : (M < 2048 ? M : 2048);
+    LN_DISPATCH(k_layernorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, mean, rstd, dx, dw_partial, db_partial, M, (int)N, QB)
+    if (int e = coat_launch_status()) return e;
+    if (w_dtype < 0) return COAT_OK;
+    const int cols_blocks = (int)((N + 31) / 32);
+    switch (w_dtype) {
+        case COAT_F32:
+            hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(256), 0, st, db_partial, db, (int)grid, (int)N);
+            break;
+        case COAT_BF16:
+            hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(256), 0, st, db_partial, db, (int)grid, (int)N);
+            break;
+        default:
+            hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(256), 0, st, db_partial, db, (int)grid, (int)N);
+            break;
+    }
+    return coat_launch_status();
+}

@@ -11,71 +11,10 @@
 // partial row; a second kernel sums the partials in block order.
 #include <math.h>
 
-#include "coat_device.h"
 #include "coat_host.h"
+#include "norm_common.h"
 
 namespace coat {
-
-__device__ __forceinline__ float block_sum_256(float v, float* smem) {
-    v = cluster_sum<64>(v);
-    const int wave = threadIdx.x >> 6;
-    __syncthreads();  // smem may still be read from a previous call
-    if ((threadIdx.x & 63) == 0) smem[wave] = v;
-    __syncthreads();
-    return ((smem[0] + smem[1]) + smem[2]) + smem[3];
-}
-__device__ __forceinline__ float block_max_256(float v, float* smem) {
-    v = cluster_max<64>(v);
-    const int wave = threadIdx.x >> 6;
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) smem[wave] = v;
-    __syncthreads();
-    return fmaxf(fmaxf(smem[0], smem[1]), fmaxf(smem[2], smem[3]));
-}
-
-template <int KIND> __device__ __forceinline__ void dequant16(const uint8_t* q, const void* s, int s_dt, int64_t row_off,
-                                                             int64_t srow_off, int col, int qb, float* v) {
-    uint4 c = *(const uint4*)(q + row_off + col);
-    float sc;
-    const int64_t si = srow_off + col / qb;
-    if (s_dt == kBF16) sc = u2f((uint32_t)((const uint16_t*)s)[si] << 16);
-    else if (s_dt == kF32) sc = ((const float*)s)[si];
-    else sc = f16lo(((const uint16_t*)s)[si]);
-    uint32_t w[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        float f[4];
-        fp8x4_to_f32<KIND>(w[k], f);
-#pragma unroll
-        for (int i = 0; i < 4; i++) v[4 * k + i] = f[i] * sc;
-    }
-}
-template <int WDT> __device__ __forceinline__ void load_w16(const void* w, int col, float* o) {
-    if (WDT == kF32) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float4 t = ((const float4*)((const float*)w + col))[i];
-            o[4 * i] = t.x; o[4 * i + 1] = t.y; o[4 * i + 2] = t.z; o[4 * i + 3] = t.w;
-        }
-    } else {
-        const uint4* src = (const uint4*)((const uint16_t*)w + col);
-        uint4 a = src[0], b = src[1];
-        uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            o[2 * k] = WDT == kBF16 ? bf16lo(u[k]) : f16lo(u[k]);
-            o[2 * k + 1] = WDT == kBF16 ? bf16hi(u[k]) : f16hi(u[k]);
-        }
-    }
-}
-__device__ __forceinline__ void store_bf16_16(void* p, int64_t off, const float* v) {
-    uint32_t w[8];
-#pragma unroll
-    for (int k = 0; k < 8; k++) w[k] = pack_bf16x2(v[2 * k], v[2 * k + 1]);
-    uint4* dst = (uint4*)((uint16_t*)p + off);
-    dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
-    dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
-}
 
 // Forward: y = bf16(x * rstd * w), rstd[row], row scale (max|y| + 1e-10)/fp8max (bf16), tensor max of the row scales.
 template <int KIND, int WDT, int ITERS>
@@ -189,34 +128,6 @@ __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__
     }
 }
 
-// dw[col] = sum over blocks (in block order) of the partials, stored in the weight's dtype.
-template <int WDT>
-__global__ __launch_bounds__(256) void k_rmsnorm_dw(const float* __restrict__ partial, void* __restrict__ dw, int nblocks,
-                                                     int N) {
-    // 32 columns per block, the partial rows split over 8 thread slices (fixed order: deterministic), 8 loads in flight
-    __shared__ float red[8][32];
-    const int c = threadIdx.x & 31, slice = threadIdx.x >> 5;
-    const int col = blockIdx.x * 32 + c;
-    float acc[8];
-#pragma unroll
-    for (int u = 0; u < 8; u++) acc[u] = 0.0f;
-    if (col < N) {
-        for (int b0 = slice * 8; b0 < nblocks; b0 += 64) {
-#pragma unroll
-            for (int u = 0; u < 8; u++)
-                if (b0 + u < nblocks) acc[u] += partial[(int64_t)(b0 + u) * N + col];
-        }
-    }
-    red[slice][c] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
-    __syncthreads();
-    if (slice == 0 && col < N) {
-        float s = 0.0f;
-#pragma unroll
-        for (int k = 0; k < 8; k++) s += red[k][c];
-        store_from_f32<WDT>(dw, col, s);
-    }
-}
-
 }  // namespace coat
 
 using namespace coat;
@@ -276,9 +187,9 @@ extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x
     if (int e = coat_launch_status()) return e;
     const int cols_blocks = (int)((N + 31) / 32);
     switch (w_dtype) {
-        case COAT_F32: hipLaunchKernelGGL((k_rmsnorm_dw<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
-        case COAT_BF16: hipLaunchKernelGGL((k_rmsnorm_dw<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
-        default: hipLaunchKernelGGL((k_rmsnorm_dw<kF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        case COAT_F32: hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        case COAT_BF16: hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        default: hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
     }
     return coat_launch_status();
 }

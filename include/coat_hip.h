@@ -118,6 +118,22 @@ int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dty
                               int w_dtype, const float* rstd, void* dx, void* dw, float* dw_partial, int n_partial,
                               int64_t M, int64_t N, int QB, void* stream);
 
+/* rq/func_layernorm_noparam.py:193 fp8_layernorm_noparam_forward (kernel :53-115) and rq/func_layernorm_param.py:258
+ * fp8_layernorm_param_forward (kernel :51-125): y fp32 [M,N] = (x - mean) * rstd (* w + b); mean, rstd [M] fp32;
+ * s_row [M] bf16 row scales (max|y| + 1e-10) / fp8max; s_max as above.  w_dtype < 0: no affine parameters (w, b
+ * ignored); otherwise w and b share that dtype.  N <= 16384, N % 16 == 0. */
+int coat_fp8_layernorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, const void* b,
+                               int w_dtype, float* y, void* s_row, float* mean, float* rstd, float* s_max, int64_t M,
+                               int64_t N, int QB, float eps, void* stream);
+/* rq/func_layernorm_noparam.py:250 fp8_layernorm_noparam_backward (kernel :125-190) and
+ * rq/func_layernorm_param.py:309 fp8_layernorm_param_backward (kernels :134-226, :229-255): dx bf16 [M,N]; with
+ * parameters also dw, db [N] in w's dtype through the caller-provided fp32 workspaces dw_partial, db_partial
+ * [n_partial, N] (summed in block order; the reference accumulates under a spin lock in w's dtype). */
+int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* w,
+                                int w_dtype, const float* mean, const float* rstd, void* dx, void* dw, void* db,
+                                float* dw_partial, float* db_partial, int n_partial, int64_t M, int64_t N, int QB,
+                                void* stream);
+
 /* ---- GEMM -------------------------------------------------------------------------------------------
  * rq/linear.py:172 fp8matmul (kernel :61-169): C[M,N] = (A[M,K] . B[N,K]^T) * (float(*scale_a) * float(*scale_b))
  * (+ bias[N]), fp32 accumulation on FP8 MFMA.  A and B are row-major with K contiguous (the reference passes B as

@@ -305,6 +305,51 @@ def fp8_rmsnorm_backward(q, s, g, w, rstd, QB, accumulate=torch.float64):
     return dx, dw
 
 
+# ----------------------------------------------------------------------------- LayerNorm
+def layernorm_forward_value(q, s, QB, eps, w=None, b=None, accumulate=torch.float32):
+    """rq/func_layernorm_noparam.py:86-104 / rq/func_layernorm_param.py:85-107: x = dequant; mean = sum(x)/N;
+    var = sum((x-mean)^2)/N; rstd = 1/sqrt(var+eps); y = (x-mean)*rstd (* w + b), all fp32."""
+    x = _dequant32(q, s, QB)
+    N = x.shape[1]
+    mean = (x.to(accumulate).sum(dim=1) / N).float()
+    d = x - mean.unsqueeze(1)
+    var = ((d * d).to(accumulate).sum(dim=1) / N).float()
+    rstd = 1.0 / torch.sqrt(var + eps)
+    y = d * rstd.unsqueeze(1)
+    if w is not None:
+        y = y * w.float().unsqueeze(0) + b.float().unsqueeze(0)
+    return y, mean, rstd
+
+
+def fp8_layernorm_forward(q, s, QB, eps, w=None, b=None, accumulate=torch.float32):
+    """rq/func_layernorm_noparam.py:193-247 / rq/func_layernorm_param.py:258-306: the normalised tensor stays fp32
+    (:205), row scale (max|y|+1e-10)/fp8max stored bf16 (:106-112), max over rows, division+transpose of the fp32 y."""
+    y, mean, rstd = layernorm_forward_value(q, s, QB, eps, w, b, accumulate)
+    s_row = ((y.abs().amax(dim=1) + SCALE_MIN_THRES) / FP8_MAX_VALUE[q.dtype]).to(torch.bfloat16)
+    qy, s_pt, qy_t = fp8_division_transpose(y, QB, q.dtype, s_row.max())
+    return qy, s_pt, qy_t, mean, rstd
+
+
+def fp8_layernorm_backward(q, s, g, mean, rstd, QB, w=None, accumulate=torch.float64):
+    """rq/func_layernorm_noparam.py:164-190 / rq/func_layernorm_param.py:186-226, :229-255:
+    wdy = w*dy (dy without parameters); c1 = sum(xhat*wdy)/N; c2 = sum(wdy)/N; dx = (wdy - (xhat*c1 + c2))*rstd -> bf16;
+    dw = sum_rows(dy*xhat), db = sum_rows(dy) (the reference accumulates them under a lock in w's dtype; stated here is
+    the float64 sum rounded once)."""
+    x = _dequant32(q, s, QB)
+    N = x.shape[1]
+    dy = g.float()
+    xhat = (x - mean.float().unsqueeze(1)) * rstd.float().unsqueeze(1)
+    wdy = dy if w is None else w.float().unsqueeze(0) * dy
+    c1 = ((xhat * wdy).to(accumulate).sum(dim=1) / N).float()
+    c2 = (wdy.to(accumulate).sum(dim=1) / N).float()
+    dx = ((wdy - (xhat * c1.unsqueeze(1) + c2.unsqueeze(1))) * rstd.float().unsqueeze(1)).to(torch.bfloat16)
+    if w is None:
+        return dx
+    dw = (dy * xhat).to(accumulate).sum(dim=0).to(w.dtype)
+    db = dy.to(accumulate).sum(dim=0).to(w.dtype)
+    return dx, dw, db
+
+
 # ----------------------------------------------------------------------------- the reference tests' own definition
 def quantize_tensor_ref_test(x, QB, fp8type):
     """tests/test_utils.py:61-67 ("per_group"): scale = bf16(amax / fp8max) (no 1e-10), and the

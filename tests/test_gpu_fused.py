@@ -141,6 +141,46 @@ def test_rmsnorm_forward_backward(dev, N):
     assert torch.equal(dw, dw2) and torch.equal(dx, dx2)
 
 
+@pytest.mark.parametrize("N,affine", [(2048, False), (5120, False), (4096 + 1024 * 8, False), (2048, True), (5120, True)])
+def test_layernorm_forward_backward(dev, N, affine):
+    rq = _rq()
+    M = 512
+    x, g = rand(20, shape=(M, N)) + 0.25, rand(21, 0.01, shape=(M, N))
+    w = (1 + 0.1 * torch.randn(N, generator=torch.Generator().manual_seed(22))).bfloat16() if affine else None
+    bb = (0.1 * torch.randn(N, generator=torch.Generator().manual_seed(23))).bfloat16() if affine else None
+    q, s = pg(x)
+    if affine:
+        qy, spt, qyt, (w_, b_, mean, rstd, nw) = rq.fp8_layernorm_param_forward(q.to(dev), s.to(dev), w.to(dev), bb.to(dev), QB, 1e-5)
+    else:
+        qy, spt, qyt, (mean, rstd, nw) = rq.fp8_layernorm_noparam_forward(q.to(dev), s.to(dev), QB, 1e-5)
+    wq, wspt, wqt, wmean, wrstd = R.fp8_layernorm_forward(q, s, QB, 1e-5, w, bb, accumulate=torch.float64)
+    assert torch.allclose(mean.cpu(), wmean, rtol=1e-5, atol=1e-7)
+    assert torch.allclose(rstd.cpu(), wrstd, rtol=2e-6, atol=0)
+    assert spt.item() == wspt.item()
+    codes_close(qy, wq, 2e-3)
+    assert torch.equal(b(qyt), b(qy).t())
+    if affine:
+        dx, dw, db = rq.fp8_layernorm_param_backward(q.to(dev), s.to(dev), g.to(dev), QB, w.to(dev), bb.to(dev), mean, rstd, nw)
+        wdx, wdw, wdb = R.fp8_layernorm_backward(q, s, g, wmean, wrstd, QB, w)
+        assert dw.dtype == w.dtype and torch.allclose(dw.cpu().float(), wdw.float(), rtol=1e-2, atol=1e-3)
+        assert db.dtype == w.dtype and torch.allclose(db.cpu().float(), wdb.float(), rtol=1e-2, atol=1e-3)
+        dx2, dw2, db2 = rq.fp8_layernorm_param_backward(q.to(dev), s.to(dev), g.to(dev), QB, w.to(dev), bb.to(dev), mean, rstd, nw)
+        assert torch.equal(dw, dw2) and torch.equal(db, db2) and torch.equal(dx, dx2)
+    else:
+        dx = rq.fp8_layernorm_noparam_backward(q.to(dev), s.to(dev), g.to(dev), QB, mean, rstd, nw)
+        wdx = R.fp8_layernorm_backward(q, s, g, wmean, wrstd, QB)
+    # dx = (wdy - (xhat*c1 + c2))*rstd cancels: where the result is below 2^-12 of the tensor's largest gradient the
+    # fp32 summation order of c1 / c2 decides its bits, so those elements are held to that absolute bound instead
+    big = wdx.float().abs().max()
+    small = (wdx.float().abs() < big * 2.0 ** -12) & (dx.cpu().float().abs() < big * 2.0 ** -12)
+    bf16_close(torch.where(small.to(dev), torch.zeros_like(dx), dx), torch.where(small, torch.zeros_like(wdx), wdx), 5e-3, max_ulp=4)
+    # batched input keeps its leading dimensions
+    q3, s3 = q.reshape(4, M // 4, N).to(dev), s.reshape(4, M // 4, N // QB).to(dev)
+    if not affine:
+        qy3, spt3, qyt3, _ = rq.fp8_layernorm_noparam_forward(q3, s3, QB, 1e-5, transpose_output_2d=True)
+        assert qy3.shape == (4, M // 4, N) and qyt3.shape == (N, M) and torch.equal(b(qy3).reshape(M, N), b(qy))
+
+
 def test_larger_groups_and_float32_scales(dev):
     rq = _rq()
     x1, x2 = rand(13, shape=(128, 512)), rand(14, shape=(128, 512))

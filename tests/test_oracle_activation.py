@@ -193,3 +193,32 @@ def test_rmsnorm_against_functional_and_autograd():
     assert spt.item() == ((v.abs().max() + 1e-10) / 448).bfloat16().item()
     assert torch.equal(qy.view(torch.uint8), R.cast_fp8(v.bfloat16().float() / spt.float(), E4).view(torch.uint8))
     assert torch.equal(qyt.view(torch.uint8), qy.view(torch.uint8).t())
+
+
+@pytest.mark.parametrize("affine", [False, True])
+def test_layernorm_against_functional_and_autograd(affine):
+    M, N = 48, 256
+    x = _x(M, N, 22, outliers=False) + 0.3  # a non-zero mean, so that forgetting the mean subtraction shows
+    g = _x(M, N, 23, outliers=False) * 0.01
+    w = (1 + 0.1 * _x(1, N, 24, outliers=False).float()).reshape(N).bfloat16() if affine else None
+    bb = (0.1 * _x(1, N, 25, outliers=False).float()).reshape(N).bfloat16() if affine else None
+    q, s = _pg(x)
+    xd = R._dequant32(q, s, 16).double().requires_grad_(True)
+    wd = w.double().requires_grad_(True) if affine else None
+    bd = bb.double().requires_grad_(True) if affine else None
+    ref = F.layer_norm(xd, (N,), wd, bd, 1e-5)
+    v, mean, rstd = R.layernorm_forward_value(q, s, 16, 1e-5, w, bb)
+    assert torch.allclose(v.double(), ref.detach(), rtol=2e-6, atol=2e-7)
+    assert torch.allclose(mean.double(), xd.detach().mean(dim=1), rtol=1e-5, atol=1e-7)
+    assert torch.allclose(rstd.double(), (xd.detach().var(dim=1, unbiased=False) + 1e-5).rsqrt(), rtol=1e-6)
+    ref.backward(g.double())
+    out = R.fp8_layernorm_backward(q, s, g, mean, rstd, 16, w)
+    dx = out[0] if affine else out
+    assert (dx.double() - xd.grad).abs().max() <= xd.grad.abs().max() * 2.0 ** -8
+    if affine:
+        assert torch.allclose(out[1].double(), wd.grad, rtol=1e-2, atol=1e-4) and out[1].dtype == w.dtype
+        assert torch.allclose(out[2].double(), bd.grad, rtol=1e-2, atol=1e-4) and out[2].dtype == w.dtype
+    qy, spt, qyt, _, _ = R.fp8_layernorm_forward(q, s, 16, 1e-5, w, bb)
+    assert spt.item() == ((v.abs().max() + 1e-10) / 448).bfloat16().item()
+    assert torch.equal(qy.view(torch.uint8), R.cast_fp8(v / spt.float(), E4).view(torch.uint8))  # divides the fp32 y
+    assert torch.equal(qyt.view(torch.uint8), qy.view(torch.uint8).t())
