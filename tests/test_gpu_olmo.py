@@ -1,0 +1,127 @@
+"""GPU: CoatOLMoSequentialBlock forward + backward, held to the same bars as the Llama decoder layer
+(tests/test_gpu_layer.py): forward within 5 % (relative Frobenius) of the CPU oracle chained through the same FP8
+quantization points, forward and every gradient within 12 % of the same block differentiated in fp32 torch."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+
+def build(dev, D=512, heads=8, I=1536, memory_efficient=True, seed=0):
+    from coat_amd.models.coat_olmo import CoatOLMoConfig, CoatOLMoSequentialBlock
+    torch.manual_seed(seed)
+    cfg = CoatOLMoConfig(d_model=D, n_heads=heads, mlp_hidden_size=2 * I,
+                         coat_fp8_args={"weight_memory_efficient": memory_efficient})
+    blk = CoatOLMoSequentialBlock(0, cfg)
+    for p in blk.parameters():
+        torch.nn.init.normal_(p, std=0.02)
+    return blk.to(dev).to(torch.bfloat16), cfg
+
+
+def attention(q, k, v, nh):
+    from coat_amd.models.coat_llama import apply_rotary_pos_emb, rotary_cos_sin
+    B, S, D = q.shape
+    hd = D // nh
+    q, k, v = (t.view(B, S, nh, hd).transpose(1, 2) for t in (q, k, v))
+    cos, sin = rotary_cos_sin(torch.arange(S, device=q.device).unsqueeze(0), hd, 10000.0, torch.float32)
+    q, k = apply_rotary_pos_emb(q.float(), k.float(), cos, sin)
+    return F.scaled_dot_product_attention(q.to(v.dtype), k.to(v.dtype), v, is_causal=True).transpose(1, 2).reshape(B, S, D)
+
+
+def reference_block(blk, x, dtype=torch.float32):
+    W = {n: p.detach().to(dtype).requires_grad_(True) for n, p in blk.named_parameters()}
+    x = x.detach().to(dtype).requires_grad_(True)
+    D = x.shape[-1]
+    h = F.layer_norm(x, (D,), None, None, 1e-5)
+    q, k, v = (h @ W["BeforeAttention.att_proj.weight"].t()).split(blk.fused_dims, dim=-1)
+    a = attention(q, k, v, blk.config.n_heads)
+    x1 = x + a @ W["AfterAttention.attn_out.weight"].t()
+    up, gate = (F.layer_norm(x1, (D,), None, None, 1e-5) @ W["MLPResidual.ff_proj.weight"].t()).chunk(2, dim=-1)
+    y = x1 + (F.silu(gate) * up) @ W["MLPResidual.ff_out.weight"].t()
+    return x, y, W
+
+
+def rel(a, b):
+    return ((a.float().cpu() - b.float().cpu()).norm() / b.float().cpu().norm()).item()
+
+
+def oracle_block_forward(blk, x):
+    """coat_olmo.py:160-207, :310-345, :480-555 restated with oracle/activation_ref.py on the CPU."""
+    from oracle import activation_ref as R
+    W = {n: p.detach().cpu() for n, p in blk.named_parameters()}
+    B, S, D = x.shape
+    QB = 16
+    x2 = x.detach().cpu().reshape(-1, D)
+
+    def wq(name):
+        return R.fp8_division(W[name], QB, "E4M3")
+
+    qx, sx = R.fp8_quantize(x2, QB, "E4M3")
+    ln_x, ln_s, _, _, _ = R.fp8_layernorm_forward(qx, sx, QB, 1e-5, accumulate=torch.float64)
+    w8, ws = wq("BeforeAttention.att_proj.weight")
+    qkv = R.fp8_linear_forward(ln_x, ln_s, w8, ws, False, QB).float().reshape(B, S, -1)
+    q, k, v = qkv.split(blk.fused_dims, dim=-1)
+    attn = attention(q, k, v, blk.config.n_heads).reshape(B * S, D).bfloat16()
+    fq, fs, _ = R.fp8_quantize_pertensor(attn, QB, "E4M3")
+    w8, ws = wq("AfterAttention.attn_out.weight")
+    h1, (q1, s1) = R.fp8_add_Ifp_Ifp_Ofp_Og16(x2, R.fp8_linear_forward(fq, fs, w8, ws, False, QB), torch.float8_e4m3fn, QB)
+    ln_x, ln_s, _, _, _ = R.fp8_layernorm_forward(q1, s1, QB, 1e-5, accumulate=torch.float64)
+    w8, ws = wq("MLPResidual.ff_proj.weight")
+    fc1_x, fc1_s = R.fp8matmul(ln_x, w8.t(), True, ln_s, ws, QB, accumulate=torch.float64)
+    up_x, gate_x = (t.contiguous() for t in fc1_x.chunk(2, dim=-1))
+    up_s, gate_s = (t.contiguous() for t in fc1_s.chunk(2, dim=-1))
+    silu_x, silu_s = R.fp8_silu_forward(gate_x, gate_s, QB)
+    mul_x, mul_s, _ = R.fp8_mul_forward(silu_x, silu_s, up_x, up_s, QB)
+    w8, ws = wq("MLPResidual.ff_out.weight")
+    h2, (q2, s2) = R.fp8_add_Ifp_Ifp_Ofp_Og16(h1, R.fp8_linear_forward(mul_x, mul_s, w8, ws, False, QB), torch.float8_e4m3fn, QB)
+    return h2.reshape(B, S, D), q2.reshape(B, S, D), s2.reshape(B, S, D // QB)
+
+
+@pytest.mark.parametrize("memory_efficient", [True, False])
+def test_olmo_block_forward_backward(dev, memory_efficient):
+    from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
+    from coat_amd.utils._fp8manager import FP8Manager
+    from oracle import activation_ref as R
+    blk, cfg = build(dev, memory_efficient=memory_efficient)
+    blk.train()
+    B, S, D = 2, 128, cfg.d_model
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(B, S, D, generator=g).bfloat16().to(dev)
+    gy = (torch.randn(B, S, D, generator=g) * 1e-2).bfloat16().to(dev)
+    bgn, end = Coat_quantize_bgn(blk.qargs).to(dev), Coat_quantize_end(blk.qargs).to(dev)
+
+    FP8Manager.is_first_microbatch = True
+    xin = x.clone().requires_grad_(True)
+    h, qh, sh = bgn(xin)
+    h, qh, sh, cache = blk(h, qh, sh)
+    assert cache is None and h.dtype == torch.bfloat16 and qh.dtype == torch.float8_e4m3fn and sh.shape == (B, S, D // 16)
+    y = end(h, qh, sh)
+    y.backward(gy)
+
+    xr, yr, W = reference_block(blk, x)
+    yr.backward(gy.float())
+    oh, oq, osc = oracle_block_forward(blk, x)
+    assert rel(y.detach().cpu() - x.cpu(), oh - x.cpu()) < 0.05
+    deq_gpu = R.fp8_dequantize(qh.detach().cpu().reshape(-1, D), sh.detach().cpu().reshape(-1, D // 16), 16)
+    deq_cpu = R.fp8_dequantize(oq.reshape(-1, D), osc.reshape(-1, D // 16), 16)
+    assert rel(deq_gpu, deq_cpu) < 0.05
+    assert rel(deq_gpu, h.detach().reshape(-1, D)) < 0.04
+    assert rel(y.detach() - x, yr.detach() - x.float()) < 0.12
+    assert rel(xin.grad, xr.grad) < 0.12
+    for n, p in blk.named_parameters():
+        assert p.grad is not None, n
+        assert rel(p.grad, W[n].grad) < 0.12, (n, rel(p.grad, W[n].grad))
+
+    # second micro-batch with cached weight scales / FP8 weights: identical result
+    FP8Manager.is_first_microbatch = False
+    blk.zero_grad()
+    h2, qh2, sh2 = bgn(x.clone().requires_grad_(True))
+    h2, qh2, sh2, _ = blk(h2, qh2, sh2)
+    assert torch.equal(h2, h) and torch.equal(qh2.view(torch.uint8), qh.view(torch.uint8))
+    FP8Manager.is_first_microbatch = True
+
+    blk.eval()
+    with torch.no_grad():
+        he, qe, se, _ = blk(x, None, None)
+    assert qe is None and rel(he, yr.detach()) < 0.02
