@@ -296,8 +296,7 @@ __global__ __launch_bounds__(256) void k_division_transpose(const void* __restri
 template <int XDT, int SDT, int KIND, int QB, int TM>
 __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restrict__ x, void* __restrict__ q,
                                                              void* __restrict__ s_out, void* __restrict__ qt,
-                                                             void* __restrict__ st_out, int64_t M, int64_t N,
-                                                             int tiles_per_block) {
+                                                             void* __restrict__ st_out, int64_t M, int64_t N) {
     constexpr int VEC = VecOf<XDT>::kVec;
     constexpr int ESIZE = 16 / VEC;
     constexpr int LPG = QB / VEC;
@@ -307,11 +306,16 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
     enable_fp8_saturation();
     const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = (N + kTileN - 1) / kTileN;
     const int64_t SN = N / QB, SM = M / QB;
-    // A block walks a contiguous range of tile ids; ids run down a 64-column strip (m fastest), so the 8-byte pieces
-    // of transposed scales and the 64-byte pieces of transposed codes that consecutive tiles write are neighbours and
-    // merge in L2.  The next tile's input is fetched into registers before the barrier and lands during phase 2.
-    const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_block;
-    const int64_t t_end = min(t_begin + tiles_per_block, tiles_m * tiles_n);
+    // A block quantizes two tiles that are neighbours along n, so the two 64-byte halves of every 128-byte line of q
+    // come from the same CU within microseconds and merge in L2.  Blocks are dispatched round-robin over the 8 XCDs
+    // (block b runs on XCD b % 8): XCD x owns the tile-column pairs j = x (mod 8) and walks down m, so the 64-byte
+    // pieces of a q^T row written by vertically adjacent tiles meet in the same L2 as well.  The second tile's input
+    // is fetched into registers before the barrier and lands during phase 2 of the first.
+    const int64_t pair = ((int64_t)(blockIdx.x >> 3) / tiles_m) * 8 + (blockIdx.x & 7);
+    const int64_t tm = (int64_t)(blockIdx.x >> 3) % tiles_m;
+    if (2 * pair >= tiles_n) return;
+    const int64_t t_begin = 0, t_end = min((int64_t)2, tiles_n - 2 * pair);
+#define COAT_QT_ORIGIN(t) const int64_t m0 = tm * TM, n0 = (2 * pair + (t)) * kTileN
 
     // phase-1 jobs: VEC consecutive elements (16 bytes); a row of the tile is 64/VEC jobs (a multiple of LPG)
     constexpr int JPR = kTileN / VEC;
@@ -320,7 +324,7 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
     constexpr int NIT = JOBS / 256;
     uint4 raw[NIT];
     auto fetch = [&](int64_t t) {
-        const int64_t m0 = (t % tiles_m) * TM, n0 = (t / tiles_m) * kTileN;
+        COAT_QT_ORIGIN(t);
 #pragma unroll
         for (int it = 0; it < NIT; it++) {
             const int job = threadIdx.x + it * 256;
@@ -330,7 +334,7 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
     };
     if (t_begin < t_end) fetch(t_begin);
     for (int64_t t = t_begin; t < t_end; t++) {
-        const int64_t m0 = (t % tiles_m) * TM, n0 = (t / tiles_m) * kTileN;
+        COAT_QT_ORIGIN(t);
 #pragma unroll
         for (int it = 0; it < NIT; it++) {
             const int job = threadIdx.x + it * 256;
@@ -379,6 +383,7 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
         }
         __syncthreads();  // the tile is rewritten by the next iteration
     }
+#undef COAT_QT_ORIGIN
 }
 
 }  // namespace coat
@@ -560,13 +565,13 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
     if (QB > 64) return COAT_ESHAPE;  // column groups must fit the 64-wide tile
     hipStream_t st = (hipStream_t)stream;
     constexpr int TM = 64;
-    const int64_t ntiles = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
-    const int tiles_per_block = (int)((ntiles + 8191) / 8192);  // one tile per block up to 32 blocks per CU (measured faster than fewer, longer blocks)
-    const int64_t blocks = (ntiles + tiles_per_block - 1) / tiles_per_block;
+    const int64_t tiles_m = (M + TM - 1) / TM, pairs_n = ((N + kTileN - 1) / kTileN + 1) / 2;
+    const int64_t blocks = ((pairs_n + 7) / 8) * 8 * tiles_m;  // see the kernel for the block -> tile-pair mapping
+    if (blocks >= ((int64_t)1 << 31)) return COAT_ESHAPE;
 #define LAUNCH_QT(QBV)                                                                                               \
     DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                 \
         hipLaunchKernelGGL((k_quantize_transpose<XDT, SDT, KIND, QBV, TM>), dim3((unsigned)blocks), dim3(256), 0, st, \
-                           x, q, s, qt, st_out, M, N, tiles_per_block);                                              \
+                           x, q, s, qt, st_out, M, N);                                                               \
         return coat_launch_status();                                                                                 \
     })))
     switch (QB) {
