@@ -28,7 +28,7 @@ def adamw_bytes(numel):
     return numel * 16 + ngroups * 48
 
 
-def make_adamw_workload(dev, shape, torch):
+def make_adamw_workload(dev, shape, torch, expand=True):
     from coat_amd.optimizer import qoptim_cuda
 
     numel = shape[0] * shape[1]
@@ -49,12 +49,19 @@ def make_adamw_workload(dev, shape, torch):
 
     def step():
         state["step"] += 1
-        qoptim_cuda.fp8_adamw_expand_step(p, grads[state["step"] % len(grads)], *st, *hp, state["step"], 128, 16)
+        if expand:
+            qoptim_cuda.fp8_adamw_expand_step(p, grads[state["step"] % len(grads)], *st, *hp, state["step"], 128, 16)
+        else:  # the same step without Dynamic Range Expansion: codes and scales only
+            qoptim_cuda.fp8_adamw_step(p, grads[state["step"] % len(grads)], st[0], st[1], st[4], st[5], *hp,
+                                       state["step"], 128)
 
     for _ in range(9):  # steps 1..9: builds a realistic moment state (k, c per group), untimed
         step()
-    return step, adamw_bytes(numel), {"workload": "CoatAdamW.step fp32 [11008,4096], DRE on, step 10+, qgroup 128",
-                                      "numel": numel, "kernel": "k_fp8_adamw<f32,expand>"}
+    if expand:
+        return step, adamw_bytes(numel), {"workload": "CoatAdamW.step fp32 [11008,4096], DRE on, step 10+, qgroup 128",
+                                          "numel": numel, "kernel": "k_fp8_adamw_expand"}
+    return step, numel * 16 + ng * 16, {"workload": "CoatAdamW.step fp32 [11008,4096], DRE off, step 10+, qgroup 128",
+                                        "numel": numel, "kernel": "k_fp8_adamw_plain"}
 
 
 def make_quantize_workload(dev, torch, transpose):
@@ -347,7 +354,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="adamw", choices=["adamw", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
+    ap.add_argument("--workload", default="adamw", choices=["adamw", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
                              "silu_mul", "rmsnorm", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ramp-seconds", type=float, default=1.5,
@@ -376,8 +383,8 @@ def main():
     is_gemm = args.workload.startswith("gemm")
     if args.workload.startswith("layer") or args.workload == "linear":
         return bench_layer(args, dev, torch)
-    if args.workload == "adamw":
-        step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch)
+    if args.workload in ("adamw", "adamw_plain"):
+        step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch, expand=args.workload == "adamw")
     elif is_gemm:
         step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1])
     elif args.workload == "silu_mul":

@@ -183,12 +183,28 @@ __global__ __launch_bounds__(256) void k_fp8_adamw_plain(void* __restrict__ para
     // "+ 1e-20" is a double-precision add narrowed to float in the reference
     const float snew_m = (float)((double)mx_m + 1e-20) / 448.0f;
     const float snew_v = (float)((double)mx_v + 1e-20) / 448.0f;
+    // m / s and v / s: through the reciprocal with one correction step, which gives the same FP8 code as the IEEE
+    // quotient (every FP8 rounding boundary is a quotient the correction reproduces exactly); tiny scales, where the
+    // reciprocal would overflow, take the plain division (wave-uniform choice)
+    if (__all(snew_m >= kMinFastDivScale && snew_v >= kMinFastDivScale)) {
+        const float rm = 1.0f / snew_m, rv = 1.0f / snew_v;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        store_codes4(exp_avg, e0 + 32 * j, lim,
-                     cvt4_fp8<kE4M3>(m[j][0] / snew_m, m[j][1] / snew_m, m[j][2] / snew_m, m[j][3] / snew_m));
-        store_codes4(exp_avg_sq, e0 + 32 * j, lim,
-                     cvt4_fp8<kE4M3>(v[j][0] / snew_v, v[j][1] / snew_v, v[j][2] / snew_v, v[j][3] / snew_v));
+        for (int j = 0; j < 4; j++) {
+            store_codes4(exp_avg, e0 + 32 * j, lim,
+                         cvt4_fp8<kE4M3>(div_by_scale(m[j][0], snew_m, rm), div_by_scale(m[j][1], snew_m, rm),
+                                         div_by_scale(m[j][2], snew_m, rm), div_by_scale(m[j][3], snew_m, rm)));
+            store_codes4(exp_avg_sq, e0 + 32 * j, lim,
+                         cvt4_fp8<kE4M3>(div_by_scale(v[j][0], snew_v, rv), div_by_scale(v[j][1], snew_v, rv),
+                                         div_by_scale(v[j][2], snew_v, rv), div_by_scale(v[j][3], snew_v, rv)));
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            store_codes4(exp_avg, e0 + 32 * j, lim,
+                         cvt4_fp8<kE4M3>(m[j][0] / snew_m, m[j][1] / snew_m, m[j][2] / snew_m, m[j][3] / snew_m));
+            store_codes4(exp_avg_sq, e0 + 32 * j, lim,
+                         cvt4_fp8<kE4M3>(v[j][0] / snew_v, v[j][1] / snew_v, v[j][2] / snew_v, v[j][3] / snew_v));
+        }
     }
     if (gvalid && lam == 0) {
         scale_m[gi] = snew_m;
