@@ -200,17 +200,15 @@ class Bf16DecoderLayer:
 
     def __call__(self, x):
         import torch.nn.functional as F
-        from coat_amd.models.coat_llama import apply_rotary_pos_emb, rotary_cos_sin
+        from coat_amd.models.coat_llama import fused_rotary
         p, torch = self.p, self.torch
         B, S, H = x.shape
         hd = H // self.nh
         h = F.rms_norm(x, (H,), p["input_layernorm.weight"], 1e-5)
-        q = F.linear(h, p["BeforeAttention.q_proj.weight"]).view(B, S, self.nh, hd).transpose(1, 2)
-        k = F.linear(h, p["BeforeAttention.k_proj.weight"]).view(B, S, self.nh, hd).transpose(1, 2)
+        # the same fused RoPE kernel as the FP8 layer uses, so that the comparison is about the FP8 flow only
+        q = fused_rotary(F.linear(h, p["BeforeAttention.q_proj.weight"]), self.nh, hd, 10000.0)
+        k = fused_rotary(F.linear(h, p["BeforeAttention.k_proj.weight"]), self.nh, hd, 10000.0)
         v = F.linear(h, p["BeforeAttention.v_proj.weight"]).view(B, S, self.nh, hd).transpose(1, 2)
-        pos = torch.arange(S, device=x.device).unsqueeze(0).expand(B, -1)
-        cos, sin = rotary_cos_sin(pos, hd, 10000.0, x.dtype)
-        q, k = apply_rotary_pos_emb(q, k, cos, sin)
         a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, H)
         x1 = x + F.linear(a, p["AfterAttention.o_proj.weight"])
         h2 = F.rms_norm(x1, (H,), p["post_attention_layernorm.weight"], 1e-5)
@@ -242,12 +240,16 @@ def make_layer_workload(dev, torch, size):
     def step_fp8():
         FP8Manager.is_first_microbatch = state["first"]  # True once, then False (benchmark_llamalayer.py:185-191)
         state["first"] = False
+        for p in layer.parameters():
+            p.grad = None  # forward + backward only: no accumulation into an existing gradient
         xin = x.detach().requires_grad_(True)
         h, q, s = bgn(xin)
         (h, q, s), = layer(h, q, s)
         end(h, q, s).backward(gy)
 
     def step_bf16():
+        for p in ref.p.values():
+            p.grad = None
         xin = x.detach().requires_grad_(True)
         ref(xin).backward(gy)
 

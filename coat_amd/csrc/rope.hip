@@ -1,0 +1,66 @@
+// Rotary position embedding for the bf16 attention of the decoder layers, forward and backward in one pass each.
+//
+// The reference applies RoPE with separate torch kernels (transformers' apply_rotary_pos_emb as called from
+// coat/models/coat_llama.py:1029-1030; olmo's RotaryEmbedding from coat/models/coat_olmo.py:862-863): two multiplies, a
+// negate, a concatenation and an add per tensor and direction, each a full pass over q and k.  Here one streaming
+// kernel reads x once and writes the rotated tensor once; the backward pass is the same kernel with the angle negated.
+//   x, y: bf16 [rows, heads, head_dim] (rows = batch * seq, contiguous), "half" layout: element d pairs with d + head_dim/2
+//   cos_tab, sin_tab: fp32 [n_pos, head_dim/2];  position of a row = pos[row] if pos is given, else row % seq_len
+//   y1 = x1 cos - x2 sin,  y2 = x2 cos + x1 sin   (inverse: sin -> -sin), computed in fp32, rounded once to bf16.
+#include "coat_device.h"
+#include "coat_host.h"
+
+namespace coat {
+
+__global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab,
+                                                    const int64_t* __restrict__ pos, int64_t rows, int seq_len, int heads,
+                                                    int head_dim, float sign) {
+    const int half = head_dim >> 1;
+    const int cpr = half >> 3;                      // 16-byte chunks per half row
+    const int64_t total = rows * heads * cpr;       // one job = 8 pairs
+    for (int64_t job = (int64_t)blockIdx.x * 256 + threadIdx.x; job < total; job += (int64_t)gridDim.x * 256) {
+        const int c = (int)(job % cpr);
+        const int64_t rh = job / cpr;               // row * heads + head
+        const int64_t row = rh / heads;
+        const int64_t p = pos ? pos[row] : row % seq_len;
+        const uint16_t* src = x + rh * head_dim + c * 8;
+        const uint4 a = *(const uint4*)src, b = *(const uint4*)(src + half);
+        const float4* ct = (const float4*)(cos_tab + p * half + c * 8);
+        const float4* st = (const float4*)(sin_tab + p * half + c * 8);
+        const float4 c0 = ct[0], c1 = ct[1], s0 = st[0], s1 = st[1];
+        const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+        uint32_t o1[4], o2[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float x1l = bf16lo(aw[k]), x1h = bf16hi(aw[k]), x2l = bf16lo(bw[k]), x2h = bf16hi(bw[k]);
+            const float sl = sign * sn[2 * k], sh = sign * sn[2 * k + 1];
+            o1[k] = pack_bf16x2(x1l * cs[2 * k] - x2l * sl, x1h * cs[2 * k + 1] - x2h * sh);
+            o2[k] = pack_bf16x2(x2l * cs[2 * k] + x1l * sl, x2h * cs[2 * k + 1] + x1h * sh);
+        }
+        uint16_t* dst = y + rh * head_dim + c * 8;
+        *(uint4*)dst = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+        *(uint4*)(dst + half) = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+    }
+}
+
+}  // namespace coat
+
+using namespace coat;
+
+extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, const int64_t* pos,
+                              int64_t rows, int seq_len, int heads, int head_dim, int inverse, void* stream) {
+    if (rows < 0 || heads <= 0 || head_dim <= 0 || seq_len <= 0) return COAT_EINVAL;
+    if (head_dim % 16 != 0) return COAT_ESHAPE;  // 8 pairs per lane
+    if (rows == 0) return COAT_OK;
+    if (!x || !y || !cos_tab || !sin_tab) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(y) || !coat_aligned16(cos_tab) || !coat_aligned16(sin_tab)) return COAT_EALIGN;
+    const int64_t total = rows * heads * (head_dim / 16);
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(k_rope_bf16, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
+                       (uint16_t*)y, cos_tab, sin_tab, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f);
+    return coat_launch_status();
+}

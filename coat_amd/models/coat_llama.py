@@ -354,6 +354,60 @@ def apply_rotary_pos_emb(q, k, cos, sin):
     return (q * cos) + (_rotate_half(q) * sin), (k * cos) + (_rotate_half(k) * sin)
 
 
+_ROPE_TABLES = {}
+
+
+def rotary_tables(n_pos, head_dim, theta, device):
+    """fp32 cos / sin tables [n_pos, head_dim / 2] for the fused RoPE kernel (cached per device and shape)."""
+    key = (str(device), int(n_pos), int(head_dim), float(theta))
+    if key not in _ROPE_TABLES:
+        inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, device=device, dtype=torch.float32) / head_dim))
+        ang = torch.arange(n_pos, device=device, dtype=torch.float32)[:, None] * inv_freq[None, :]
+        _ROPE_TABLES[key] = (ang.cos().contiguous(), ang.sin().contiguous())
+    return _ROPE_TABLES[key]
+
+
+class _FusedRoPE(torch.autograd.Function):
+    """x bf16 [B, S, heads * head_dim] -> rotated tensor viewed as [B, heads, S, head_dim]; one HIP kernel per direction
+    (``coat_rope_bf16``; the backward pass is the rotation by the negated angle)."""
+
+    @staticmethod
+    def forward(ctx, x, cos_tab, sin_tab, pos, heads, head_dim):
+        from .. import _hip
+        B, S, _ = x.shape
+        x = _hip.dense(x)
+        y = torch.empty_like(x)
+        _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(x), _hip.ptr(y), _hip.ptr(cos_tab), _hip.ptr(sin_tab), _hip.ptr(pos),
+                                             B * S, S, heads, head_dim, 0, _hip.stream(x.device)), "rope forward")
+        ctx.save_for_backward(cos_tab, sin_tab, pos)
+        ctx.dims = (B, S, heads, head_dim)
+        return y.view(B, S, heads, head_dim).transpose(1, 2)
+
+    @staticmethod
+    def backward(ctx, g):
+        from .. import _hip
+        cos_tab, sin_tab, pos = ctx.saved_tensors
+        B, S, heads, head_dim = ctx.dims
+        g = _hip.dense(g.transpose(1, 2).to(torch.bfloat16))  # physically [B, S, heads, head_dim]
+        dx = torch.empty_like(g)
+        _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(g), _hip.ptr(dx), _hip.ptr(cos_tab), _hip.ptr(sin_tab), _hip.ptr(pos),
+                                             B * S, S, heads, head_dim, 1, _hip.stream(g.device)), "rope backward")
+        return dx.view(B, S, heads * head_dim), None, None, None, None, None
+
+
+def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=None):
+    """RoPE on a projection output x [B, S, heads * head_dim] (bf16, on the GPU); returns [B, heads, S, head_dim]."""
+    B, S, _ = x.shape
+    if position_ids is None:
+        cos_tab, sin_tab = rotary_tables(S, head_dim, theta, x.device)
+        pos = None
+    else:
+        n_pos = max(int(max_positions or 0), S)
+        cos_tab, sin_tab = rotary_tables(n_pos, head_dim, theta, x.device)
+        pos = position_ids.expand(B, S).reshape(-1).to(torch.int64).clamp(0, n_pos - 1).contiguous()
+    return _FusedRoPE.apply(x, cos_tab, sin_tab, pos, heads, head_dim)
+
+
 class LlamaSdpaAttentionWithoutLinear(nn.Module):
     """RoPE + causal scaled-dot-product attention on already projected q / k / v (the projections live in the
     Before / AfterAttention modules).  bf16, not part of the FP8 flow."""
@@ -376,16 +430,22 @@ class LlamaSdpaAttentionWithoutLinear(nn.Module):
         if past_key_value is not None or use_cache:
             raise NotImplementedError("KV caching is not part of the training path built here")
         bsz, q_len, _ = query_states.size()
-        q = query_states.view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        k = key_states.view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         v = value_states.view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        if position_embeddings is None:
-            if position_ids is None:
-                position_ids = torch.arange(q_len, device=q.device).unsqueeze(0).expand(bsz, -1)
-            cos, sin = rotary_cos_sin(position_ids, self.head_dim, self.rope_theta, q.dtype)
+        if position_embeddings is None and query_states.is_cuda and query_states.dtype == torch.bfloat16:
+            # one fused kernel per tensor and direction instead of mul / neg / cat / add passes
+            max_pos = getattr(self.config, "max_position_embeddings", None)
+            q = fused_rotary(query_states, self.num_heads, self.head_dim, self.rope_theta, position_ids, max_pos)
+            k = fused_rotary(key_states, self.num_key_value_heads, self.head_dim, self.rope_theta, position_ids, max_pos)
         else:
-            cos, sin = position_embeddings
-        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+            q = query_states.view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+            k = key_states.view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+            if position_embeddings is None:
+                if position_ids is None:
+                    position_ids = torch.arange(q_len, device=q.device).unsqueeze(0).expand(bsz, -1)
+                cos, sin = rotary_cos_sin(position_ids, self.head_dim, self.rope_theta, q.dtype)
+            else:
+                cos, sin = position_embeddings
+            q, k = apply_rotary_pos_emb(q, k, cos, sin)
         if self.num_key_value_groups > 1:
             k = k.repeat_interleave(self.num_key_value_groups, dim=1)
             v = v.repeat_interleave(self.num_key_value_groups, dim=1)

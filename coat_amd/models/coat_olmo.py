@@ -22,7 +22,7 @@ from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_If
                                             fp8_transpose)
 from ..utils._fp8_quantization_config import QuantizationConfig
 from .coat_llama import (E4M3, _as_e4m3_input, _as_e5m2_grad, _backward_weight_t, _forward_weight, _ResidualBase,
-                         apply_rotary_pos_emb, rotary_cos_sin)
+                         apply_rotary_pos_emb, fused_rotary, rotary_cos_sin)
 
 __all__ = ["CoatOLMoConfig", "CoatOLMoBeforeAttentionResidual", "CoatOLMoAfterAttentionResidual",
            "CoatOLMoMLPResidual", "CoatOLMoSequentialBlock"]
@@ -253,9 +253,19 @@ class CoatOLMoSequentialBlock(nn.Module):
         B, T, C = q.size()
         dtype = k.dtype
         hd = C // self.config.n_heads
+        v = v.view(B, T, self.config.effective_n_kv_heads, hd).transpose(1, 2)
+        if self.config.rope and q.is_cuda and dtype == torch.bfloat16:
+            # fused kernel, fp32 arithmetic on fp32 tables (what rope_full_precision asks for)
+            q = fused_rotary(q, self.config.n_heads, hd, self.config.rope_theta)
+            k = fused_rotary(k, self.config.effective_n_kv_heads, hd, self.config.rope_theta)
+        else:
+            q, k = self._rope_unfused(q, k, hd, dtype)
+        return self._sdpa(q, k, v, attention_bias, B, T, C)
+
+    def _rope_unfused(self, q, k, hd, dtype):
+        B, T, _ = q.shape
         q = q.view(B, T, self.config.n_heads, hd).transpose(1, 2)
         k = k.view(B, T, self.config.effective_n_kv_heads, hd).transpose(1, 2)
-        v = v.view(B, T, self.config.effective_n_kv_heads, hd).transpose(1, 2)
         if self.config.rope:
             pos = torch.arange(T, device=q.device).unsqueeze(0)
             if self.config.rope_full_precision:
@@ -265,6 +275,9 @@ class CoatOLMoSequentialBlock(nn.Module):
             else:
                 cos, sin = rotary_cos_sin(pos, hd, self.config.rope_theta, dtype)
                 q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        return q, k
+
+    def _sdpa(self, q, k, v, attention_bias, B, T, C):
         if k.size(1) != q.size(1):
             rep = q.size(1) // k.size(1)
             k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)

@@ -134,6 +134,15 @@ int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_d
                                 float* dw_partial, float* db_partial, int n_partial, int64_t M, int64_t N, int QB,
                                 void* stream);
 
+/* Rotary position embedding of the bf16 attention (no single counterpart in the reference, which applies it with
+ * several torch kernels: transformers' apply_rotary_pos_emb as called at coat/models/coat_llama.py:1029-1030, olmo's
+ * RotaryEmbedding at coat/models/coat_olmo.py:862-863).  x, y bf16 [rows, heads, head_dim], rows = batch * seq;
+ * cos_tab / sin_tab fp32 [n_pos, head_dim / 2]; pos int64 [rows] or NULL (position = row % seq_len);
+ * y1 = x1 cos - x2 sin, y2 = x2 cos + x1 sin on the (d, d + head_dim/2) pairs; inverse != 0 negates the angle, which
+ * is the backward pass.  head_dim % 16 == 0. */
+int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, const int64_t* pos,
+                   int64_t rows, int seq_len, int heads, int head_dim, int inverse, void* stream);
+
 /* ---- GEMM -------------------------------------------------------------------------------------------
  * rq/linear.py:172 fp8matmul (kernel :61-169): C[M,N] = (A[M,K] . B[N,K]^T) * (float(*scale_a) * float(*scale_b))
  * (+ bias[N]), fp32 accumulation on FP8 MFMA.  A and B are row-major with K contiguous (the reference passes B as
