@@ -76,18 +76,17 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 
 // s_waitcnt vmcnt(N) only (expcnt / lgkmcnt left at their maxima), gfx9 encoding.
 #define COAT_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (0x7 << 4) | (0xF << 8) | ((((N) >> 4) & 0x3) << 14))
-// the same with lgkmcnt(0): all LDS reads issued so far have returned
-#define COAT_WAIT_VMCNT_LGKM0(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (0x7 << 4) | (0x0 << 8) | ((((N) >> 4) & 0x3) << 14))
+// lgkmcnt(0) only: all LDS reads issued so far have returned
+#define COAT_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
 
 // Eight waves (2 along M x 4 along N), each 128 x 64 of the 256 x 256 tile as 4 x 2 tiles of
 // v_mfma_f32_32x32x64_f8f6f4, two waves per SIMD.
 // Persistent: the grid is one block per CU; a block walks its share of the output tiles and the LDS ring runs straight
 // across tile boundaries, so the first slabs of the next tile are already in flight while the epilogue stores drain.
-template <int FMT_A, int FMT_B, int EPI>
+template <int FMT_A, int FMT_B, int EPI, bool VEC16>
 __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     constexpr int NWN = 4, NW = 2 * NWN;      // waves along N, waves per block
     constexpr int TJ = BN / (NWN * 32);       // n-tiles per wave (2); m-tiles per wave is 4
-    constexpr int LI = BM / (NW * 8);         // load instructions per wave per slab (each covers 8 rows)
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -113,61 +112,67 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
         n0 = ((tile % width) / gsize) * BN;
     };
 
-    // ---- global -> LDS without passing through registers.  The ring holds 5 slabs; slab u of a tile is the A slab
-    // (u even) or the B slab (u odd) of K-step u / 2.  One wave instruction fills 1 KiB of LDS contiguously (lane i at
-    // +16 i) = 8 slab rows; the lane picks the global chunk that belongs at its position under the swizzle.
-    // Out-of-range rows / K-tail chunks use an offset beyond the buffer's extent, which fills zeros.
-    const v4i rsrcA = make_rsrc(G.A, (uint32_t)(G.M * G.K));
-    const v4i rsrcB = make_rsrc(G.B, (uint32_t)(G.N * G.K));
+    // ---- global -> LDS without passing through registers.  The ring holds 5 slabs; slab u of this block's slab
+    // sequence is the A slab (u even) or the B slab (u odd) of K-step u / 2 and lives in slot u % 5.  One wave
+    // instruction fills 1 KiB of LDS contiguously (lane i at +16 i) = 8 slab rows; the lane picks the global chunk
+    // that belongs at its position under the swizzle.  Out-of-range rows / K-tail chunks use an offset beyond the
+    // buffer's extent, which fills zeros.
+    //
+    // Ping-pong schedule.  The two waves of a SIMD work half a K-step apart: waves 0-3 (role 0) and waves 4-7 (role 1)
+    // alternate between a memory phase (read the 24 fragments of a K-step from LDS into registers, issue 8 loads of a
+    // later slab) and a compute phase (16 MFMAs back to back, nothing else in the instruction stream), separated by
+    // block-wide barriers; role 1 starts one phase late.  In every phase each SIMD has one wave feeding the matrix
+    // pipe and one wave doing memory work, so a load or LDS read that waits for its unit never delays an MFMA.
+    //   phase 2j-1: role 0 mem(j)  [reads slabs A(j) B(j); loads B(j+1)]   role 1 MFMA(j-1)
+    //   phase 2j  : role 0 MFMA(j)                                          role 1 mem(j) [reads A(j) B(j); loads A(j+2)]
+    // Slots: B(j+1) replaces A(j-1) and A(j+2) replaces B(j-1), both last read in phase 2j-2; a wave waits for its own
+    // loads at the end of its compute phase (a whole phase after issuing them), before the barrier that publishes them.
+    const int role = wave >> 2;                     // 0: loads B slabs, 1: loads A slabs
+    const v4i rsrc = role ? make_rsrc(G.A, (uint32_t)(G.M * G.K)) : make_rsrc(G.B, (uint32_t)(G.N * G.K));
+    const int R = role ? G.M : G.N;                 // rows of the matrix this wave loads
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
     const int nstep = (G.K + BK - 1) / BK;
-    // load cursor: tile iteration lt, K-step lstep of that tile, ring slot sl_load; slabs go A, B, A, B, ...
     constexpr int kOob = 0x7FFFFFFF;
-    int offA[LI], offB[LI], kc[LI];  // per-lane byte offsets of K-step 0 (kOob for rows outside the matrix)
-    const int lrow = wave * (LI * 8) + (lane >> 3);  // + 8 i
-#pragma unroll
-    for (int i = 0; i < LI; i++) kc[i] = swz_chunk(lrow + 8 * i, lane & 7) * 16;
-    int lt = 0, lstep = 0, sl_load = 0;
+    constexpr int LI = 8;                           // load instructions per wave per slab (8 rows each; 4 waves per slab)
+    const int lrow = (wave & 3) * (LI * 8) + (lane >> 3);  // + 8 i
+    // rows 8 i apart alternate between two swizzle patterns, and two instructions of the same parity differ by a
+    // multiple of 16 rows, which goes into the scalar offset: two per-lane offsets suffice
+    int kc[2], off[2];
+    kc[0] = swz_chunk(lrow, lane & 7) * 16;
+    kc[1] = swz_chunk(lrow + 8, lane & 7) * 16;
+    // load cursor: tile iteration lt, K-step lstep of that tile, global K-step counter lg (gives the ring slot)
+    int lt = 0, lstep = 0, lslot = role ? 0 : 1;    // A(g) lives in slot 2g % 5, B(g) in (2g + 1) % 5
+    int lr0 = 0;                                    // first row (of the loaded matrix) of the tile being loaded
+    bool ledge = false;                             // its rows run past the end of the matrix (or there is no such tile)
     auto set_load_tile = [&](int it) {
-        int m0 = 0, n0 = 0;
         const bool live = it < my_ntiles;
+        int m0 = 0, n0 = 0;
         if (live) tile_origin(it, m0, n0);
+        lr0 = live ? (role ? m0 : n0) : R;
+        ledge = lr0 + BM > R;
 #pragma unroll
-        for (int i = 0; i < LI; i++) {
-            const int row = lrow + 8 * i;
-            offA[i] = (live && m0 + row < G.M) ? (m0 + row) * G.K + kc[i] : kOob;
-            offB[i] = (live && n0 + row < G.N) ? (n0 + row) * G.K + kc[i] : kOob;
-        }
+        for (int p = 0; p < 2; p++) off[p] = live ? (lr0 + lrow + 8 * p) * G.K + kc[p] : 0;
     };
     set_load_tile(0);
-    // one load instruction (8 slab rows) of the A / B slab at the cursor.  Interior K-steps add the step's K offset
-    // as the instruction's scalar offset (no per-lane arithmetic); only a last, partial K-step masks lanes past K.
-    auto dma_row = [&](const v4i& rsrc, int off, int kci, int i) {
+    // The K-step offset and the 16-row multiple go into the scalar offset, which takes no part in the range check:
+    // rows past the matrix end and chunks past K (edge tiles / a last partial K-step only) are masked by hand.
+    auto issue_slab = [&]() {
         const int k0 = lstep * BK;
-        const uint32_t dst = lds_base + sl_load * kUnitBytes + (wave * LI + i) * (8 * BK);
-        int v = off;
-        if (k0 + BK > G.K && k0 + kci >= G.K) v = kOob;
-        lds_dma16(rsrc, dst, v, k0);
-    };
-    auto dma_A = [&](int i) { dma_row(rsrcA, offA[i], kc[i], i); };
-    auto dma_B = [&](int i) { dma_row(rsrcB, offB[i], kc[i], i); };
-    auto next_A = [&]() { sl_load = sl_load + 1 == NUNIT ? 0 : sl_load + 1; };
-    auto next_B = [&]() {
-        sl_load = sl_load + 1 == NUNIT ? 0 : sl_load + 1;
+        const uint32_t dst = lds_base + lslot * kUnitBytes + (wave & 3) * (LI * 8 * BK);
+        const bool check = ledge || k0 + BK > G.K;
+#pragma unroll
+        for (int i = 0; i < LI; i++) {
+            int v = off[i & 1];
+            if (check) {
+                if (lr0 + lrow + 8 * i >= R || k0 + kc[i & 1] >= G.K) v = kOob;
+            }
+            lds_dma16(rsrc, dst + i * (8 * BK), v, k0 + (i >> 1) * 16 * G.K);
+        }
+        lslot = lslot + 2 >= NUNIT ? lslot + 2 - NUNIT : lslot + 2;
         if (++lstep == nstep) {
             lstep = 0;
-            set_load_tile(++lt);  // past the last tile: zero fills, which keep the outstanding-load counts uniform
+            set_load_tile(++lt);  // past the last tile: zero fills
         }
-    };
-    auto issue_A = [&]() {
-#pragma unroll
-        for (int i = 0; i < LI; i++) dma_A(i);
-        next_A();
-    };
-    auto issue_B = [&]() {
-#pragma unroll
-        for (int i = 0; i < LI; i++) dma_B(i);
-        next_B();
     };
     // fragment addresses (bytes inside a slab) for this lane and K-substep 0: row = tile base + lane % 32, 16-byte
     // chunks 2 * (lane / 32) + h; the chunks of substep 1 are those + 4, i.e. the address with bit 6 flipped.
@@ -179,7 +184,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
         fa_off[h] = rowa * BK + (swz_chunk(rowa, c) << 4);
         fb_off[h] = rowb * BK + (swz_chunk(rowb, c) << 4);
     }
-    int sl_frag = 0;  // ring slot of the A slab of the K-step being multiplied (its B slab is in the next slot)
+    int sl_frag = 0;  // ring slot of the A slab of the K-step whose fragments are read next (its B slab: next slot)
     auto load_fa = [&](int slot_a, int sub, int t) -> v8i {
         const uint8_t* sa = lds + slot_a * kUnitBytes + t * 32 * BK;
         const int x = sub * 64;
@@ -195,86 +200,65 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
 
     v16f acc[TJ][4];  // [n-tile j][m-tile i]
     v8i fax[4], fbx[TJ], fay[4], fby[TJ];  // fragments of K-substep 0 (x) and 1 (y)
-    // prologue: two K-steps in flight (A0 B0 A1 B1), wait for the first step's two slabs, fetch its substep-0 fragments
-    issue_A();
-    issue_B();
-    issue_A();
-    issue_B();
-    COAT_WAIT_VMCNT(2 * LI);
+    // prologue: A(0) B(0) A(1) in flight (role 1: two A slabs, role 0: one B slab), all landed and published
+    issue_slab();
+    if (role) issue_slab();
+    COAT_WAIT_VMCNT(0);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-#pragma unroll
-    for (int t = 0; t < 4; t++) fax[t] = load_fa(sl_frag, 0, t);
-#pragma unroll
-    for (int t = 0; t < TJ; t++) fbx[t] = load_fb(sl_frag, 0, t);
+    if (role) __builtin_amdgcn_s_barrier();  // role 1 runs one phase behind
 #define COAT_MFMA(FB_, FA_, J, I) \
     acc[J][I] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FB_[J], FA_[I], acc[J][I], FMT_B, FMT_A, 0, 0, 0, 0)
-#define COAT_PIN() __builtin_amdgcn_sched_barrier(0)
-    // One K-step of 128 = 2 substeps x 8 MFMAs per wave, with one barrier in the middle:
-    //   multiply substep 0 while reading the substep-1 fragments;
-    //   wait until those reads have returned and at most the newest slab is outstanding, barrier: every wave now holds
-    //   all it needs from this step's two slabs in registers, and the next step's slabs have landed and are visible
-    //   (loads return in order, so this holds also when epilogue stores of the previous tile are still in the count);
-    //   multiply substep 1 while refilling this step's two slots and reading the next step's substep-0 fragments.
-    // Loads and LDS reads are spread between the MFMAs by hand (and pinned) so that the matrix pipe never waits for a
-    // burst of address arithmetic after the barrier.
-    static_assert(TJ == 2 && LI == 4 && NW == 8, "the interleaving below is written for eight waves of 128 x 64");
-    auto step = [&]() {
-        // substep 0: 8 MFMAs; between them the substep-1 fragment reads and the four loads of the A slab two steps ahead
-        COAT_MFMA(fbx, fax, 0, 0); COAT_PIN();
-        fay[0] = load_fa(sl_frag, 1, 0); fby[0] = load_fb(sl_frag, 1, 0); COAT_PIN();
-        COAT_MFMA(fbx, fax, 0, 1); COAT_PIN();
-        dma_A(0); COAT_PIN();
-        COAT_MFMA(fbx, fax, 0, 2); COAT_PIN();
-        fay[1] = load_fa(sl_frag, 1, 1); fby[1] = load_fb(sl_frag, 1, 1); COAT_PIN();
-        COAT_MFMA(fbx, fax, 0, 3); COAT_PIN();
-        dma_A(1); COAT_PIN();
-        COAT_MFMA(fbx, fax, 1, 0); COAT_PIN();
-        fay[2] = load_fa(sl_frag, 1, 2); fay[3] = load_fa(sl_frag, 1, 3); COAT_PIN();
-        COAT_MFMA(fbx, fax, 1, 1); COAT_PIN();
-        dma_A(2); COAT_PIN();
-        COAT_MFMA(fbx, fax, 1, 2); COAT_PIN();
-        dma_A(3); next_A(); COAT_PIN();
-        COAT_MFMA(fbx, fax, 1, 3); COAT_PIN();
-        COAT_WAIT_VMCNT_LGKM0(LI);
+    static_assert(TJ == 2 && NW == 8, "the schedule is written for eight waves of 128 x 64");
+    auto mem_phase = [&]() {
+#pragma unroll
+        for (int t = 0; t < 4; t++) fax[t] = load_fa(sl_frag, 0, t);
+#pragma unroll
+        for (int t = 0; t < TJ; t++) fbx[t] = load_fb(sl_frag, 0, t);
+#pragma unroll
+        for (int t = 0; t < 4; t++) fay[t] = load_fa(sl_frag, 1, t);
+#pragma unroll
+        for (int t = 0; t < TJ; t++) fby[t] = load_fb(sl_frag, 1, t);
+        sl_frag = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
+        issue_slab();
+        // every fragment has arrived before the barrier: the compute phase has nothing to wait for, and the slabs
+        // just read may be overwritten by loads issued after the barrier that follows the compute phase
+        COAT_WAIT_LGKM0();
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        const int sl_next = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
-        // substep 1: 8 MFMAs; between them the next step's substep-0 fragment reads and the four loads of its
-        // successor's B slab
-        COAT_MFMA(fby, fay, 0, 0); COAT_PIN();
-        fax[0] = load_fa(sl_next, 0, 0); fbx[0] = load_fb(sl_next, 0, 0); COAT_PIN();
-        COAT_MFMA(fby, fay, 0, 1); COAT_PIN();
-        dma_B(0); COAT_PIN();
-        COAT_MFMA(fby, fay, 0, 2); COAT_PIN();
-        fax[1] = load_fa(sl_next, 0, 1); fbx[1] = load_fb(sl_next, 0, 1); COAT_PIN();
-        COAT_MFMA(fby, fay, 0, 3); COAT_PIN();
-        dma_B(1); COAT_PIN();
-        COAT_MFMA(fby, fay, 1, 0); COAT_PIN();
-        fax[2] = load_fa(sl_next, 0, 2); fax[3] = load_fa(sl_next, 0, 3); COAT_PIN();
-        COAT_MFMA(fby, fay, 1, 1); COAT_PIN();
-        dma_B(2); COAT_PIN();
-        COAT_MFMA(fby, fay, 1, 2); COAT_PIN();
-        dma_B(3); next_B(); COAT_PIN();
-        COAT_MFMA(fby, fay, 1, 3); COAT_PIN();
-        sl_frag = sl_next;
+    };
+    auto compute_phase = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) COAT_MFMA(fbx, fax, j, i);
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) COAT_MFMA(fby, fay, j, i);
+        __builtin_amdgcn_sched_barrier(0);
+        COAT_WAIT_VMCNT(0);  // this wave's loads (issued a phase ago) and, once per tile, its epilogue stores
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
     };
     const float scale = load_rt_f32(G.sa, 0, G.s_dt) * load_rt_f32(G.sb, 0, G.s_dt);
     if (EPI != kEpiBf16) enable_fp8_saturation();
     const int half = lane >> 5;
+    constexpr bool vec16 = VEC16;  // rows of C start 16-byte aligned (N % 8 == 0): 16-byte stores
 
-    for (int it = 0; it < my_ntiles; it++) {
-#pragma unroll
-    for (int j = 0; j < TJ; j++)
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
-    for (int ks = 0; ks < nstep; ks++) step();
+    // Tile loop.  The epilogue of tile it-1 opens the first memory phase of tile it (the other role computes
+    // meanwhile); after the last tile it runs on its own.
+    for (int it = 0; it <= my_ntiles; it++) {
+    if (it > 0) {
     int m0, n0;
-    tile_origin(it, m0, n0);
+    tile_origin(it - 1, m0, n0);
 
     // ---- epilogue (stores are not waited for: they drain while the next tile is multiplied)
+    uint8_t* const c_tile = (uint8_t*)G.C + ((int64_t)m0 * G.N + n0) * 2;  // bf16 output: origin of this tile
+    const uint32_t c_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * G.N + wn * (TJ * 32) + 8 * half) * 2;
+    const int m_lim = G.M - m0 - wm * 128 - (lane & 31);   // row i * 32 of this lane exists iff i * 32 < m_lim
+    const int n_lim = G.N - n0 - wn * (TJ * 32) - 8 * half;  // column offset c of this lane exists iff c < n_lim
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int m = m0 + wm * 128 + i * 32 + (lane & 31);
@@ -293,7 +277,24 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                         if (n < G.N) v[4 * q + e] += load_rt_f32(G.bias, n, G.bias_dt);
                     }
             }
-            if (EPI == kEpiBf16) {
+            __builtin_amdgcn_sched_barrier(0);  // one accumulator tile at a time: keeps the epilogue's live ranges short
+            if (EPI == kEpiBf16 && vec16) {
+                // lanes l and l + 32 hold the two 8-byte halves of a 16-byte run of row m for each quad; swapping the
+                // halves of two neighbouring quads between them (v_permlane32_swap) leaves every lane with one whole
+                // 16-byte run: half as many store instructions, each covering 32 rows x 32 bytes
+#pragma unroll
+                for (int qp = 0; qp < 2; qp++) {
+                    uint32_t a0 = pack_bf16x2(v[8 * qp], v[8 * qp + 1]), a1 = pack_bf16x2(v[8 * qp + 2], v[8 * qp + 3]);
+                    uint32_t b0 = pack_bf16x2(v[8 * qp + 4], v[8 * qp + 5]), b1 = pack_bf16x2(v[8 * qp + 6], v[8 * qp + 7]);
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+                    // lanes < 32 now hold quad 2 qp whole (n = 16 qp .. + 7 of this 32-column tile), lanes >= 32 quad
+                    // 2 qp + 1.  Address = uniform tile / sub-tile base (scalar) + one 32-bit per-lane offset.
+                    uint8_t* base = c_tile + ((int64_t)(i * 32) * G.N + j * 32 + 16 * qp) * 2;
+                    if (i * 32 < m_lim && j * 32 + 16 * qp < n_lim)  // N % 8 == 0: a 16-byte run is inside or outside as a whole
+                        *(uint4*)(base + c_lane_off) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+                }
+            } else if (EPI == kEpiBf16) {
                 if (m < G.M) {
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
@@ -333,7 +334,35 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
             }
         }
     }
+    }  // epilogue of tile it - 1
+    if (it == my_ntiles) break;
+#pragma unroll
+    for (int j = 0; j < TJ; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
+    // the rest of the tile's first memory phase: fragments of K-step 0 and this phase's loads
+#pragma unroll
+    for (int t = 0; t < 4; t++) fax[t] = load_fa(sl_frag, 0, t);
+#pragma unroll
+    for (int t = 0; t < TJ; t++) fbx[t] = load_fb(sl_frag, 0, t);
+#pragma unroll
+    for (int t = 0; t < 4; t++) fay[t] = load_fa(sl_frag, 1, t);
+#pragma unroll
+    for (int t = 0; t < TJ; t++) fby[t] = load_fb(sl_frag, 1, t);
+    sl_frag = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
+    issue_slab();
+    COAT_WAIT_LGKM0();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    compute_phase();
+    for (int ks = 1; ks < nstep; ks++) {
+        mem_phase();
+        compute_phase();
+    }
     }  // tiles
+    if (!role) __builtin_amdgcn_s_barrier();  // role 0 started a phase early: its last barrier pairs with role 1's
     COAT_WAIT_VMCNT(0);  // drain the trailing zero-fill slabs before the block may exit
 }
 
@@ -372,17 +401,23 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     const int grid = min(((ntiles + 7) / 8) * 8, n_cu);
     const size_t lds_bytes = kLdsBytes;
     hipStream_t st = (hipStream_t)stream;
-#define GEMM_LAUNCH(FA, FB, EP)                                                                                    \
+#define GEMM_LAUNCH_V(FA, FB, EP, V16)                                                                                  \
     {                                                                                                              \
         static bool attr_set = false;                                                                              \
         if (!attr_set) {                                                                                           \
-            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP>,                 \
+            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP, V16>,                 \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);        \
             if (e != hipSuccess) return (int)e;                                                                    \
             attr_set = true;                                                                                       \
         }                                                                                                          \
-        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP>), dim3(grid), dim3(512), lds_bytes, st, G); \
+        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, V16>), dim3(grid), dim3(512), lds_bytes, st, G); \
         return coat_launch_status();                                                                               \
+    }
+// the 16-byte-store epilogue only exists for the bf16 output
+#define GEMM_LAUNCH(FA, FB, EP)                                                  \
+    {                                                                            \
+        if (EP == kEpiBf16 && (N & 7) == 0) GEMM_LAUNCH_V(FA, FB, EP, true)      \
+        GEMM_LAUNCH_V(FA, FB, EP, false)                                         \
     }
 #define GEMM_FMT(EP)                                                             \
     if (fmt_a == COAT_E4M3 && fmt_b == COAT_E4M3) GEMM_LAUNCH(0, 0, EP)          \
