@@ -259,6 +259,12 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     const uint32_t c_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * G.N + wn * (TJ * 32) + 8 * half) * 2;
     const int m_lim = G.M - m0 - wm * 128 - (lane & 31);   // row i * 32 of this lane exists iff i * 32 < m_lim
     const int n_lim = G.N - n0 - wn * (TJ * 32) - 8 * half;  // column offset c of this lane exists iff c < n_lim
+    // quantized output: fp8 codes [M, N] and bf16 scales [M, N / 16] (N % 16 == 0), same addressing scheme
+    uint8_t* const q_tile = (uint8_t*)G.C + ((int64_t)m0 * G.N + n0);
+    uint8_t* const s_tile = (uint8_t*)G.Cs + ((int64_t)m0 * (G.N >> 4) + (n0 >> 4)) * 2;
+    const uint32_t q_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * G.N + wn * (TJ * 32) + 8 * half);
+    const uint32_t s_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * (G.N >> 4) + wn * (TJ * 2)) * 2;
+    const int q_n_lim = G.N - n0 - wn * (TJ * 32);          // a 16-column group at offset c exists iff c < q_n_lim
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int m = m0 + wm * 128 + i * 32 + (lane & 31);
@@ -310,7 +316,8 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                 }
             } else {
                 constexpr int KIND = EPI == kEpiQuantE4M3 ? kE4M3 : kE5M2;
-                // group g2 of 16 consecutive n = quads 2*g2, 2*g2+1 of this lane and of lane ^ 32
+                // group g2 of 16 consecutive n = quads 2*g2, 2*g2+1 of this lane and of lane ^ 32; after the swap a
+                // lane holds 8 consecutive codes (lanes < 32 the group's first half, lanes >= 32 its second half)
 #pragma unroll
                 for (int g2 = 0; g2 < 2; g2++) {
                     float amax = 0.0f;
@@ -319,16 +326,18 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                     amax = fmaxf(amax, lane_xor_f32(amax, 32));
                     const float s = group_scale<KIND>(amax);
                     const float r = 1.0f / s;
-                    const int ng = n0 + wn * (TJ * 32) + j * 32 + 16 * g2;  // first n of the group
-                    if (m < G.M && ng < G.N) {
-#pragma unroll
-                        for (int qq = 0; qq < 2; qq++) {
-                            const int q = 2 * g2 + qq;
-                            const uint32_t w = cvt4_fp8<KIND>(div_by_scale(v[4 * q], s, r), div_by_scale(v[4 * q + 1], s, r),
-                                                              div_by_scale(v[4 * q + 2], s, r), div_by_scale(v[4 * q + 3], s, r));
-                            *(uint32_t*)((uint8_t*)G.C + (int64_t)m * G.N + nb + 8 * q) = w;
+                    const uint32_t w0 = cvt4_fp8<KIND>(div_by_scale(v[8 * g2], s, r), div_by_scale(v[8 * g2 + 1], s, r),
+                                                       div_by_scale(v[8 * g2 + 2], s, r), div_by_scale(v[8 * g2 + 3], s, r));
+                    const uint32_t w1 = cvt4_fp8<KIND>(div_by_scale(v[8 * g2 + 4], s, r), div_by_scale(v[8 * g2 + 5], s, r),
+                                                       div_by_scale(v[8 * g2 + 6], s, r), div_by_scale(v[8 * g2 + 7], s, r));
+                    const auto sw = __builtin_amdgcn_permlane32_swap(w0, w1, false, false);
+                    if (i * 32 < m_lim && j * 32 + 16 * g2 < q_n_lim) {
+                        uint8_t* base = q_tile + ((int64_t)(i * 32) * G.N + j * 32 + 16 * g2);
+                        *(uint2*)(base + q_lane_off) = make_uint2(sw[0], sw[1]);
+                        if (half == 0) {
+                            uint8_t* sbase = s_tile + ((int64_t)(i * 32) * (G.N >> 4) + j * 2 + g2) * 2;
+                            *(uint16_t*)(sbase + s_lane_off) = (uint16_t)f2bf16(s);
                         }
-                        if (half == 0) ((uint16_t*)G.Cs)[(int64_t)m * (G.N >> 4) + (ng >> 4)] = (uint16_t)f2bf16(s);
                     }
                 }
             }
