@@ -155,17 +155,15 @@ def make_silu_mul_workload(dev, torch):
     def step():
         qg, sg = rq.fp8_quantize(gate, QB, "E4M3")
         qu, su = rq.fp8_quantize(up, QB, "E4M3")
-        qs, ss = rq.fp8_silu_forward(qg, sg, QB)
-        rq.fp8_mul_forward(qs, ss, qu, su, QB, transpose_output_2d=True)
-        g1, _ = rq.fp8_mul_backward(qs, ss, qu, su, g, QB, "E5M2", output_quantized_transpose=True)
-        rq.fp8_silu_backward(qg, sg, g1, QB, "E5M2", output_quantized_transpose=True)
+        qs, ss, _, _, _ = rq.fp8_silu_mul_forward(qg, sg, qu, su, QB, transpose_output_2d=True)
+        rq.fp8_silu_mul_backward(qg, sg, qu, su, qs, ss, g, QB, "E5M2")
 
     E = M * N
     # forward: read 2 bf16 inputs (4E), write gate / up / silu codes + scales 3(E + E/8), write product q + q^T (2E);
     # backward: read g (2E) + the three saved FP8 tensors 3(E + E/8), write two gradients as q + q^T (4E)
     nbytes = int(4 * E + 3 * (E + E / 8) + 2 * E + 2 * E + 3 * (E + E / 8) + 4 * E)
     return step, nbytes, {"workload": f"SiLU(gate)*up fwd + bwd chain on bf16 [{M},{N}], 1x16 e4m3 / per-tensor e5m2 outputs",
-                          "M": M, "N": N, "kernel": "k_quantize_pg, k_elementwise, k_division_transpose"}
+                          "M": M, "N": N, "kernel": "k_quantize_pg, k_silu_mul, k_division_transpose"}
 
 
 def make_rmsnorm_workload(dev, torch):

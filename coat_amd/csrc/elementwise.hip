@@ -159,6 +159,104 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
     if (A.s_max) block_atomic_max_nonneg(A.s_max, tensor_max, smem_max);
 }
 
+// ---- SiLU(gate) * up in one pass, forward and backward -------------------------------------------------------------
+// The reference runs SiLU and the product as separate kernels (silu_fwd.py:152 then mul_fwd.py:191; mul_bwd.py:221 then
+// silu_bwd.py:170), re-reading the FP8 SiLU output and writing / re-reading the bf16 gradient of the product in between.
+// These kernels produce bit-identical tensors in one pass: every rounding the chain performs (SiLU -> per-group FP8 with
+// a bf16 scale -> dequantize; g * up -> bf16) is performed in registers.
+struct SiluMulArgs {
+    const void *gate, *s_gate, *up, *s_up, *silu, *s_silu;  // per-group FP8 inputs (silu: backward only) and their scales
+    const void* g;                                          // backward: bf16 gradient of the product
+    void *q_silu, *s_silu_out;                              // forward: per-group FP8 SiLU output + bf16 scales (saved for backward)
+    void* y;                                                // forward: bf16 product;  backward: bf16 gradient of gate
+    void* y2;                                               // backward: bf16 gradient of up
+    float *s_max, *s_max2;                                  // max of the fp32 group scales of y / y2
+    int64_t nchunk;
+    int qb, s_dtype;
+};
+
+template <int KIND> __device__ __forceinline__ void dequant_words(const uint32_t* w, float scale, float* v) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float f[4];
+        fp8x4_to_f32<KIND>(w[k], f);
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[4 * k + i] = f[i] * scale;
+    }
+}
+__device__ __forceinline__ float round_bf16(float x) { return u2f((uint32_t)f2bf16(x) << 16); }
+__device__ __forceinline__ float amax16(const float* v) {
+    float a = fmaxf(fabsf(v[0]), fabsf(v[1]));
+#pragma unroll
+    for (int i = 2; i < 16; i++) a = fmaxf(a, fabsf(v[i]));
+    return a;
+}
+
+template <bool BWD, int KIND_IN, int KIND_OUT>
+__global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
+    __shared__ float smem_max[4];
+    enable_fp8_saturation();
+    const int lpg = A.qb >> 4;
+    float tmax = 0.0f, tmax2 = 0.0f;
+    for (int64_t base = (int64_t)blockIdx.x * 256; base < A.nchunk; base += (int64_t)gridDim.x * 256) {
+        const int64_t chunk = base + threadIdx.x;
+        const bool ok = chunk < A.nchunk;
+        const int64_t c = ok ? chunk : 0;
+        const int64_t gidx = (c * 16) / A.qb;
+        float a[16], b[16];
+        load_fp8x16<KIND_IN>(A.gate, c, load_scale_rt(A.s_gate, gidx, A.s_dtype), a);
+        load_fp8x16<KIND_IN>(A.up, c, load_scale_rt(A.s_up, gidx, A.s_dtype), b);
+        if (!BWD) {
+            float sv[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) sv[i] = sigmoid_f32(a[i]) * a[i];
+            const float s = group_scale<KIND_IN>(cluster_max_rt(amax16(sv), lpg));
+            const float r = 1.0f / s;
+            uint32_t w[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                w[k] = cvt4_fp8<KIND_IN>(div_by_scale(sv[4 * k], s, r), div_by_scale(sv[4 * k + 1], s, r),
+                                         div_by_scale(sv[4 * k + 2], s, r), div_by_scale(sv[4 * k + 3], s, r));
+            if (ok) {
+                *(uint4*)((uint8_t*)A.q_silu + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+                if ((threadIdx.x % lpg) == 0) ((uint16_t*)A.s_silu_out)[gidx] = (uint16_t)f2bf16(s);
+            }
+            // what the product kernel would read back: the codes times the bf16-rounded scale
+            float d[16], v[16];
+            dequant_words<KIND_IN>(w, round_bf16(s), d);
+#pragma unroll
+            for (int i = 0; i < 16; i++) v[i] = d[i] * b[i];
+            if (ok) store_bf16x16(A.y, c, v);
+            const float s2 = group_scale<KIND_IN>(cluster_max_rt(amax16(v), lpg));
+            tmax = fmaxf(tmax, ok ? s2 : 0.0f);
+        } else {
+            float sl[16], g[16], v[16], v2[16];
+            load_fp8x16<KIND_IN>(A.silu, c, load_scale_rt(A.s_silu, gidx, A.s_dtype), sl);
+            load_bf16x16(A.g, c, g);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                v2[i] = g[i] * sl[i];                       // gradient of up
+                const float g1 = round_bf16(g[i] * b[i]);   // gradient of SiLU's output as the chain stores it (bf16)
+                const float sig = sigmoid_f32(a[i]);
+                v[i] = (sig + (a[i] * sig) * (1 - sig)) * g1;
+            }
+            if (ok) {
+                store_bf16x16(A.y, c, v);
+                store_bf16x16(A.y2, c, v2);
+            }
+            const float s1 = group_scale<KIND_OUT>(cluster_max_rt(amax16(v), lpg));
+            const float s2 = group_scale<KIND_OUT>(cluster_max_rt(amax16(v2), lpg));
+            tmax = fmaxf(tmax, ok ? s1 : 0.0f);
+            tmax2 = fmaxf(tmax2, ok ? s2 : 0.0f);
+        }
+    }
+    block_atomic_max_nonneg(A.s_max, tmax, smem_max);
+    if (BWD) {
+        __syncthreads();
+        block_atomic_max_nonneg(A.s_max2, tmax2, smem_max);
+    }
+}
+
 }  // namespace coat
 
 using namespace coat;
@@ -262,4 +360,50 @@ extern "C" int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s
     if (M * N == 0) return COAT_OK;
     if (!x1 || !x2 || !y) return COAT_EINVAL;
     return launch_ew<kAddBwd>(A, COAT_E4M3, fp8_out, (hipStream_t)stream);
+}
+
+static int silu_mul_launch(SiluMulArgs& A, bool bwd, int fp8_in, int fp8_out, int64_t M, int64_t N, int QB, int s_dtype,
+                           hipStream_t st) {
+    if (M < 0 || N < 0) return COAT_EINVAL;
+    if (QB < 16 || QB > 1024 || (QB & (QB - 1)) || N % QB != 0) return COAT_ESHAPE;
+    if (s_dtype != COAT_BF16 && s_dtype != COAT_F32 && s_dtype != COAT_F16) return COAT_EDTYPE;
+    if (fp8_in != COAT_E4M3 && fp8_in != COAT_E5M2) return COAT_EINVAL;
+    if (bwd && fp8_out != COAT_E4M3 && fp8_out != COAT_E5M2) return COAT_EINVAL;
+    if (M * N == 0) return COAT_OK;
+    const void* ptrs[] = {A.gate, A.up, A.silu, A.g, A.q_silu, A.y, A.y2};
+    for (const void* p : ptrs)
+        if (!coat_aligned16(p)) return COAT_EALIGN;
+    A.nchunk = M * N / 16;
+    A.qb = QB;
+    A.s_dtype = s_dtype;
+    int64_t blocks = (A.nchunk + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+#define SM_LAUNCH(B, KI, KO) hipLaunchKernelGGL((k_silu_mul<B, KI, KO>), dim3((unsigned)blocks), dim3(256), 0, st, A)
+    if (!bwd) {
+        if (fp8_in == COAT_E4M3) SM_LAUNCH(false, kE4M3, kE4M3); else SM_LAUNCH(false, kE5M2, kE5M2);
+    } else if (fp8_in == COAT_E4M3) {
+        if (fp8_out == COAT_E4M3) SM_LAUNCH(true, kE4M3, kE4M3); else SM_LAUNCH(true, kE4M3, kE5M2);
+    } else {
+        if (fp8_out == COAT_E4M3) SM_LAUNCH(true, kE5M2, kE4M3); else SM_LAUNCH(true, kE5M2, kE5M2);
+    }
+#undef SM_LAUNCH
+    return coat_launch_status();
+}
+
+extern "C" int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
+                                         int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M,
+                                         int64_t N, int QB, void* stream) {
+    if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !q_silu || !s_silu || !y || !s_max)) return COAT_EINVAL;
+    SiluMulArgs A = {gate, s_gate, up, s_up, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr, 0, 0, 0};
+    return silu_mul_launch(A, false, fp8, fp8, M, N, QB, s_dtype, (hipStream_t)stream);
+}
+
+extern "C" int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, const void* up, const void* s_up,
+                                          const void* silu, const void* s_silu, int fp8_in, int s_dtype, const void* g,
+                                          void* y_gate, float* s_max_gate, void* y_up, float* s_max_up, int fp8_out,
+                                          int64_t M, int64_t N, int QB, void* stream) {
+    if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !silu || !s_silu || !g || !y_gate || !s_max_gate || !y_up || !s_max_up))
+        return COAT_EINVAL;
+    SiluMulArgs A = {gate, s_gate, up, s_up, silu, s_silu, g, nullptr, nullptr, y_gate, y_up, s_max_gate, s_max_up, 0, 0, 0};
+    return silu_mul_launch(A, true, fp8_in, fp8_out, M, N, QB, s_dtype, (hipStream_t)stream);
 }

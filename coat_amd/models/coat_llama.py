@@ -26,7 +26,8 @@ from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_If
                                             fp8_division_transpose, fp8_linear_backward, fp8_linear_forward,
                                             fp8_mul_backward, fp8_mul_forward, fp8_quantize_pertensor,
                                             fp8_quantize_pertensor_transpose, fp8_rmsnorm_backward,
-                                            fp8_rmsnorm_forward, fp8_silu_backward, fp8_silu_forward, fp8_transpose)
+                                            fp8_rmsnorm_forward, fp8_silu_backward, fp8_silu_forward, fp8_silu_mul_backward,
+                                            fp8_silu_mul_forward, fp8_transpose)
 from ..utils._fp8_quantization_config import QuantizationConfig
 from ..utils._fp8_weightcache import FP8CacheWeightModule
 from ..utils._fp8manager import FP8Manager
@@ -275,8 +276,9 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
                                             group_size)
         up_x, up_s = fp8_linear_forward(ln_x, ln_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits), w2_s, True,
                                         group_size)
-        silu_x, silu_s = fp8_silu_forward(gate_x, gate_s, group_size)
-        mul_x, mul_s, mul_x_t = fp8_mul_forward(silu_x, silu_s, up_x, up_s, group_size, transpose_output_2d=True)
+        # one kernel for fp8_silu_forward + fp8_mul_forward of the reference (:664-668), same tensors
+        silu_x, silu_s, mul_x, mul_s, mul_x_t = fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, group_size,
+                                                                      transpose_output_2d=True)
         fc3_x = fp8_linear_forward(mul_x, mul_s, _forward_weight(w3_origin, w3, w3_s, qargs, fwobits), w3_s, False,
                                    group_size)
         fp_x, (out_x, out_s) = fp8_add_Ifp_Ifp_Ofp_Og16(re_x, fc3_x, mul_x.dtype, group_size)
@@ -305,10 +307,9 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
         fc3_g, weight3_grad = fp8_linear_backward(mul_x_t, mul_s, out_g, out_gs_max, out_g_t, w3_t, w3_s, group_size)
         del out_g, out_g_t, w3_t
         # element-wise product (1 = gate branch, 2 = up branch) and SiLU
-        mul_g1, (mul_g2, mul_gs2, mul_g2_t) = fp8_mul_backward(silu_x, silu_s, up_x, up_s, fc3_g, group_size,
-                                                              fwobits["babit"], output_quantized_transpose=True)
-        silu_g, silu_gs, silu_g_t = fp8_silu_backward(gate_x, gate_s, mul_g1, group_size, fwobits["babit"],
-                                                      output_quantized_transpose=True)
+        # one kernel for fp8_mul_backward + fp8_silu_backward of the reference (:741-748), same tensors
+        (silu_g, silu_gs, silu_g_t), (mul_g2, mul_gs2, mul_g2_t) = fp8_silu_mul_backward(
+            gate_x, gate_s, up_x, up_s, silu_x, silu_s, fc3_g, group_size, fwobits["babit"])
         # gate / up projections
         w1_t = _backward_weight_t(w1_saved, w1_s, qargs, fwobits)
         w2_t = _backward_weight_t(w2_saved, w2_s, qargs, fwobits)

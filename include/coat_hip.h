@@ -106,6 +106,21 @@ int coat_fp8_add_fwd(const void* x1, const void* x2, void* y, void* q, void* s_q
 int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s_y, float* s_max, int fp8_out, int64_t M,
                      int64_t N, int QB, void* stream);
 
+/* SiLU(gate) * up in one pass; bit-identical to the reference's two-kernel chains, which re-read the FP8 SiLU output
+ * (forward: rq/silu_fwd.py:152 then rq/mul_fwd.py:191) and round-trip the bf16 gradient of the product (backward:
+ * rq/mul_bwd.py:221 then rq/silu_bwd.py:170).  No single counterpart in the reference; used by the MLP module.
+ * forward: q_silu / s_silu = per-group FP8 SiLU(gate) with bf16 scales (saved for backward), y = bf16 product of the
+ * dequantized SiLU and up, *s_max = max of the product's fp32 group scales (fp8 = format of gate / up / silu). */
+int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
+                              int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M, int64_t N,
+                              int QB, void* stream);
+/* backward: y_up = bf16(g * silu), y_gate = bf16(silu'(gate) * bf16(g * up)); *s_max_* = max of their fp32 group
+ * scales for the format fp8_out (the per-tensor division that follows is coat_fp8_division). */
+int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, const void* up, const void* s_up, const void* silu,
+                               const void* s_silu, int fp8_in, int s_dtype, const void* g, void* y_gate,
+                               float* s_max_gate, void* y_up, float* s_max_up, int fp8_out, int64_t M, int64_t N,
+                               int QB, void* stream);
+
 /* rq/func_rmsnorm.py:223 fp8_rmsnorm_forward (kernel :54-111): y = bf16(x * rstd * w); s_row [M] bf16 row scales
  * (max|y| + 1e-10) / fp8max; rstd [M] fp32; s_max as above.  N <= 16384, N % 16 == 0. */
 int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype, void* y,

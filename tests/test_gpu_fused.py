@@ -181,6 +181,33 @@ def test_layernorm_forward_backward(dev, N, affine):
         assert qy3.shape == (4, M // 4, N) and qyt3.shape == (N, M) and torch.equal(b(qy3).reshape(M, N), b(qy))
 
 
+@pytest.mark.parametrize("fp8,QBv", [("E4M3", 16), ("E4M3", 64)])
+def test_fused_silu_mul_equals_the_two_kernel_chains(dev, fp8, QBv):
+    """coat_fp8_silu_mul_forward / _backward against fp8_silu_forward -> fp8_mul_forward and fp8_mul_backward ->
+    fp8_silu_backward (each checked against the oracle above): every output tensor bit for bit."""
+    rq = _rq()
+    M, N = 384, 1024
+    gate, up, g = rand(30, shape=(M, N)), rand(31, shape=(M, N)), rand(32, 0.01, shape=(M, N))
+    qg, sg = rq.fp8_quantize(gate.to(dev), QBv, fp8)
+    qu, su = rq.fp8_quantize(up.to(dev), QBv, fp8)
+    silu_x, silu_s = rq.fp8_silu_forward(qg, sg, QBv)
+    mul_x, mul_s, mul_x_t = rq.fp8_mul_forward(silu_x, silu_s, qu, su, QBv, transpose_output_2d=True)
+    f_silu_x, f_silu_s, f_mul_x, f_mul_s, f_mul_x_t = rq.fp8_silu_mul_forward(qg, sg, qu, su, QBv, transpose_output_2d=True)
+    assert torch.equal(b(f_silu_x), b(silu_x)) and torch.equal(f_silu_s, silu_s)
+    assert f_mul_s.item() == mul_s.item() and torch.equal(b(f_mul_x), b(mul_x)) and torch.equal(b(f_mul_x_t), b(mul_x_t))
+    gd = g.to(dev)
+    g1, (uq, us, uqt) = rq.fp8_mul_backward(silu_x, silu_s, qu, su, gd, QBv, "E5M2", output_quantized_transpose=True)
+    gq, gs, gqt = rq.fp8_silu_backward(qg, sg, g1, QBv, "E5M2", output_quantized_transpose=True)
+    (f_gq, f_gs, f_gqt), (f_uq, f_us, f_uqt) = rq.fp8_silu_mul_backward(qg, sg, qu, su, silu_x, silu_s, gd, QBv, "E5M2")
+    assert f_gs.item() == gs.item() and torch.equal(b(f_gq), b(gq)) and torch.equal(b(f_gqt), b(gqt))
+    assert f_us.item() == us.item() and torch.equal(b(f_uq), b(uq)) and torch.equal(b(f_uqt), b(uqt))
+    # batched inputs keep their leading dimension
+    q3, s3 = qg.reshape(2, M // 2, N), sg.reshape(2, M // 2, N // QBv)
+    u3, us3 = qu.reshape(2, M // 2, N), su.reshape(2, M // 2, N // QBv)
+    o = rq.fp8_silu_mul_forward(q3, s3, u3, us3, QBv)
+    assert o[0].shape == (2, M // 2, N) and o[2].shape == (2, M // 2, N) and torch.equal(b(o[2]).reshape(M, N), b(mul_x))
+
+
 def test_larger_groups_and_float32_scales(dev):
     rq = _rq()
     x1, x2 = rand(13, shape=(128, 512)), rand(14, shape=(128, 512))
