@@ -3,12 +3,12 @@ Reference: coat/activation/real_quantization/_division.py:153-207."""
 import torch
 
 from ... import _hip
-from .common import FP8_MAX_VALUE, SCALE_MIN_THRES, as_fp8_dtype, flatten_2d, no_stochastic, restore
+from .common import FP8_MAX_VALUE, SCALE_MIN_THRES, as_fp8_dtype, flatten_2d, new_max, no_stochastic, restore
 
 
 def absmax_scale(x, fp8type):
     """(x.abs().max() + 1e-10) / fp8max in x's dtype (reference :178-179), one pass over x."""
-    amax = torch.zeros((), dtype=torch.float32, device=x.device)
+    amax = new_max(x.device)
     _hip.check(_hip.lib().coat_absmax(_hip.ptr(x), _hip.dt(x), _hip.ptr(amax), x.numel(), _hip.stream(x.device)), "absmax")
     return (amax.to(x.dtype) + SCALE_MIN_THRES) / FP8_MAX_VALUE[fp8type]
 

@@ -2,7 +2,7 @@
 import torch
 
 from ... import _hip
-from .common import flatten_2d
+from .common import flatten_2d, new_max  # noqa: F401  (re-exported for the fused launchers)
 
 
 def prep_pg(x, s_x):
@@ -17,8 +17,3 @@ def prep_bf16(g):
     if g.dtype != torch.bfloat16:
         g = g.to(torch.bfloat16)
     return _hip.dense(g)
-
-
-def new_max(device):
-    """Zero-initialised fp32 device scalar for the order-independent atomic maximum of the group scales."""
-    return torch.zeros((), dtype=torch.float32, device=device)

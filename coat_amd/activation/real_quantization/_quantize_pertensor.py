@@ -4,7 +4,7 @@ import torch
 
 from ... import _hip
 from ._division import _division
-from .common import convert_str_to_fp8, flatten_2d, no_stochastic, restore
+from .common import convert_str_to_fp8, flatten_2d, new_max, no_stochastic, restore
 
 
 def group_scales_and_max(x, QB, fp8type, scale_dtype=torch.bfloat16, want_pg=True):
@@ -14,7 +14,7 @@ def group_scales_and_max(x, QB, fp8type, scale_dtype=torch.bfloat16, want_pg=Tru
     the maximum equals the reference's ``s_y.max()`` over the rounded scales (reference :139)."""
     M, N = x.shape
     s_pg = torch.empty((M, N // QB), dtype=scale_dtype, device=x.device) if want_pg else None
-    s_max = torch.zeros((), dtype=torch.float32, device=x.device)
+    s_max = new_max(x.device)
     _hip.check(_hip.lib().coat_fp8_group_scales(_hip.ptr(x), _hip.dt(x), _hip.ptr(s_pg), _hip.dt(scale_dtype),
                                                 _hip.ptr(s_max), M, N, QB, _hip.fp8(fp8type), _hip.stream(x.device)),
                "fp8_group_scales")

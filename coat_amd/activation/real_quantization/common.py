@@ -43,3 +43,26 @@ def no_stochastic(stochastic):
         raise NotImplementedError(
             "stochastic rounding is not built (no caller in the reference enables it: "
             "fp8linear.py:88,101; coat_llama.py:297,335,749)")
+
+
+_MAX_POOL = {}
+_MAX_POOL_SIZE = 1024
+
+
+def new_max(device):
+    """Zero-initialised fp32 device scalar for the order-independent atomic maximum of the group scales.
+
+    Scalars are handed out from a zero-filled pool (one fill kernel per 1024 of them instead of one each; a slot is
+    never reused, and the pool lives as long as any of its slots).  Pools are kept per device and stream, so a slot is
+    always used on the stream that zeroed it."""
+    device = torch.device(device)
+    if device.type != "cuda":
+        return torch.zeros((), dtype=torch.float32, device=device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    pool = _MAX_POOL.get(key)
+    if pool is None or pool[1] >= _MAX_POOL_SIZE:
+        pool = [torch.zeros(_MAX_POOL_SIZE, dtype=torch.float32, device=device), 0]
+        _MAX_POOL[key] = pool
+    i = pool[1]
+    pool[1] = i + 1
+    return pool[0][i]
