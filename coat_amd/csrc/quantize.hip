@@ -293,18 +293,18 @@ __global__ __launch_bounds__(256) void k_division_transpose(const void* __restri
 // Tile = TM x 64 fp32 values in LDS (pitch 65 words).  Phase 1 does the row-direction groups exactly like
 // k_quantize_pg and parks the fp32 values in LDS; phase 2 gives every lane a (column, 16-row chunk) job:
 // amax over the chunk (and over QB/16 neighbouring lanes), quantize, one 16-byte store into qt.
-template <int XDT, int SDT, int KIND, int QB, int TM>
+template <int XDT, int SDT, int KIND, int QB, int TM, int TN>
 __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restrict__ x, void* __restrict__ q,
                                                              void* __restrict__ s_out, void* __restrict__ qt,
                                                              void* __restrict__ st_out, int64_t M, int64_t N) {
     constexpr int VEC = VecOf<XDT>::kVec;
     constexpr int ESIZE = 16 / VEC;
     constexpr int LPG = QB / VEC;
-    constexpr int PITCH = kTileN + 1;
-    static_assert(QB <= kTileN && TM % QB == 0, "tile must hold whole groups in both directions");
-    __shared__ float tile[TM * PITCH];
+    constexpr int PITCH = TN + 1;
+    static_assert(QB <= TN && TM % QB == 0, "tile must hold whole groups in both directions");
+    extern __shared__ float tile[];  // TM x PITCH fp32 (dynamic: 65 KiB for the 128 x 128 tile of QB = 128)
     enable_fp8_saturation();
-    const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = (N + kTileN - 1) / kTileN;
+    const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
     const int64_t SN = N / QB, SM = M / QB;
     // A block quantizes two tiles that are neighbours along n, so the two 64-byte halves of every 128-byte line of q
     // come from the same CU within microseconds and merge in L2.  Blocks are dispatched round-robin over the 8 XCDs
@@ -315,10 +315,10 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
     const int64_t tm = (int64_t)(blockIdx.x >> 3) % tiles_m;
     if (2 * pair >= tiles_n) return;
     const int64_t t_begin = 0, t_end = min((int64_t)2, tiles_n - 2 * pair);
-#define COAT_QT_ORIGIN(t) const int64_t m0 = tm * TM, n0 = (2 * pair + (t)) * kTileN
+#define COAT_QT_ORIGIN(t) const int64_t m0 = tm * TM, n0 = (2 * pair + (t)) * TN
 
     // phase-1 jobs: VEC consecutive elements (16 bytes); a row of the tile is 64/VEC jobs (a multiple of LPG)
-    constexpr int JPR = kTileN / VEC;
+    constexpr int JPR = TN / VEC;
     constexpr int JOBS = TM * JPR;
     static_assert(JOBS % 256 == 0, "phase 1 keeps all lanes of a group in the same iteration");
     constexpr int NIT = JOBS / 256;
@@ -362,7 +362,7 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
         // neighbouring 16-byte pieces of one qt row; groups of QB rows are QB/16 neighbouring lanes.
         constexpr int MC = TM / 16;
         constexpr int LPG_T = QB / 16;
-        constexpr int JOBS2 = MC * kTileN;
+        constexpr int JOBS2 = MC * TN;
         static_assert(JOBS2 % 256 == 0, "phase 2 keeps all lanes of a group in the same iteration");
         for (int job = threadIdx.x; job < JOBS2; job += 256) {
             int mc = job % MC, col = job / MC;
@@ -562,22 +562,34 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
     if (M * N == 0) return COAT_OK;
     if (!x || !q || !s || !qt || !st_out) return COAT_EINVAL;
     if (!coat_aligned16(x) || !coat_aligned16(q) || !coat_aligned16(qt)) return COAT_EALIGN;
-    if (QB > 64) return COAT_ESHAPE;  // column groups must fit the 64-wide tile
+    if (QB > 128) return COAT_ESHAPE;  // groups must fit the tile in both directions (the reference tunes 16..128)
     hipStream_t st = (hipStream_t)stream;
-    constexpr int TM = 64;
-    const int64_t tiles_m = (M + TM - 1) / TM, pairs_n = ((N + kTileN - 1) / kTileN + 1) / 2;
+    // 64 x 64 tiles for QB <= 64, one 128 x 128 tile shape for QB = 128
+    const int T = QB == 128 ? 128 : 64;
+    const int64_t tiles_m = (M + T - 1) / T, pairs_n = ((N + T - 1) / T + 1) / 2;
     const int64_t blocks = ((pairs_n + 7) / 8) * 8 * tiles_m;  // see the kernel for the block -> tile-pair mapping
     if (blocks >= ((int64_t)1 << 31)) return COAT_ESHAPE;
-#define LAUNCH_QT(QBV)                                                                                               \
+#define LAUNCH_QT(QBV, TV)                                                                                           \
     DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                 \
-        hipLaunchKernelGGL((k_quantize_transpose<XDT, SDT, KIND, QBV, TM>), dim3((unsigned)blocks), dim3(256), 0, st, \
-                           x, q, s, qt, st_out, M, N);                                                               \
+        constexpr int kLds = TV * (TV + 1) * 4;                                                                      \
+        if (kLds > 65536) {                                                                                          \
+            static bool attr_set = false;                                                                            \
+            if (!attr_set) {                                                                                         \
+                hipError_t e = hipFuncSetAttribute((const void*)k_quantize_transpose<XDT, SDT, KIND, QBV, TV, TV>,   \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLds);                \
+                if (e != hipSuccess) return (int)e;                                                                  \
+                attr_set = true;                                                                                     \
+            }                                                                                                        \
+        }                                                                                                            \
+        hipLaunchKernelGGL((k_quantize_transpose<XDT, SDT, KIND, QBV, TV, TV>), dim3((unsigned)blocks), dim3(256),   \
+                           kLds, st, x, q, s, qt, st_out, M, N);                                                     \
         return coat_launch_status();                                                                                 \
     })))
     switch (QB) {
-        case 16: LAUNCH_QT(16); break;
-        case 32: LAUNCH_QT(32); break;
-        case 64: LAUNCH_QT(64); break;
+        case 16: LAUNCH_QT(16, 64); break;
+        case 32: LAUNCH_QT(32, 64); break;
+        case 64: LAUNCH_QT(64, 64); break;
+        case 128: LAUNCH_QT(128, 128); break;
         default: return COAT_ESHAPE;
     }
 #undef LAUNCH_QT

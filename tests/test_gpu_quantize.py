@@ -75,7 +75,8 @@ def test_fp8_quantize_3d_and_scale_dtype(dev):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("fp8,QB,M,N", [("E4M3", 16, 128, 192), ("E5M2", 16, 64, 64), ("E4M3", 32, 96, 160),
-                                        ("E4M3", 64, 128, 128), ("E4M3", 16, 16, 16), ("E4M3", 16, 208, 80)])
+                                        ("E4M3", 64, 128, 128), ("E4M3", 16, 16, 16), ("E4M3", 16, 208, 80),
+                                        ("E4M3", 128, 384, 640), ("E5M2", 128, 128, 128)])
 def test_fp8_quantize_transpose_bit_exact(dev, dtype, fp8, QB, M, N):
     rq = _rq()
     x = make_x(M, N, 4, dtype)
@@ -83,6 +84,10 @@ def test_fp8_quantize_transpose_bit_exact(dev, dtype, fp8, QB, M, N):
         x[:32, :128] = special_x(dtype)
     (q, s), (qt, st) = rq.fp8_quantize_transpose(x.to(dev), QB, fp8)
     (wq, ws), (wqt, wst) = R.fp8_quantize_transpose(x, QB, fp8)
+    if QB == 128:  # the reference's own test calls it with fp32 scales (tests/test_fp8_quantize.py:70)
+        (q32, s32), (qt32, st32) = rq.fp8_quantize_transpose(x.to(dev), QB, fp8, scale_dtype=torch.float32)
+        (_, ws32), (_, wst32) = R.fp8_quantize_transpose(x, QB, fp8, scale_dtype=torch.float32)
+        assert torch.equal(s32.cpu(), ws32) and torch.equal(st32.cpu(), wst32) and eq_bytes(q32, q) and eq_bytes(qt32, qt)
     assert qt.shape == (N, M) and st.shape == (N, M // QB)
     assert torch.equal(s.cpu(), ws) and eq_bytes(q, wq)
     assert torch.equal(st.cpu(), wst) and eq_bytes(qt, wqt)
