@@ -18,6 +18,7 @@ _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 _FP8 = {torch.float8_e4m3fn: E4M3, torch.float8_e5m2: E5M2}
 
 _vp, _i, _i64, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+_u64 = ctypes.c_uint64
 
 # name -> argument types (all functions return int except the two string getters)
 SIGNATURES = {
@@ -26,6 +27,7 @@ SIGNATURES = {
     "coat_fp8_group_scales": [_vp, _i, _vp, _i, _vp, _i64, _i64, _i, _i, _vp],
     "coat_absmax": [_vp, _i, _vp, _i64, _vp],
     "coat_fp8_division": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],
+    "coat_fp8_division_stochastic": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _u64, _vp],
     "coat_fp8_transpose": [_vp, _vp, _i64, _i64, _vp],
     "coat_fp8_dequantize": [_vp, _i, _vp, _i, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_silu_forward": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],

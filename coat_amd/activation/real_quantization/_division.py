@@ -3,7 +3,10 @@ Reference: coat/activation/real_quantization/_division.py:153-207."""
 import torch
 
 from ... import _hip
-from .common import FP8_MAX_VALUE, SCALE_MIN_THRES, as_fp8_dtype, flatten_2d, new_max, no_stochastic, restore
+from .common import FP8_MAX_VALUE, SCALE_MIN_THRES, as_fp8_dtype, flatten_2d, new_max, restore
+
+# the seed the reference's kernels pass to tl.rand (reference :110; _division_transpose.py:117)
+STOCHASTIC_SEED = 0
 
 
 def absmax_scale(x, fp8type):
@@ -13,7 +16,7 @@ def absmax_scale(x, fp8type):
     return (amax.to(x.dtype) + SCALE_MIN_THRES) / FP8_MAX_VALUE[fp8type]
 
 
-def _division(x, fp8type, s_y, want_q, want_qt, what):
+def _division(x, fp8type, s_y, want_q, want_qt, what, stochastic=False):
     M, N = x.shape
     if s_y is None:
         s_y = absmax_scale(x, fp8type)
@@ -22,15 +25,20 @@ def _division(x, fp8type, s_y, want_q, want_qt, what):
     s_dev = s_y if s_y.is_cuda else s_y.to(x.device)
     y = torch.empty_like(x, dtype=fp8type) if want_q else None
     y_t = torch.empty((N, M), dtype=fp8type, device=x.device) if want_qt else None
-    _hip.check(_hip.lib().coat_fp8_division(_hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.dt(s_dev), _hip.ptr(y),
-                                            _hip.ptr(y_t), M, N, _hip.fp8(fp8type), _hip.stream(x.device)), what)
+    if stochastic:
+        _hip.check(_hip.lib().coat_fp8_division_stochastic(
+            _hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.dt(s_dev), _hip.ptr(y), _hip.ptr(y_t), M, N,
+            _hip.fp8(fp8type), STOCHASTIC_SEED, _hip.stream(x.device)), what)
+    else:
+        _hip.check(_hip.lib().coat_fp8_division(_hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.dt(s_dev), _hip.ptr(y),
+                                                _hip.ptr(y_t), M, N, _hip.fp8(fp8type), _hip.stream(x.device)), what)
     return y, s_y, y_t
 
 
 def fp8_division(x, QB, fp8type, s_y=None, stochastic=False):
-    """x -> (y fp8, s_y); y = fp8(x / float(s_y)); s_y defaults to (absmax + 1e-10) / fp8max."""
-    no_stochastic(stochastic)
+    """x -> (y fp8, s_y); y = fp8(x / float(s_y)); s_y defaults to (absmax + 1e-10) / fp8max.
+    stochastic: the reference's noise-then-round branch (reference :96-112, :130-150), same Philox stream."""
     x, batch = flatten_2d(x)
     x = _hip.dense(x)
-    y, s_y, _ = _division(x, as_fp8_dtype(fp8type), s_y, True, False, "fp8_division")
+    y, s_y, _ = _division(x, as_fp8_dtype(fp8type), s_y, True, False, "fp8_division", stochastic)
     return restore(y, batch), s_y

@@ -4,7 +4,7 @@ import torch
 
 from ... import _hip
 from ._division import _division
-from .common import convert_str_to_fp8, flatten_2d, new_max, no_stochastic, restore
+from .common import convert_str_to_fp8, flatten_2d, new_max, restore
 
 
 def group_scales_and_max(x, QB, fp8type, scale_dtype=torch.bfloat16, want_pg=True):
@@ -22,11 +22,10 @@ def group_scales_and_max(x, QB, fp8type, scale_dtype=torch.bfloat16, want_pg=Tru
 
 
 def fp8_quantize_pertensor(x, QB, fp8type, stochastic=False, scale_dtype=torch.bfloat16):
-    """Returns (y fp8, s_y_max 0-dim, s_y per-group)."""
-    no_stochastic(stochastic)
+    """Returns (y fp8, s_y_max 0-dim, s_y per-group).  stochastic goes to the division pass (reference :140)."""
     x, batch = flatten_2d(x)
     x = _hip.dense(x)
     fp8type = convert_str_to_fp8[fp8type]  # the reference accepts only the string here (:118)
     s_y, s_y_max = group_scales_and_max(x, QB, fp8type, scale_dtype)
-    y, s_y_max, _ = _division(x, fp8type, s_y_max, True, False, "fp8_quantize_pertensor")
+    y, s_y_max, _ = _division(x, fp8type, s_y_max, True, False, "fp8_quantize_pertensor", stochastic)
     return restore(y, batch), s_y_max, restore(s_y, batch)

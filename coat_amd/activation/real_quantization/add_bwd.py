@@ -5,12 +5,12 @@ import torch
 from ... import _hip
 from ._division import _division
 from ._fused import new_max, prep_bf16
-from .common import as_fp8_dtype, flatten_2d, no_stochastic, restore
+from .common import as_fp8_dtype, flatten_2d, restore
 
 
 def fp8_add_Ifp_Ifp_Ofp_Opt(x1, x2, QB, fp8type, stochastic=False):
-    """Returns (y bf16, (q fp8 per-tensor, s_max 0-dim, s per-group)); the division quantizes the bf16 sum."""
-    no_stochastic(stochastic)
+    """Returns (y bf16, (q fp8 per-tensor, s_max 0-dim, s per-group)); the division quantizes the bf16 sum
+    (stochastic applies to that division, reference :192)."""
     _, batch = flatten_2d(x1)
     for t in (x1, x2):
         if t.dtype != torch.bfloat16:
@@ -24,5 +24,6 @@ def fp8_add_Ifp_Ifp_Ofp_Opt(x1, x2, QB, fp8type, stochastic=False):
     s_max = new_max(x1.device)
     _hip.check(_hip.lib().coat_fp8_add_bwd(_hip.ptr(x1), _hip.ptr(x2), _hip.ptr(y1), _hip.ptr(s_y2), _hip.ptr(s_max),
                                            _hip.fp8(fp8type), M, N, QB, _hip.stream(x1.device)), "fp8_add_Ifp_Ifp_Ofp_Opt")
-    qy2, s_y2_max, _ = _division(y1, fp8type, s_max.to(torch.bfloat16), True, False, "fp8_add_Ifp_Ifp_Ofp_Opt")
+    qy2, s_y2_max, _ = _division(y1, fp8type, s_max.to(torch.bfloat16), True, False, "fp8_add_Ifp_Ifp_Ofp_Opt",
+                                 stochastic)
     return restore(y1, batch), (restore(qy2, batch), s_y2_max, restore(s_y2, batch))

@@ -38,11 +38,10 @@ def restore(y, batch):
     return y if batch is None else y.reshape(batch, -1, y.shape[-1])
 
 
-def no_stochastic(stochastic):
+def no_stochastic(stochastic, why):
+    """For the two entry points whose stochastic branch does not compile in the reference itself."""
     if stochastic:
-        raise NotImplementedError(
-            "stochastic rounding is not built (no caller in the reference enables it: "
-            "fp8linear.py:88,101; coat_llama.py:297,335,749)")
+        raise NotImplementedError(f"stochastic=True is not available here: {why}")
 
 
 _MAX_POOL = {}

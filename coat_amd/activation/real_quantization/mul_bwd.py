@@ -4,13 +4,14 @@ import torch
 from ... import _hip
 from ._division import _division
 from ._fused import new_max, prep_bf16, prep_pg
-from .common import as_fp8_dtype, no_stochastic, restore
+from .common import as_fp8_dtype, restore
 
 
 def fp8_mul_backward(x1, s_x1, x2, s_x2, g, QB, fp8type, stochastic=False, output_quantized_transpose=False):
     """Returns (y1 bf16, (y2 bf16, s_y2)) or (y1 bf16, (qy2, s_y2_max, qy2_t)):
-    y1 = g * x2 is the gradient of x1, y2 = g * x1 the gradient of x2."""
-    no_stochastic(stochastic)
+    y1 = g * x2 is the gradient of x1, y2 = g * x1 the gradient of x2.
+    ``stochastic`` is accepted and has no effect, as in the reference (mul_bwd.py:236-239 allocates noise that the
+    kernel never reads, and the division at :305 is called without the flag)."""
     x1, s_x1, batch = prep_pg(x1, s_x1)
     x2, s_x2, _ = prep_pg(x2, s_x2)
     g = prep_bf16(g)

@@ -4,12 +4,12 @@ import torch
 from ... import _hip
 from ._division import _division
 from ._fused import new_max, prep_bf16, prep_pg
-from .common import as_fp8_dtype, no_stochastic, restore
+from .common import as_fp8_dtype, restore
 
 
 def fp8_silu_backward(x, s_x, g, QB, fp8type, stochastic=False, output_quantized_transpose=False):
-    """Returns (y bf16, s_y per-group) or, with output_quantized_transpose, (qy, s_y_max, qy_t [N, M])."""
-    no_stochastic(stochastic)
+    """Returns (y bf16, s_y per-group) or, with output_quantized_transpose, (qy, s_y_max, qy_t [N, M]).
+    ``stochastic`` is accepted and has no effect, as in the reference (silu_bwd.py:170-242 never reads it)."""
     x, s_x, batch = prep_pg(x, s_x)
     g = prep_bf16(g)
     M, N = x.shape

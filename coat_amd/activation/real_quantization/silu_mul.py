@@ -7,7 +7,7 @@ import torch
 from ... import _hip
 from ._division import _division
 from ._fused import new_max, prep_bf16, prep_pg
-from .common import as_fp8_dtype, no_stochastic, restore
+from .common import as_fp8_dtype, restore
 
 
 def fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, QB, transpose_output_2d=False):
@@ -37,8 +37,8 @@ def fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, QB, transpose_output_2d=Fal
 def fp8_silu_mul_backward(gate_x, gate_s, up_x, up_s, silu_x, silu_s, g, QB, fp8type, stochastic=False):
     """Equivalent to ``mul_g1, up_grad = fp8_mul_backward(silu_x, silu_s, up_x, up_s, g, QB, fp8type,
     output_quantized_transpose=True)`` followed by ``gate_grad = fp8_silu_backward(gate_x, gate_s, mul_g1, QB, fp8type,
-    output_quantized_transpose=True)``.  Returns ((gate_q, gate_s, gate_q_t), (up_q, up_s, up_q_t))."""
-    no_stochastic(stochastic)
+    output_quantized_transpose=True)``.  Returns ((gate_q, gate_s, gate_q_t), (up_q, up_s, up_q_t)).
+    ``stochastic`` has no effect, as in both of those reference functions."""
     gate_x, gate_s, batch = prep_pg(gate_x, gate_s)
     up_x, up_s, _ = prep_pg(up_x, up_s)
     silu_x, silu_s, _ = prep_pg(silu_x, silu_s)

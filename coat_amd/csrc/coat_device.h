@@ -119,6 +119,47 @@ __device__ __forceinline__ float div_by_scale(float x, float s, float r) {
 }
 constexpr float kMinFastDivScale = 0x1p-60f;
 
+// ------------------------------------------------------------------------------------------------ stochastic rounding
+// Philox-4x32, 10 rounds, counter (c0, 0, 0, 0), key (k0, k1): first output word.  This is the stream the
+// reference draws with tl.rand(seed, offset) (coat/activation/real_quantization/_division.py:107-110):
+// key = the 64-bit seed, c0 = the element's linear index.
+__device__ __forceinline__ uint32_t philox4x32_10_word0(uint32_t c0, uint32_t k0, uint32_t k1) {
+    uint32_t c1 = 0, c2 = 0, c3 = 0;
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        const uint32_t hi_b = __umulhi(0xCD9E8D57u, c2), lo_b = 0xCD9E8D57u * c2;
+        const uint32_t hi_a = __umulhi(0xD2511F53u, c0), lo_a = 0xD2511F53u * c0;
+        c0 = hi_b ^ c1 ^ k0;
+        c2 = hi_a ^ c3 ^ k1;
+        c1 = lo_b;
+        c3 = lo_a;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return c0;
+}
+// Random word -> fp32 in [0, 1) the way Triton's uint_to_uniform_float does: fold the negative half of the
+// int32 range onto the non-negative one, convert (round to nearest even), scale by just under 2^-31.
+__device__ __forceinline__ float uniform_from_word(uint32_t w) {
+    int32_t x = (int32_t)w;
+    x = x < 0 ? -x - 1 : x;
+    return (float)x * 4.6566127342e-10f;
+}
+// The reference's _stochastic_rounding (coat/activation/real_quantization/_division.py:130-150): add
+// noise * (one FP8 step of q's binade) to |q|, clamp to the binade, keep the sign; the caller then converts with
+// round-to-nearest.  Below twice the smallest subnormal the step is the smallest subnormal itself and the
+// ceiling 2^m_bit times it; the lower clamp lifts zeros to the smallest subnormal, as the reference does.
+template <int KIND> __device__ __forceinline__ float stochastic_perturb(float q, float noise) {
+    constexpr float kSubMin = KIND == kE4M3 ? 0x1p-9f : 0x1p-16f;
+    constexpr float kSteps = KIND == kE4M3 ? 8.0f : 4.0f;  // 2^m_bit
+    const float e = fmaxf(u2f(f2u(q) & 0x7F800000u), kSubMin);
+    const bool sub = e == kSubMin;
+    const float nz = (e * noise) * (sub ? 1.0f : 1.0f / kSteps);  // division by a power of two, exact either way
+    float a = fabsf(q) + nz;
+    a = fminf(fmaxf(a, e), (sub ? kSteps : 2.0f) * e);
+    return u2f(f2u(a) | (f2u(q) & 0x80000000u));
+}
+
 // ------------------------------------------------------------------------------------------------ cross-lane
 // DPP controls: quad_perm(1,0,3,2)=0xB1, quad_perm(2,3,0,1)=0x4E, row_half_mirror=0x141, row_mirror=0x140.
 template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {

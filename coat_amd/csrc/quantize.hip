@@ -63,6 +63,19 @@ template <int KIND, int VEC> __device__ __forceinline__ void quantize_vec_slow(c
     for (int i = 0; i < VEC / 4; i++)
         out[i] = cvt4_fp8<KIND>(v[4 * i] / s, v[4 * i + 1] / s, v[4 * i + 2] / s, v[4 * i + 3] / s);
 }
+// Stochastic variant: the quotient of element (e0 + k) is perturbed with Philox noise drawn at that linear index.
+template <int KIND, int VEC>
+__device__ __forceinline__ void quantize_vec_sr(const float* v, float s, float r, bool fast, uint32_t e0, uint32_t k0,
+                                                uint32_t k1, uint32_t* out) {
+    float t[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        const float qv = fast ? div_by_scale(v[k], s, r) : v[k] / s;
+        t[k] = stochastic_perturb<KIND>(qv, uniform_from_word(philox4x32_10_word0(e0 + (uint32_t)k, k0, k1)));
+    }
+#pragma unroll
+    for (int i = 0; i < VEC / 4; i++) out[i] = cvt4_fp8<KIND>(t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3]);
+}
 template <int VEC> __device__ __forceinline__ void store_codes(void* q, int64_t e, const uint32_t* c) {
     if (VEC == 8) *(uint2*)((uint8_t*)q + e) = make_uint2(c[0], c[1]);
     else *(uint32_t*)((uint8_t*)q + e) = c[0];
@@ -140,10 +153,12 @@ __global__ __launch_bounds__(256) void k_absmax(const void* __restrict__ x, floa
 }
 
 // ------------------------------------------------------------------------------------------------
-// K4: per-tensor division over the flat array, q = fp8(x / float(*s)).
-template <int XDT, int SDT, int KIND, int UNROLL>
+// K4: per-tensor division over the flat array, q = fp8(x / float(*s)).  SR: stochastic rounding with the
+// Philox key (k0, k1) (the reference's branch, coat/activation/real_quantization/_division.py:96-112).
+template <int XDT, int SDT, int KIND, int UNROLL, bool SR>
 __global__ __launch_bounds__(256) void k_division(const void* __restrict__ x, const void* __restrict__ s_ptr,
-                                                   void* __restrict__ q, int64_t nvec, int64_t numel) {
+                                                   void* __restrict__ q, int64_t nvec, int64_t numel, uint32_t k0,
+                                                   uint32_t k1) {
     constexpr int VEC = VecOf<XDT>::kVec;
     enable_fp8_saturation();
     const float s = load_as_f32<SDT>(s_ptr, 0);
@@ -161,14 +176,17 @@ __global__ __launch_bounds__(256) void k_division(const void* __restrict__ x, co
         int64_t i = base + (int64_t)u * 256;
         if (i < nvec) {
             uint32_t c[VEC / 4];
-            if (fast) quantize_vec<KIND, VEC>(v[u], s, r, c);
+            if (SR) quantize_vec_sr<KIND, VEC>(v[u], s, r, fast, (uint32_t)(i * VEC), k0, k1, c);
+            else if (fast) quantize_vec<KIND, VEC>(v[u], s, r, c);
             else quantize_vec_slow<KIND, VEC>(v[u], s, c);
             store_codes<VEC>(q, i * VEC, c);
         }
     }
     if (blockIdx.x == 0 && threadIdx.x < numel - nvec * VEC) {
         int64_t e = nvec * VEC + threadIdx.x;
-        uint32_t w = cvt_pk_fp8<KIND>(load_as_f32<XDT>(x, e) / s, 0.0f, 0u, false);
+        float qv = load_as_f32<XDT>(x, e) / s;
+        if (SR) qv = stochastic_perturb<KIND>(qv, uniform_from_word(philox4x32_10_word0((uint32_t)e, k0, k1)));
+        uint32_t w = cvt_pk_fp8<KIND>(qv, 0.0f, 0u, false);
         ((uint8_t*)q)[e] = (uint8_t)(w & 0xFF);
     }
 }
@@ -244,10 +262,12 @@ __device__ __forceinline__ void store_tile_transposed(const uint32_t* tile, void
 
 // K5 / K6: q = fp8(x / *s) and/or its transpose; RAW = input already FP8 bytes (pure transpose).
 // Requires N % 16 == 0 and M % 16 == 0.
-template <int XDT, int SDT, int KIND, bool RAW, bool WRITE_Q, int TM>
+// SR: stochastic rounding, noise index = the element's linear index in x
+// (coat/activation/real_quantization/_division_transpose.py:103-119).
+template <int XDT, int SDT, int KIND, bool RAW, bool WRITE_Q, int TM, bool SR>
 __global__ __launch_bounds__(256) void k_division_transpose(const void* __restrict__ x, const void* __restrict__ s_ptr,
                                                              void* __restrict__ q, void* __restrict__ qt, int64_t M,
-                                                             int64_t N) {
+                                                             int64_t N, uint32_t k0, uint32_t k1) {
     __shared__ uint32_t tile[TM * kPitchDw];
     enable_fp8_saturation();
     const int64_t tiles_n = (N + kTileN - 1) / kTileN;
@@ -275,7 +295,8 @@ __global__ __launch_bounds__(256) void k_division_transpose(const void* __restri
                 for (int h = 0; h < 16 / VEC; h++) {
                     float v[VEC];
                     load_vec<XDT>(x, m * N + n + h * VEC, v);
-                    if (fast) quantize_vec<KIND, VEC>(v, s, r, c + h * (VEC / 4));
+                    if (SR) quantize_vec_sr<KIND, VEC>(v, s, r, fast, (uint32_t)(m * N + n + h * VEC), k0, k1, c + h * (VEC / 4));
+                    else if (fast) quantize_vec<KIND, VEC>(v, s, r, c + h * (VEC / 4));
                     else quantize_vec_slow<KIND, VEC>(v, s, c + h * (VEC / 4));
                 }
                 if (WRITE_Q) *(uint4*)((uint8_t*)q + m * N + n) = make_uint4(c[0], c[1], c[2], c[3]);
@@ -490,20 +511,22 @@ extern "C" int coat_absmax(const void* x, int x_dtype, float* amax, int64_t nume
     return COAT_EINVAL;
 }
 
-extern "C" int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
-                                 int64_t N, int fp8, void* stream) {
+template <bool SR>
+static int division_launch(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M, int64_t N,
+                           int fp8, uint64_t seed, void* stream) {
     if (M < 0 || N < 0) return COAT_EINVAL;
     if (M * N == 0) return COAT_OK;
     if (!x || !s || (!q && !qt)) return COAT_EINVAL;
     if (!coat_aligned16(x) || !coat_aligned16(q) || !coat_aligned16(qt)) return COAT_EALIGN;
     hipStream_t st = (hipStream_t)stream;
+    const uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
     if (!qt) {
         DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
             constexpr int VEC = VecOf<XDT>::kVec;
             int64_t numel = M * N, nvec = numel / VEC;
             int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
             if (blocks == 0) blocks = 1;
-            hipLaunchKernelGGL((k_division<XDT, SDT, KIND, 4>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, nvec, numel);
+            hipLaunchKernelGGL((k_division<XDT, SDT, KIND, 4, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, nvec, numel, k0, k1);
             return coat_launch_status();
         })));
         return COAT_EINVAL;
@@ -513,16 +536,28 @@ extern "C" int coat_fp8_division(const void* x, int x_dtype, const void* s, int 
     int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
     if (q) {
         DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
-            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, true, TM>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N);
+            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, true, TM, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N, k0, k1);
             return coat_launch_status();
         })));
     } else {
         DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
-            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, false, TM>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N);
+            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, false, TM, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N, k0, k1);
             return coat_launch_status();
         })));
     }
     return COAT_EINVAL;
+}
+
+extern "C" int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
+                                 int64_t N, int fp8, void* stream) {
+    return division_launch<false>(x, x_dtype, s, s_dtype, q, qt, M, N, fp8, 0, stream);
+}
+
+extern "C" int coat_fp8_division_stochastic(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt,
+                                            int64_t M, int64_t N, int fp8, uint64_t seed, void* stream) {
+    // the noise counter is the 32-bit linear element index, as in the reference's int32 offset arithmetic
+    if (M > 0 && N > 0 && M * N > ((int64_t)1 << 32)) return COAT_ESHAPE;
+    return division_launch<true>(x, x_dtype, s, s_dtype, q, qt, M, N, fp8, seed, stream);
 }
 
 extern "C" int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, void* stream) {
@@ -533,8 +568,8 @@ extern "C" int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, 
     if (!coat_aligned16(x) || !coat_aligned16(y)) return COAT_EALIGN;
     constexpr int TM = 64;
     int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
-    hipLaunchKernelGGL((k_division_transpose<kBF16, kBF16, kE4M3, true, false, TM>), dim3((unsigned)blocks), dim3(256), 0,
-                       (hipStream_t)stream, x, nullptr, nullptr, y, M, N);
+    hipLaunchKernelGGL((k_division_transpose<kBF16, kBF16, kE4M3, true, false, TM, false>), dim3((unsigned)blocks), dim3(256), 0,
+                       (hipStream_t)stream, x, nullptr, nullptr, y, M, N, 0u, 0u);
     return coat_launch_status();
 }
 

@@ -66,6 +66,14 @@ int coat_absmax(const void* x, int x_dtype, float* amax, int64_t numel, void* st
 int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
                       int64_t N, int fp8, void* stream);
 
+/* The same two entry points with stochastic=True (rq/_division.py:96-112 and :130-150 _stochastic_rounding;
+ * rq/_division_transpose.py:103-119): the quotient of element i (linear index in x) is moved up by
+ * noise_i * (one FP8 step of its binade), clamped to the binade, then rounded to nearest.  noise_i is Triton's
+ * tl.rand(seed, i): Philox-4x32-10, key = seed, counter = (i, 0, 0, 0), first word mapped to [0, 1).  The reference
+ * hard-codes seed 0.  M * N <= 2^32 (the counter is the 32-bit index). */
+int coat_fp8_division_stochastic(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
+                                 int64_t N, int fp8, uint64_t seed, void* stream);
+
 /* rq/_transpose.py:85 fp8_transpose (kernel :39-82): byte transpose, x [M,N] -> y [N,M]. */
 int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, void* stream);
 

@@ -87,8 +87,13 @@ def fp8_group_scales(x, QB, fp8type, scale_dtype=torch.bfloat16):
 
 
 def absmax_scale(x, fp8type):
-    """rq/_division.py:178-179: (x.abs().max() + 1e-10) / fp8max evaluated in x's own dtype."""
-    return (x.abs().max() + SCALE_MIN_THRES) / FP8_MAX_VALUE[_fp8(fp8type)]
+    """rq/_division.py:178-179: (x.abs().max() + 1e-10) / fp8max evaluated in x's own dtype, on the device.
+    torch's device kernel for a tensor divided by a Python number multiplies by the fp32 reciprocal of the number
+    (aten/src/ATen/native/cuda/BinaryDivTrueKernel.cu, the CPU-scalar branch); the CPU kernel divides.  The
+    reference runs on the device, so the reciprocal form is the one restated here."""
+    a = (x.abs().max() + SCALE_MIN_THRES).float()
+    inv = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(FP8_MAX_VALUE[_fp8(fp8type)], dtype=torch.float32)
+    return (a * inv).to(x.dtype)
 
 
 def fp8_division(x, QB, fp8type, s_y=None):

@@ -179,3 +179,16 @@ def test_config1_size_properties(dev):
     # full-size parity on a slab of rows against the oracle
     wq, ws = R.fp8_quantize(x[:256], 16, "E4M3")
     assert eq_bytes(q1[:256], wq) and torch.equal(s1[:256].cpu(), ws)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_default_division_scale_is_the_device_expression(dev, dtype):
+    """(absmax + 1e-10) / fp8max as torch evaluates it on the device (a multiplication by the fp32 reciprocal)."""
+    rq = _rq()
+    for seed in range(12):
+        x = make_x(16, 64, 100 + seed, dtype, scale=0.37 * (seed + 1))
+        for fp8 in ("E4M3", "E5M2"):
+            _, s = rq.fp8_division(x.to(dev), 16, fp8)
+            ws = R.absmax_scale(x, fp8)
+            assert s.dtype == dtype and torch.equal(s.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
+                                                    ws.view(torch.int16 if dtype != torch.float32 else torch.int32))
