@@ -195,6 +195,24 @@ int coat_fp8_adamw_step(void* params, const void* grads, int p_dtype, void* exp_
                         void* exp_avg_sq, float* scale_exp_avg_sq, float beta1, float beta2, float lr, float wd,
                         float eps, int step, int qgroup_size, int64_t numel, int64_t n_scale, void* stream);
 
+/* coat/activation/liger/cross_entropy.py:24-222 liger_cross_entropy_kernel as launched by cross_entropy_forward
+ * (:240-299): softmax cross-entropy over x [n_rows, n_cols] (row pitch x_stride elements, fp32 / bf16 / fp16).
+ * On return x holds the gradient of the reduced loss w.r.t. the logits, loss[row] (and z_loss[row] when z_loss is
+ * not NULL) the row's contribution, both in x's dtype; rows whose target equals ignore_index get zeros.
+ * target: int64 [n_rows].  reduction: 0 "none", 1 "mean", 2 "sum"; for "mean" the divisor is read from
+ * *n_non_ignore (one int64 in device memory: the number of targets != ignore_index), so the host never waits for it
+ * (the reference calls .item(), :262).  has_softcap != 0: logits pass through softcap * tanh(x / softcap) first. */
+int coat_cross_entropy_forward(void* x, int x_dtype, int64_t x_stride, const int64_t* target, void* loss, void* z_loss,
+                               const int64_t* n_non_ignore, int64_t n_rows, int64_t n_cols, int64_t ignore_index,
+                               float lse_square_scale, float label_smoothing, int reduction, float softcap,
+                               int has_softcap, void* stream);
+
+/* coat/activation/liger/cross_entropy.py:302-325 cross_entropy_backward (element_mul_kernel, liger/utils.py):
+ * x *= *grad_output in place; grad_output is one element of g_dtype in device memory.  The kernel itself returns
+ * without touching x when the factor is 1 (the reference compares on the host with torch.equal, a synchronisation). */
+int coat_cross_entropy_scale_grad(void* x, int x_dtype, int64_t x_stride, const void* grad_output, int g_dtype,
+                                  int64_t n_rows, int64_t n_cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
