@@ -236,6 +236,112 @@ class Bf16DecoderLayer:
         return x1 + F.linear(m, p["MLPResidual.down_proj.weight"])
 
 
+class Bf16OLMoBlock:
+    """The OLMo sequential block in plain bf16 torch (non-parametric LayerNorm, fused qkv and up/gate projections,
+    SwiGLU), the baseline of --workload olmo_block."""
+
+    def __init__(self, torch, blk):
+        self.p = {n: p.detach().clone().requires_grad_(True) for n, p in blk.named_parameters()}
+        self.nh, self.fused_dims = blk.config.n_heads, blk.fused_dims
+
+    def __call__(self, x):
+        import torch.nn.functional as F
+        from coat_amd.models.coat_llama import fused_rotary
+        p = self.p
+        B, S, D = x.shape
+        hd = D // self.nh
+        q, k, v = F.linear(F.layer_norm(x, (D,), None, None, 1e-5), p["BeforeAttention.att_proj.weight"]).split(self.fused_dims, dim=-1)
+        q = fused_rotary(q.contiguous(), self.nh, hd, 10000.0)
+        k = fused_rotary(k.contiguous(), self.nh, hd, 10000.0)
+        v = v.reshape(B, S, self.nh, hd).transpose(1, 2)
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, D)
+        x1 = x + F.linear(a, p["AfterAttention.attn_out.weight"])
+        up, gate = F.linear(F.layer_norm(x1, (D,), None, None, 1e-5), p["MLPResidual.ff_proj.weight"]).chunk(2, dim=-1)
+        return x1 + F.linear(F.silu(gate) * up, p["MLPResidual.ff_out.weight"])
+
+
+def make_olmo_workload(dev, torch):
+    """CoatOLMoSequentialBlock fwd+bwd at the OLMo-7B shape (d_model 4096, 32 heads, mlp_hidden_size 22016),
+    batch 4 x seq 2048, random init N(0, 0.02) (coat/models/coat_olmo.py:910-1076)."""
+    from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
+    from coat_amd.models.coat_olmo import CoatOLMoConfig, CoatOLMoSequentialBlock
+    from coat_amd.utils._fp8manager import FP8Manager
+
+    D, heads, hidden = 4096, 32, 22016
+    B, S = 4, 2048
+    torch.manual_seed(0)
+    cfg = CoatOLMoConfig(d_model=D, n_heads=heads, mlp_hidden_size=hidden)
+    blk = CoatOLMoSequentialBlock(0, cfg)
+    for p in blk.parameters():
+        torch.nn.init.normal_(p, std=0.02)
+    blk = blk.to(dev).to(torch.bfloat16).train()
+    bgn, end = Coat_quantize_bgn(blk.qargs), Coat_quantize_end(blk.qargs)
+    x = torch.randn(B, S, D, device=dev, dtype=torch.bfloat16)
+    gy = torch.randn(B, S, D, device=dev, dtype=torch.bfloat16) * 1e-2
+    ref = Bf16OLMoBlock(torch, blk)
+    state = {"first": True}
+
+    def step_fp8():
+        FP8Manager.is_first_microbatch = state["first"]
+        state["first"] = False
+        for p in blk.parameters():
+            p.grad = None
+        h, q, s = bgn(x.detach().requires_grad_(True))
+        h, q, s, _ = blk(h, q, s)
+        end(h, q, s).backward(gy)
+
+    def step_bf16():
+        for p in ref.p.values():
+            p.grad = None
+        ref(x.detach().requires_grad_(True)).backward(gy)
+
+    gemm_flops = 3 * 2 * B * S * (4 * D * D + D * hidden + D * hidden // 2)
+    return step_fp8, step_bf16, gemm_flops, {
+        "workload": f"CoatOLMoSequentialBlock fwd+bwd, OLMo-7B shape (d_model {D}, heads {heads}, mlp_hidden_size {hidden}), "
+                    f"batch {B} x seq {S}, FP8 linears/activations/LayerNorm, bf16 SDPA attention",
+        "tokens": B * S, "gemm_flops": gemm_flops}
+
+
+def make_layernorm_workload(dev, torch):
+    """Non-parametric LayerNorm on the FP8 block input [8192,4096] -> per-tensor FP8 (+ transpose), and its backward
+    (coat/activation/real_quantization/func_layernorm_noparam.py:193-297), as the OLMo block calls them."""
+    import coat_amd.activation.real_quantization as rq
+
+    M, N, QB = 8192, 4096, 16
+    gen = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(M, N, generator=gen, device=dev).bfloat16()
+    g = (torch.randn(M, N, generator=gen, device=dev) * 1e-2).bfloat16()
+    q, s = rq.fp8_quantize(x, QB, "E4M3")
+
+    def step():
+        qy, sy, qyt, (mean, rstd, nw) = rq.fp8_layernorm_noparam_forward(q, s, QB, 1e-5, transpose_output_2d=True)
+        rq.fp8_layernorm_noparam_backward(q, s, g, QB, mean, rstd, nw)
+
+    E = M * N
+    nbytes = int((E + E / 8) + 2 * E + (E + E / 8) + 2 * E + 2 * E)  # fwd: codes+scales in, q + q^T out; bwd: codes+scales, dy in, dx out
+    return step, nbytes, {"workload": f"LayerNorm (no parameters) fwd (FP8 in -> per-tensor FP8 + transpose) + bwd on [{M},{N}]",
+                          "M": M, "N": N, "kernel": "k_layernorm_fwd, k_division_transpose, k_layernorm_bwd"}
+
+
+def make_division_workload(dev, torch, stochastic):
+    """Per-tensor division bf16 [8192,4096] -> e5m2 with a given scale, deterministic or with the reference's stochastic
+    rounding (coat/activation/real_quantization/_division.py:153-207): 2 bytes read + 1 written per element."""
+    import coat_amd.activation.real_quantization as rq
+
+    M, N = 8192, 4096
+    gen = torch.Generator(device=dev).manual_seed(0)
+    xs = [torch.randn(M, N, generator=gen, device=dev).bfloat16() for _ in range(6)]
+    scale = torch.tensor(0.01, device=dev, dtype=torch.bfloat16)
+    it = {"i": 0}
+
+    def step():
+        it["i"] = (it["i"] + 1) % len(xs)
+        rq.fp8_division(xs[it["i"]], 16, "E5M2", scale, stochastic=stochastic)
+
+    return step, 3 * M * N, {"workload": f"fp8_division bf16 [{M},{N}] -> e5m2, stochastic={stochastic}", "M": M, "N": N,
+                            "kernel": "k_division"}
+
+
 def make_layer_workload(dev, torch, size):
     """BASELINE configs[4]: COAT Llama decoder layer fwd+bwd, batch 4 x seq 2048, random init N(0, 0.02)."""
     from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
@@ -334,6 +440,8 @@ def ramp_clocks(step, seconds, torch):
 def bench_layer(args, dev, torch):
     if args.workload == "linear":
         step_fp8, step_bf16, gemm_flops, cfg = make_linear_workload(dev, torch)
+    elif args.workload == "olmo_block":
+        step_fp8, step_bf16, gemm_flops, cfg = make_olmo_workload(dev, torch)
     else:
         step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1])
 
@@ -378,7 +486,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adamw", choices=["adamw", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
-                             "silu_mul", "rmsnorm", "cross_entropy", "layer_7b", "layer_13b"])
+                             "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr", "olmo_block", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ramp-seconds", type=float, default=1.5,
                     help="untimed continuous run of the step before the W warmup steps: an idle MI355X sits at ~100 MHz and "
@@ -404,7 +512,7 @@ def main():
     torch.cuda.set_device(dev)
 
     is_gemm = args.workload.startswith("gemm")
-    if args.workload.startswith("layer") or args.workload == "linear":
+    if args.workload.startswith("layer_") or args.workload in ("linear", "olmo_block"):
         return bench_layer(args, dev, torch)
     if args.workload in ("adamw", "adamw_plain"):
         step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch, expand=args.workload == "adamw")
@@ -412,6 +520,10 @@ def main():
         step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1])
     elif args.workload == "cross_entropy":
         step, nbytes, cfg = make_cross_entropy_workload(dev, torch)
+    elif args.workload == "layernorm":
+        step, nbytes, cfg = make_layernorm_workload(dev, torch)
+    elif args.workload in ("division", "division_sr"):
+        step, nbytes, cfg = make_division_workload(dev, torch, args.workload == "division_sr")
     elif args.workload == "silu_mul":
         step, nbytes, cfg = make_silu_mul_workload(dev, torch)
     elif args.workload == "rmsnorm":

@@ -127,8 +127,9 @@ __device__ __forceinline__ uint32_t philox4x32_10_word0(uint32_t c0, uint32_t k0
     uint32_t c1 = 0, c2 = 0, c3 = 0;
 #pragma unroll
     for (int r = 0; r < 10; r++) {
-        const uint32_t hi_b = __umulhi(0xCD9E8D57u, c2), lo_b = 0xCD9E8D57u * c2;
-        const uint32_t hi_a = __umulhi(0xD2511F53u, c0), lo_a = 0xD2511F53u * c0;
+        const uint64_t pb = (uint64_t)0xCD9E8D57u * c2, pa = (uint64_t)0xD2511F53u * c0;  // one 32x32->64 multiply each
+        const uint32_t hi_b = (uint32_t)(pb >> 32), lo_b = (uint32_t)pb;
+        const uint32_t hi_a = (uint32_t)(pa >> 32), lo_a = (uint32_t)pa;
         c0 = hi_b ^ c1 ^ k0;
         c2 = hi_a ^ c3 ^ k1;
         c1 = lo_b;

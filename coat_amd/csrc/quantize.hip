@@ -64,17 +64,23 @@ template <int KIND, int VEC> __device__ __forceinline__ void quantize_vec_slow(c
         out[i] = cvt4_fp8<KIND>(v[4 * i] / s, v[4 * i + 1] / s, v[4 * i + 2] / s, v[4 * i + 3] / s);
 }
 // Stochastic variant: the quotient of element (e0 + k) is perturbed with Philox noise drawn at that linear index.
-template <int KIND, int VEC>
-__device__ __forceinline__ void quantize_vec_sr(const float* v, float s, float r, bool fast, uint32_t e0, uint32_t k0,
-                                                uint32_t k1, uint32_t* out) {
+template <int KIND, int VEC, bool FAST>
+__device__ __forceinline__ void quantize_vec_sr_impl(const float* v, float s, float r, uint32_t e0, uint32_t k0,
+                                                     uint32_t k1, uint32_t* out) {
     float t[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; k++) {
-        const float qv = fast ? div_by_scale(v[k], s, r) : v[k] / s;
+        const float qv = FAST ? div_by_scale(v[k], s, r) : v[k] / s;
         t[k] = stochastic_perturb<KIND>(qv, uniform_from_word(philox4x32_10_word0(e0 + (uint32_t)k, k0, k1)));
     }
 #pragma unroll
     for (int i = 0; i < VEC / 4; i++) out[i] = cvt4_fp8<KIND>(t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3]);
+}
+template <int KIND, int VEC>
+__device__ __forceinline__ void quantize_vec_sr(const float* v, float s, float r, bool fast, uint32_t e0, uint32_t k0,
+                                                uint32_t k1, uint32_t* out) {
+    if (fast) quantize_vec_sr_impl<KIND, VEC, true>(v, s, r, e0, k0, k1, out);  // `fast` is uniform across the grid
+    else quantize_vec_sr_impl<KIND, VEC, false>(v, s, r, e0, k0, k1, out);
 }
 template <int VEC> __device__ __forceinline__ void store_codes(void* q, int64_t e, const uint32_t* c) {
     if (VEC == 8) *(uint2*)((uint8_t*)q + e) = make_uint2(c[0], c[1]);
