@@ -31,14 +31,14 @@ __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uin
 __device__ __forceinline__ float bf16lo(uint32_t w) { return u2f(w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
 
-// fp32 -> bf16 bits, round to nearest even, NaN quieted (same result as torch's and the hardware's).
-__device__ __forceinline__ uint32_t f2bf16(float f) {
-    uint32_t u = f2u(f);
-    uint32_t r = u + 0x7FFFu + ((u >> 16) & 1u);
-    r = (u & 0x7FFFFFFFu) > 0x7F800000u ? (u | 0x00400000u) : r;
-    return r >> 16;
+// fp32 -> bf16 bits, round to nearest even (same result as torch's): the gfx950 conversion instruction
+// v_cvt_pk_bf16_f32, one VALU operation for two values instead of ten of integer arithmetic.
+typedef float coat_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 coat_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((coat_f32x2){lo, hi}, coat_bf16x2));
 }
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) { return f2bf16(lo) | (f2bf16(hi) << 16); }
+__device__ __forceinline__ uint32_t f2bf16(float f) { return pack_bf16x2(f, 0.0f) & 0xFFFFu; }
 
 __device__ __forceinline__ float f16lo(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFF)); }
 __device__ __forceinline__ float f16hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
