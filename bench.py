@@ -220,6 +220,7 @@ class Bf16DecoderLayer:
 
     def __call__(self, x):
         import torch.nn.functional as F
+        from coat_amd.models._attention import sdpa
         from coat_amd.models.coat_llama import fused_rotary
         p, torch = self.p, self.torch
         B, S, H = x.shape
@@ -229,7 +230,7 @@ class Bf16DecoderLayer:
         q = fused_rotary(F.linear(h, p["BeforeAttention.q_proj.weight"]), self.nh, hd, 10000.0)
         k = fused_rotary(F.linear(h, p["BeforeAttention.k_proj.weight"]), self.nh, hd, 10000.0)
         v = F.linear(h, p["BeforeAttention.v_proj.weight"]).view(B, S, self.nh, hd).transpose(1, 2)
-        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, H)
+        a = sdpa(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, H)
         x1 = x + F.linear(a, p["AfterAttention.o_proj.weight"])
         h2 = F.rms_norm(x1, (H,), p["post_attention_layernorm.weight"], 1e-5)
         m = F.silu(F.linear(h2, p["MLPResidual.gate_proj.weight"])) * F.linear(h2, p["MLPResidual.up_proj.weight"])
@@ -246,6 +247,7 @@ class Bf16OLMoBlock:
 
     def __call__(self, x):
         import torch.nn.functional as F
+        from coat_amd.models._attention import sdpa
         from coat_amd.models.coat_llama import fused_rotary
         p = self.p
         B, S, D = x.shape
@@ -254,7 +256,7 @@ class Bf16OLMoBlock:
         q = fused_rotary(q.contiguous(), self.nh, hd, 10000.0)
         k = fused_rotary(k.contiguous(), self.nh, hd, 10000.0)
         v = v.reshape(B, S, self.nh, hd).transpose(1, 2)
-        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, D)
+        a = sdpa(q, k, v, is_causal=True).transpose(1, 2).reshape(B, S, D)
         x1 = x + F.linear(a, p["AfterAttention.attn_out.weight"])
         up, gate = F.linear(F.layer_norm(x1, (D,), None, None, 1e-5), p["MLPResidual.ff_proj.weight"]).chunk(2, dim=-1)
         return x1 + F.linear(F.silu(gate) * up, p["MLPResidual.ff_out.weight"])

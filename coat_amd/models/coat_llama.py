@@ -22,6 +22,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt, fp8_division,
                                             fp8_division_transpose, fp8_linear_backward, fp8_linear_forward,
                                             fp8_mul_backward, fp8_mul_forward, fp8_quantize_pertensor,
@@ -453,7 +454,7 @@ class LlamaSdpaAttentionWithoutLinear(nn.Module):
         mask = attention_mask
         if mask is not None:
             mask = mask[:, :, :, : k.shape[-2]]
-        out = F.scaled_dot_product_attention(q, k, v, attn_mask=mask,
+        out = sdpa(q, k, v, attn_mask=mask,
                                              dropout_p=self.attention_dropout if self.training else 0.0,
                                              is_causal=mask is None and q_len > 1)
         out = out.transpose(1, 2).contiguous().view(bsz, q_len, -1)

@@ -14,6 +14,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt,
                                             fp8_division_transpose, fp8_layernorm_noparam_backward,
                                             fp8_layernorm_noparam_forward, fp8_linear_backward, fp8_linear_forward,
@@ -281,7 +282,7 @@ class CoatOLMoSequentialBlock(nn.Module):
         if k.size(1) != q.size(1):
             rep = q.size(1) // k.size(1)
             k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
-        att = F.scaled_dot_product_attention(q, k, v, attn_mask=attention_bias,
+        att = sdpa(q, k, v, attn_mask=attention_bias,
                                              dropout_p=self.config.attention_dropout if self.training else 0.0,
                                              is_causal=attention_bias is None)
         return att.transpose(1, 2).contiguous().view(B, T, C)

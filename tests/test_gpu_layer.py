@@ -199,3 +199,22 @@ def test_make_state_dict_compatible():
     out = make_state_dict_compatible(sd)
     assert set(out) == {"model.layers.0.BeforeAttention.q_proj.weight", "model.layers.0.MLPResidual.down_proj.weight",
                         "model.norm.weight"}
+
+
+def test_attention_backend_choice_matches_fp32_math(dev):
+    """The backend order of coat_amd/models/_attention.py changes speed, not results: output and gradients agree
+    with fp32 softmax(QK^T / sqrt(d)) V to bf16 accuracy."""
+    from coat_amd.models._attention import sdpa
+    g = torch.Generator().manual_seed(4)
+    B, H, S, D = 2, 4, 256, 128
+    q, k, v = (torch.randn(B, S, H, D, generator=g).to(dev).bfloat16().transpose(1, 2).requires_grad_(True) for _ in range(3))
+    go = torch.randn(B, H, S, D, generator=g).to(dev).bfloat16()
+    out = sdpa(q, k, v, is_causal=True)
+    gq, gk, gv = torch.autograd.grad(out, (q, k, v), go)
+    qf, kf, vf = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+    att = (qf @ kf.transpose(-1, -2)) / D ** 0.5
+    att = att.masked_fill(torch.triu(torch.ones(S, S, dtype=torch.bool, device=dev), 1), float("-inf")).softmax(-1)
+    ref = att @ vf
+    rq, rk, rv = torch.autograd.grad(ref, (qf, kf, vf), go.float())
+    for a, b in ((out, ref), (gq, rq), (gk, rk), (gv, rv)):
+        assert ((a.float() - b).norm() / b.norm()).item() < 1e-2
