@@ -173,6 +173,10 @@ struct SiluMulArgs {
     float *s_max, *s_max2;                                  // max of the fp32 group scales of y / y2
     int64_t nchunk;
     int qb, s_dtype;
+    // Row pitches, for gate / up taken as column slices of a wider tensor and y / y2 written into one (strided != 0):
+    // chunks of 16 elements per logical row, per row of gate / up, per row of y / y2; scales per row of s_gate / s_up.
+    int strided;
+    int64_t cpr, in_cpr, in_spr, y_cpr;
 };
 
 template <int KIND> __device__ __forceinline__ void dequant_words(const uint32_t* w, float scale, float* v) {
@@ -203,9 +207,16 @@ __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
         const bool ok = chunk < A.nchunk;
         const int64_t c = ok ? chunk : 0;
         const int64_t gidx = (c * 16) / A.qb;
+        int64_t cin = c, gin = gidx, cy = c;
+        if (A.strided) {  // uniform
+            const int64_t row = c / A.cpr, col = c - row * A.cpr;
+            cin = row * A.in_cpr + col;
+            gin = row * A.in_spr + (col * 16) / A.qb;
+            cy = row * A.y_cpr + col;
+        }
         float a[16], b[16];
-        load_fp8x16<KIND_IN>(A.gate, c, load_scale_rt(A.s_gate, gidx, A.s_dtype), a);
-        load_fp8x16<KIND_IN>(A.up, c, load_scale_rt(A.s_up, gidx, A.s_dtype), b);
+        load_fp8x16<KIND_IN>(A.gate, cin, load_scale_rt(A.s_gate, gin, A.s_dtype), a);
+        load_fp8x16<KIND_IN>(A.up, cin, load_scale_rt(A.s_up, gin, A.s_dtype), b);
         if (!BWD) {
             float sv[16];
 #pragma unroll
@@ -241,8 +252,8 @@ __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
                 v[i] = (sig + (a[i] * sig) * (1 - sig)) * g1;
             }
             if (ok) {
-                store_bf16x16(A.y, c, v);
-                store_bf16x16(A.y2, c, v2);
+                store_bf16x16(A.y, cy, v);
+                store_bf16x16(A.y2, cy, v2);
             }
             const float s1 = group_scale<KIND_OUT>(cluster_max_rt(amax16(v), lpg));
             const float s2 = group_scale<KIND_OUT>(cluster_max_rt(amax16(v2), lpg));
@@ -363,8 +374,13 @@ extern "C" int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s
 }
 
 static int silu_mul_launch(SiluMulArgs& A, bool bwd, int fp8_in, int fp8_out, int64_t M, int64_t N, int QB, int s_dtype,
-                           hipStream_t st) {
+                           int64_t in_pitch, int64_t s_pitch, int64_t y_pitch, hipStream_t st) {
     if (M < 0 || N < 0) return COAT_EINVAL;
+    // pitches in elements (0 = contiguous rows); a slice must keep rows 16-byte aligned and whole groups
+    if (in_pitch == 0) in_pitch = N;
+    if (y_pitch == 0) y_pitch = N;
+    if (QB > 0 && s_pitch == 0) s_pitch = N / QB;
+    if (in_pitch < N || y_pitch < N || in_pitch % 16 != 0 || y_pitch % 16 != 0 || (!bwd && y_pitch != N)) return COAT_ESHAPE;
     if (QB < 16 || QB > 1024 || (QB & (QB - 1)) || N % QB != 0) return COAT_ESHAPE;
     if (s_dtype != COAT_BF16 && s_dtype != COAT_F32 && s_dtype != COAT_F16) return COAT_EDTYPE;
     if (fp8_in != COAT_E4M3 && fp8_in != COAT_E5M2) return COAT_EINVAL;
@@ -373,9 +389,15 @@ static int silu_mul_launch(SiluMulArgs& A, bool bwd, int fp8_in, int fp8_out, in
     const void* ptrs[] = {A.gate, A.up, A.silu, A.g, A.q_silu, A.y, A.y2};
     for (const void* p : ptrs)
         if (!coat_aligned16(p)) return COAT_EALIGN;
+    if (s_pitch < N / QB) return COAT_ESHAPE;
     A.nchunk = M * N / 16;
     A.qb = QB;
     A.s_dtype = s_dtype;
+    A.strided = in_pitch != N || y_pitch != N || s_pitch != N / QB;
+    A.cpr = N / 16;
+    A.in_cpr = in_pitch / 16;
+    A.in_spr = s_pitch;
+    A.y_cpr = y_pitch / 16;
     int64_t blocks = (A.nchunk + 255) / 256;
     if (blocks > 2048) blocks = 2048;
 #define SM_LAUNCH(B, KI, KO) hipLaunchKernelGGL((k_silu_mul<B, KI, KO>), dim3((unsigned)blocks), dim3(256), 0, st, A)
@@ -392,18 +414,19 @@ static int silu_mul_launch(SiluMulArgs& A, bool bwd, int fp8_in, int fp8_out, in
 
 extern "C" int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
                                          int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M,
-                                         int64_t N, int QB, void* stream) {
+                                         int64_t N, int QB, int64_t in_pitch, int64_t s_pitch, void* stream) {
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !q_silu || !s_silu || !y || !s_max)) return COAT_EINVAL;
     SiluMulArgs A = {gate, s_gate, up, s_up, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr, 0, 0, 0};
-    return silu_mul_launch(A, false, fp8, fp8, M, N, QB, s_dtype, (hipStream_t)stream);
+    return silu_mul_launch(A, false, fp8, fp8, M, N, QB, s_dtype, in_pitch, s_pitch, 0, (hipStream_t)stream);
 }
 
 extern "C" int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, const void* up, const void* s_up,
                                           const void* silu, const void* s_silu, int fp8_in, int s_dtype, const void* g,
                                           void* y_gate, float* s_max_gate, void* y_up, float* s_max_up, int fp8_out,
-                                          int64_t M, int64_t N, int QB, void* stream) {
+                                          int64_t M, int64_t N, int QB, int64_t in_pitch, int64_t s_pitch,
+                                          int64_t y_pitch, void* stream) {
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !silu || !s_silu || !g || !y_gate || !s_max_gate || !y_up || !s_max_up))
         return COAT_EINVAL;
     SiluMulArgs A = {gate, s_gate, up, s_up, silu, s_silu, g, nullptr, nullptr, y_gate, y_up, s_max_gate, s_max_up, 0, 0, 0};
-    return silu_mul_launch(A, true, fp8_in, fp8_out, M, N, QB, s_dtype, (hipStream_t)stream);
+    return silu_mul_launch(A, true, fp8_in, fp8_out, M, N, QB, s_dtype, in_pitch, s_pitch, y_pitch, (hipStream_t)stream);
 }

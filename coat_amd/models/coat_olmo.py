@@ -18,9 +18,8 @@ from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt,
                                             fp8_division_transpose, fp8_layernorm_noparam_backward,
                                             fp8_layernorm_noparam_forward, fp8_linear_backward, fp8_linear_forward,
-                                            fp8_mul_backward, fp8_mul_forward, fp8_quantize_pertensor,
-                                            fp8_quantize_pertensor_transpose, fp8_silu_backward, fp8_silu_forward,
-                                            fp8_transpose)
+                                            fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
+                                            fp8_silu_mul_backward_joined, fp8_silu_mul_forward, fp8_transpose)
 from ..utils._fp8_quantization_config import QuantizationConfig
 from .coat_llama import (E4M3, _as_e4m3_input, _as_e5m2_grad, _backward_weight_t, _forward_weight, _ResidualBase,
                          apply_rotary_pos_emb, fused_rotary, rotary_cos_sin)
@@ -183,10 +182,12 @@ class _CoatOLMoMLPResidual(torch.autograd.Function):
         # the fused projection writes per-group FP8 straight from the GEMM epilogue; halves: up first, gate second (:520)
         fc1_x, fc1_s = fp8_linear_forward(ln_x, ln_s, _forward_weight(w1_origin, w1, w1_s, qargs, fwobits), w1_s, True,
                                           group_size)
-        up_x, gate_x = (t.contiguous() for t in fc1_x.chunk(2, dim=-1))
-        up_s, gate_s = (t.contiguous() for t in fc1_s.chunk(2, dim=-1))
-        silu_x, silu_s = fp8_silu_forward(gate_x, gate_s, group_size)
-        mul_x, mul_s, mul_x_t = fp8_mul_forward(silu_x, silu_s, up_x, up_s, group_size, transpose_output_2d=True)
+        # the halves stay column slices of fc1_x / fc1_s (the reference copies them, :522-523); one kernel for
+        # fp8_silu_forward + fp8_mul_forward (:525-528), same tensors
+        up_x, gate_x = fc1_x.chunk(2, dim=-1)
+        up_s, gate_s = fc1_s.chunk(2, dim=-1)
+        silu_x, silu_s, mul_x, mul_s, mul_x_t = fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, group_size,
+                                                                    transpose_output_2d=True)
         fc2_x = fp8_linear_forward(mul_x, mul_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits), w2_s, False,
                                    group_size)
         fp_x, (out_x, out_s) = fp8_add_Ifp_Ifp_Ofp_Og16(re_x, fc2_x, mul_x.dtype, group_size)
@@ -213,14 +214,10 @@ class _CoatOLMoMLPResidual(torch.autograd.Function):
         w2_t = _backward_weight_t(w2_saved, w2_s, qargs, fwobits)
         fc2_g, weight2_grad = fp8_linear_backward(mul_x_t, mul_s, out_g, out_gs_max, out_g_t, w2_t, w2_s, group_size)
         del out_g, out_g_t, w2_t
-        # element-wise product and SiLU with bf16 outputs and per-group scales; the two halves are joined and quantized
-        # per tensor with the larger of their maxima (:594-606)
-        mul_g1, (mul_g2, mul_gs2) = fp8_mul_backward(silu_x, silu_s, up_x, up_s, fc2_g, group_size, fwobits["babit"])
-        silu_g, silu_gs = fp8_silu_backward(gate_x, gate_s, mul_g1, group_size, fwobits["babit"])
-        gateup_g = torch.cat([mul_g2, silu_g], dim=-1)
-        gateup_gs = torch.max(torch.cat([mul_gs2, silu_gs]))
-        gateup_g, gateup_gs, gateup_g_t = fp8_division_transpose(gateup_g, group_size, fwobits["babit"], gateup_gs,
-                                                                 stochastic=False)
+        # one kernel for the reference's fp8_mul_backward + fp8_silu_backward, writing the two bf16 gradients side by
+        # side (no torch.cat); the joined tensor is quantized per tensor with the larger of the two maxima (:594-606)
+        gateup_g, gateup_gs, gateup_g_t = fp8_silu_mul_backward_joined(gate_x, gate_s, up_x, up_s, silu_x, silu_s, fc2_g,
+                                                                       group_size, fwobits["babit"])
         w1_t = _backward_weight_t(w1_saved, w1_s, qargs, fwobits)
         fc1_g, weight1_grad = fp8_linear_backward(ln_x_t, ln_s, gateup_g, gateup_gs, gateup_g_t, w1_t, w1_s, group_size)
         in_g = fp8_layernorm_noparam_backward(in_x, in_s, fc1_g, group_size, mean, rstd, num_warps)

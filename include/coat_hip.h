@@ -121,13 +121,16 @@ int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s_y, float* 
  * dequantized SiLU and up, *s_max = max of the product's fp32 group scales (fp8 = format of gate / up / silu). */
 int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
                               int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M, int64_t N,
-                              int QB, void* stream);
+                              int QB, int64_t in_pitch, int64_t s_pitch, void* stream);
 /* backward: y_up = bf16(g * silu), y_gate = bf16(silu'(gate) * bf16(g * up)); *s_max_* = max of their fp32 group
- * scales for the format fp8_out (the per-tensor division that follows is coat_fp8_division). */
+ * scales for the format fp8_out (the per-tensor division that follows is coat_fp8_division).
+ * Row pitches in elements, 0 = contiguous: in_pitch / s_pitch for gate, up and their scales when they are the two column
+ * halves of a fused projection's output (coat/models/coat_olmo.py:520-523 chunks and copies them), y_pitch (backward
+ * only) for y_gate / y_up written side by side into one [M, 2N] tensor (coat_olmo.py:599 concatenates them). */
 int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, const void* up, const void* s_up, const void* silu,
                                const void* s_silu, int fp8_in, int s_dtype, const void* g, void* y_gate,
                                float* s_max_gate, void* y_up, float* s_max_up, int fp8_out, int64_t M, int64_t N,
-                               int QB, void* stream);
+                               int QB, int64_t in_pitch, int64_t s_pitch, int64_t y_pitch, void* stream);
 
 /* rq/func_rmsnorm.py:223 fp8_rmsnorm_forward (kernel :54-111): y = bf16(x * rstd * w); s_row [M] bf16 row scales
  * (max|y| + 1e-10) / fp8max; rstd [M] fp32; s_max as above.  N <= 16384, N % 16 == 0. */

@@ -208,6 +208,43 @@ def test_fused_silu_mul_equals_the_two_kernel_chains(dev, fp8, QBv):
     assert o[0].shape == (2, M // 2, N) and o[2].shape == (2, M // 2, N) and torch.equal(b(o[2]).reshape(M, N), b(mul_x))
 
 
+@pytest.mark.parametrize("QBv", [16, 32])
+def test_fused_silu_mul_on_column_slices_and_joined_backward(dev, QBv):
+    """gate / up taken as the two column halves of one [M, 2N] projection output (no copies), and the backward that
+    writes both gradients side by side: bit for bit the chain of the separate kernels on dense copies, torch.cat,
+    max of the group scales and fp8_division_transpose (coat/models/coat_olmo.py:520-528, :594-606)."""
+    rq = _rq()
+    B, S, N = 2, 96, 512
+    M = B * S
+    both, g = rand(40, shape=(M, 2 * N)), rand(41, 0.01, shape=(M, N))
+    q, s = rq.fp8_quantize(both.to(dev), QBv, "E4M3")
+    q3, s3 = q.reshape(B, S, 2 * N), s.reshape(B, S, 2 * N // QBv)
+    up_v, gate_v = q3.chunk(2, dim=-1)
+    ups_v, gates_v = s3.chunk(2, dim=-1)
+    assert not gate_v.is_contiguous()
+    up_d, gate_d, ups_d, gates_d = (t.contiguous() for t in (up_v, gate_v, ups_v, gates_v))
+    # forward
+    silu_x, silu_s = rq.fp8_silu_forward(gate_d, gates_d, QBv)
+    mul_x, mul_s, mul_x_t = rq.fp8_mul_forward(silu_x, silu_s, up_d, ups_d, QBv, transpose_output_2d=True)
+    f = rq.fp8_silu_mul_forward(gate_v, gates_v, up_v, ups_v, QBv, transpose_output_2d=True)
+    assert f[0].shape == (B, S, N) and torch.equal(b(f[0]), b(silu_x)) and torch.equal(f[1], silu_s)
+    assert f[3].item() == mul_s.item() and torch.equal(b(f[2]), b(mul_x)) and torch.equal(b(f[4]), b(mul_x_t))
+    # backward, joined
+    gd = g.to(dev).reshape(B, S, N)
+    g1, (ug, ugs) = rq.fp8_mul_backward(silu_x, silu_s, up_d, ups_d, gd, QBv, "E5M2")
+    gg, ggs = rq.fp8_silu_backward(gate_d, gates_d, g1, QBv, "E5M2")
+    cat = torch.cat([ug, gg], dim=-1)
+    smax = torch.max(torch.cat([ugs, ggs]))
+    wq, ws, wqt = rq.fp8_division_transpose(cat, QBv, "E5M2", smax)
+    jq, js, jqt = rq.fp8_silu_mul_backward_joined(gate_v, gates_v, up_v, ups_v, silu_x, silu_s, gd, QBv, "E5M2")
+    assert jq.shape == (B, S, 2 * N) and js.item() == ws.item()
+    assert torch.equal(b(jq), b(wq)) and torch.equal(b(jqt), b(wqt))
+    # the non-joined backward also takes the slices
+    (gq, gs_, gqt), (uq, us_, uqt) = rq.fp8_silu_mul_backward(gate_v, gates_v, up_v, ups_v, silu_x, silu_s, gd, QBv, "E5M2")
+    (dq, ds_, dqt), (eq, es_, eqt) = rq.fp8_silu_mul_backward(gate_d, gates_d, up_d, ups_d, silu_x, silu_s, gd, QBv, "E5M2")
+    assert gs_.item() == ds_.item() and torch.equal(b(gq), b(dq)) and torch.equal(b(uqt), b(eqt))
+
+
 def test_larger_groups_and_float32_scales(dev):
     rq = _rq()
     x1, x2 = rand(13, shape=(128, 512)), rand(14, shape=(128, 512))
