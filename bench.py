@@ -87,11 +87,13 @@ def make_quantize_workload(dev, torch, transpose):
                           "kernel": "k_quantize_transpose" if transpose else "k_quantize_pg"}
 
 
-def make_gemm_workload(dev, torch, which):
-    """BASELINE configs[2]: X [8192,4096] x W [11008,4096]; which = fwd | dgrad | wgrad (the three GEMMs of FP8Linear)."""
+def make_gemm_workload(dev, torch, which, grad_format="e5m2"):
+    """BASELINE configs[2]: X [8192,4096] x W [11008,4096]; which = fwd | dgrad | wgrad (the three GEMMs of FP8Linear).
+    The gradient operand is e5m2 as the reference's default bobit; grad_format="e4m3" times the all-e4m3 variant."""
     from coat_amd.activation.real_quantization.linear import fp8matmul
 
-    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+    E4 = torch.float8_e4m3fn
+    E5 = torch.float8_e5m2 if grad_format == "e5m2" else E4
     T, K, N = 8192, 4096, 11008
     gen = torch.Generator(device="cpu").manual_seed(0)
 
@@ -110,7 +112,8 @@ def make_gemm_workload(dev, torch, which):
         fp8matmul(a, b.t(), False, one, one, 16)
 
     flops = 2 * M_ * N_ * K_
-    return step, flops, {"workload": f"fp8matmul {which}: [{M_},{K_}] x [{N_},{K_}]^T -> bf16, per-tensor scales",
+    fmt = "e4m3 x e4m3" if which == "fwd" or grad_format == "e4m3" else "e5m2 x e4m3"
+    return step, flops, {"workload": f"fp8matmul {which}: [{M_},{K_}] x [{N_},{K_}]^T -> bf16, {fmt}, per-tensor scales",
                          "M": M_, "N": N_, "K": K_, "kernel": "k_fp8_gemm"}
 
 
@@ -428,6 +431,26 @@ MEASURED_TRAFFIC = {
 }
 
 
+def cpu_baseline_quantize(torch, transpose, nbytes):
+    """The torch-CPU oracle on the whole [4096,4096] input (same seeded data), all host threads, median of 5 runs."""
+    from oracle import activation_ref as R
+
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn(4096, 4096, generator=gen)
+    x[torch.rand(4096, 4096, generator=gen) < 0.001] *= 100
+    x = x.bfloat16()
+    fn = R.fp8_quantize_transpose if transpose else R.fp8_quantize
+    fn(x, 16, "E4M3")
+    ts = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        fn(x, 16, "E4M3")
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return {"value": round(nbytes / ts[2] / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"the whole bf16 [4096,4096] input, oracle/activation_ref.py ({fn.__name__}), median of 5 runs"}
+
+
 def ramp_clocks(step, seconds, torch):
     """Keep the GPU continuously busy with `step` for `seconds` (untimed) so that the timed region runs at the sustained clock."""
     if seconds <= 0:
@@ -490,6 +513,8 @@ def main():
     ap.add_argument("--workload", default="adamw", choices=["adamw", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
                              "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr", "olmo_block", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--grad-format", default="e5m2", choices=["e5m2", "e4m3"],
+                    help="FP8 format of the gradient operand of gemm_dgrad / gemm_wgrad (the reference's default is e5m2)")
     ap.add_argument("--ramp-seconds", type=float, default=1.5,
                     help="untimed continuous run of the step before the W warmup steps: an idle MI355X sits at ~100 MHz and "
                          "takes several hundred ms of load to reach its sustained shader clock, so a few ms of warmup would "
@@ -519,7 +544,7 @@ def main():
     if args.workload in ("adamw", "adamw_plain"):
         step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch, expand=args.workload == "adamw")
     elif is_gemm:
-        step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1])
+        step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1], args.grad_format)
     elif args.workload == "cross_entropy":
         step, nbytes, cfg = make_cross_entropy_workload(dev, torch)
     elif args.workload == "layernorm":
@@ -572,10 +597,13 @@ def main():
         "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
                      ("algorithmic_flops_per_launch" if is_gemm else "algorithmic_bytes_per_launch"): nbytes, "kernel_ms_avg": round(avg_ms, 5),
-                     "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5)},
+                     "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
+                     "kernel_ms_p20": round(kern_ms[len(kern_ms) // 5], 5), "kernel_ms_p80": round(kern_ms[(4 * len(kern_ms)) // 5], 5)},
     }
     if args.workload == "adamw" and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_adamw(torch)
+    elif args.workload in ("quantize", "quantize_transpose") and not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_quantize(torch, args.workload == "quantize_transpose", nbytes)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))
