@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload adamw|quantize|quantize_transpose]
 
-Default workload = BASELINE.json configs[1]: one CoatAdamW step (Dynamic Range Expansion on) on an fp32 master
+Default workload = the headline configuration: one CoatAdamW step (Dynamic Range Expansion on) on an fp32 master
 weight [11008, 4096], grads N(0, 1e-3), lr 3e-4, betas (0.9, 0.95), wd 0.1, eps 1e-8, starting at step 10 from a
 moment state produced by nine untimed steps.  A "step" is one pass of the fused kernel over the whole tensor.
 Prints ONE JSON line.  `value` is algorithmic GB/s: every distinct input read once + every output written once
@@ -88,7 +88,7 @@ def make_quantize_workload(dev, torch, transpose):
 
 
 def make_gemm_workload(dev, torch, which, grad_format="e5m2"):
-    """BASELINE configs[2]: X [8192,4096] x W [11008,4096]; which = fwd | dgrad | wgrad (the three GEMMs of FP8Linear).
+    """The Llama-2-7B MLP up-projection at 8192 tokens, X [8192,4096] x W [11008,4096]; which = fwd | dgrad | wgrad (the three GEMMs of FP8Linear).
     The gradient operand is e5m2 as the reference's default bobit; grad_format="e4m3" times the all-e4m3 variant."""
     from coat_amd.activation.real_quantization.linear import fp8matmul
 
@@ -118,7 +118,7 @@ def make_gemm_workload(dev, torch, which, grad_format="e5m2"):
 
 
 def make_linear_workload(dev, torch):
-    """BASELINE configs[2] end to end: FP8Linear forward + backward at the Llama-2-7B MLP shape: per-tensor quantization
+    """The same linear end to end: FP8Linear forward + backward at the Llama-2-7B MLP shape: per-tensor quantization
     (with transposes) of X, W and the output gradient, then the three GEMMs.  Returns (fp8 step, bf16 step, flops)."""
     from coat_amd.activation.real_quantization.fp8linear import FP8Linear
 
@@ -144,7 +144,7 @@ def make_linear_workload(dev, torch):
 
 
 def make_silu_mul_workload(dev, torch):
-    """BASELINE configs[3]: SiLU(gate) * up on bf16 [8192,11008] inputs -> FP8 with 1x16 scales (and the saved FP8
+    """The Llama-2-7B MLP activation: SiLU(gate) * up on bf16 [8192,11008] inputs -> FP8 with 1x16 scales (and the saved FP8
     activations), then the backward chain with a bf16 gradient, as CoatLlamaMLPResidual strings the kernels together
     (coat/models/coat_llama.py:664-766)."""
     import coat_amd.activation.real_quantization as rq
@@ -170,7 +170,7 @@ def make_silu_mul_workload(dev, torch):
 
 
 def make_rmsnorm_workload(dev, torch):
-    """BASELINE configs[3], second half: RMSNorm on the FP8 block input [8192,4096] -> FP8 (+ transpose), and its backward."""
+    """RMSNorm on the FP8 block input [8192,4096] -> FP8 (+ transpose), and its backward."""
     import coat_amd.activation.real_quantization as rq
 
     M, N, QB = 8192, 4096, 16
@@ -348,7 +348,7 @@ def make_division_workload(dev, torch, stochastic):
 
 
 def make_layer_workload(dev, torch, size):
-    """BASELINE configs[4]: COAT Llama decoder layer fwd+bwd, batch 4 x seq 2048, random init N(0, 0.02)."""
+    """COAT Llama decoder layer fwd+bwd, batch 4 x seq 2048, random init N(0, 0.02)."""
     from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
     from coat_amd.models.coat_llama import CoatLlamaConfig, CoatLlamaDecoderLayer
     from coat_amd.utils._fp8manager import FP8Manager
@@ -524,7 +524,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported "
-              "(every kernel on the path is independent per row / per 128-element group, see DESIGN.md)", file=sys.stderr)
+              "(every kernel on the path is independent per row / per 128-element group)", file=sys.stderr)
         sys.exit(2)
 
     import torch

@@ -157,7 +157,7 @@ def test_fp8_dequantize(dev, fp8, QB):
 
 
 def test_config1_size_properties(dev):
-    """BASELINE config 1 at full size: invariants that need no CPU pass over 16M elements per check."""
+    """The bf16 [4096, 4096] quantize configuration at full size: invariants that need no CPU pass over 16M elements per check."""
     rq = _rq()
     g = torch.Generator(device="cpu").manual_seed(0)
     x = torch.randn(4096, 4096, generator=g)
