@@ -24,6 +24,8 @@ sys.path.insert(0, os.path.join(HERE, "..", ".."))
 
 from oracle import activation_ref as R  # noqa: E402
 from oracle import adamw_ref as A  # noqa: E402
+from oracle import cross_entropy_ref as C  # noqa: E402
+from oracle import stochastic_ref as S  # noqa: E402
 
 # value -> code, by hand from the OCP FP8 specification.  e4m3fn: bias 7, no inf, NaN = S.1111.111, max 448 = 0x7E,
 # min subnormal 2^-9 = 0x01.  e5m2: bias 15, inf = S.11111.00, max 57344 = 0x7B, min subnormal 2^-16 = 0x01.
@@ -95,10 +97,47 @@ def make_adamw(expand):
     np.savez_compressed(os.path.join(HERE, "adamw_expand_1064.npz" if expand else "adamw_plain_1064.npz"), **out)
 
 
+def make_stochastic():
+    """Stochastic-rounding division of a [32, 64] tensor by 2^-3: codes for both formats (seed 0, as the reference)."""
+    g = torch.Generator().manual_seed(4242)
+    x = (torch.randn(32, 64, generator=g) * torch.logspace(-4, 1.5, 32).unsqueeze(1)).bfloat16()
+    x[0, :8] = 0.0
+    scale = torch.tensor(0.125, dtype=torch.bfloat16)
+    out = {"x_bf16": bits16(x), "scale_bf16": bits16(scale.reshape(1))}
+    for name, ft in (("e4m3", "E4M3"), ("e5m2", "E5M2")):
+        q, _, qt = S.fp8_division_transpose_stochastic(x, 16, ft, scale)
+        out[f"{name}_q"] = u8(q)
+        out[f"{name}_qt"] = u8(qt)
+    np.savez_compressed(os.path.join(HERE, "division_stochastic_32x64.npz"), **out)
+
+
+CE_CASES = {  # name: (ignore_index, lse_square_scale, label_smoothing, reduction, softcap)
+    "plain_mean": (-100, 0.0, 0.0, "mean", None),
+    "smooth_z_sum": (-100, 1e-3, 0.1, "sum", None),
+    "softcap_mean": (-100, 0.0, 0.0, "mean", 4.0),
+}
+
+
+def make_cross_entropy():
+    g = torch.Generator().manual_seed(99)
+    x = torch.randn(16, 97, generator=g) * 3
+    t = torch.randint(0, 97, (16,), generator=g)
+    t[[2, 9]] = -100
+    out = {"x": x.numpy().copy(), "target": t.numpy().copy()}
+    for name, (ii, lss, ls, red, cap) in CE_CASES.items():
+        loss, z, grad = C.cross_entropy_forward(x, t, ii, lss, ls, red, cap)
+        out[f"{name}_loss"] = np.float64(loss.item())
+        out[f"{name}_z"] = np.float64(z.item())
+        out[f"{name}_grad"] = grad.numpy().copy()
+    np.savez_compressed(os.path.join(HERE, "cross_entropy_16x97.npz"), **out)
+
+
 if __name__ == "__main__":
     with open(os.path.join(HERE, "fp8_known_answers.json"), "w") as f:
         json.dump(KNOWN, f, indent=1)
     make_quantize()
     make_adamw(True)
     make_adamw(False)
+    make_stochastic()
+    make_cross_entropy()
     print("golden fixtures written to", HERE)

@@ -19,6 +19,11 @@ KEYS_EXP = ["exp_avg", "scale_exp_avg", "expand_exp_avg", "sqrt_minmax_exp_avg",
             "exp_avg_sq", "scale_exp_avg_sq", "expand_exp_avg_sq", "sqrt_minmax_exp_avg_sq"]
 KEYS_PLAIN = ["exp_avg", "scale_exp_avg", "exp_avg_sq", "scale_exp_avg_sq"]
 FT = {"e4m3": ("E4M3", torch.float8_e4m3fn), "e5m2": ("E5M2", torch.float8_e5m2)}
+CE_CASES = {  # name: (ignore_index, lse_square_scale, label_smoothing, reduction, softcap), as tests/golden/make_golden.py
+    "plain_mean": (-100, 0.0, 0.0, "mean", None),
+    "smooth_z_sum": (-100, 1e-3, 0.1, "sum", None),
+    "softcap_mean": (-100, 0.0, 0.0, "mean", 4.0),
+}
 
 
 def known():
@@ -92,7 +97,57 @@ def test_oracle_reproduces_adamw_fixture(expand):
             assert np.array_equal(got, z[f"{k}{step}"], equal_nan=True), (k, step)
 
 
+def test_oracle_reproduces_stochastic_fixture():
+    from oracle import stochastic_ref as S
+    z = np.load(os.path.join(G, "division_stochastic_32x64.npz"))
+    x, scale = bf16_from_bits(z["x_bf16"]), bf16_from_bits(z["scale_bf16"]).reshape(())
+    for name, (ft, dt) in FT.items():
+        q, _, qt = S.fp8_division_transpose_stochastic(x, 16, ft, scale)
+        assert np.array_equal(q.view(torch.uint8).numpy(), z[f"{name}_q"])
+        assert np.array_equal(qt.view(torch.uint8).numpy(), z[f"{name}_qt"])
+
+
+def test_oracle_reproduces_cross_entropy_fixture():
+    from oracle import cross_entropy_ref as C
+    z = np.load(os.path.join(G, "cross_entropy_16x97.npz"))
+    x, t = torch.from_numpy(z["x"].copy()), torch.from_numpy(z["target"].copy())
+    for name, (ii, lss, ls, red, cap) in CE_CASES.items():
+        loss, zl, grad = C.cross_entropy_forward(x, t, ii, lss, ls, red, cap)
+        assert abs(loss.item() - float(z[f"{name}_loss"])) <= 1e-12 * abs(float(z[f"{name}_loss"]))
+        assert abs(zl.item() - float(z[f"{name}_z"])) <= 1e-12 * max(abs(float(z[f"{name}_z"])), 1e-30)
+        assert np.allclose(grad.numpy(), z[f"{name}_grad"], rtol=1e-12, atol=1e-15)
+
+
 # ------------------------------------------------------------------------------------------------ GPU: HIP path vs fixtures
+@pytest.mark.gpu
+def test_hip_stochastic_division_matches_fixture(dev):
+    import coat_amd.activation.real_quantization as rq
+    z = np.load(os.path.join(G, "division_stochastic_32x64.npz"))
+    x, scale = bf16_from_bits(z["x_bf16"]).to(dev), bf16_from_bits(z["scale_bf16"]).reshape(()).to(dev)
+    for name, (ft, dt) in FT.items():
+        q, _, qt = rq.fp8_division_transpose(x, 16, ft, scale, stochastic=True)
+        q1, _ = rq.fp8_division(x, 16, ft, scale, stochastic=True)
+        for got, key in ((q, "q"), (q1, "q"), (qt, "qt")):
+            assert np.array_equal(got.cpu().view(torch.uint8).numpy(), z[f"{name}_{key}"]), (name, key)
+
+
+@pytest.mark.gpu
+def test_hip_cross_entropy_matches_fixture(dev):
+    """fp32 logits: loss rtol 2e-6, gradient 2e-6 relative + 3e-7 / divisor (as tests/test_gpu_cross_entropy.py)."""
+    from coat_amd.activation.liger.cross_entropy import cross_entropy_forward
+    z = np.load(os.path.join(G, "cross_entropy_16x97.npz"))
+    t = torch.from_numpy(z["target"].copy())
+    for name, (ii, lss, ls, red, cap) in CE_CASES.items():
+        x = torch.from_numpy(z["x"].copy()).to(dev)
+        loss, zl, grad = cross_entropy_forward(x, t.to(dev), ii, lss, ls, red, cap, True)
+        n = float((t != ii).sum()) if red == "mean" else 1.0
+        want = torch.from_numpy(z[f"{name}_grad"])
+        assert abs(loss.item() - float(z[f"{name}_loss"])) <= 2e-6 * abs(float(z[f"{name}_loss"])), name
+        assert abs(zl.item() - float(z[f"{name}_z"])) <= 2e-6 * abs(float(z[f"{name}_z"])) + 1e-12, name
+        assert torch.all((grad.double().cpu() - want).abs() <= 2e-6 * want.abs() + 3e-7 / n), name
+
+
+
 @pytest.mark.gpu
 def test_hip_quantize_matches_fixture(dev):
     import coat_amd.activation.real_quantization as rq
