@@ -64,15 +64,16 @@ def make_adamw_workload(dev, shape, torch, expand=True):
                                         "numel": numel, "kernel": "k_fp8_adamw_plain"}
 
 
-def make_quantize_workload(dev, torch, transpose):
+def make_quantize_workload(dev, torch, transpose, shape=(4096, 4096)):
     from coat_amd.activation.real_quantization import fp8_quantize
     from coat_amd.activation.real_quantization._quantize_transpose import fp8_quantize_transpose
 
+    M, N = shape
     gen = torch.Generator(device="cpu").manual_seed(0)
-    x = torch.randn(4096, 4096, generator=gen)
-    x[torch.rand(4096, 4096, generator=gen) < 0.001] *= 100
+    x = torch.randn(M, N, generator=gen)
+    x[torch.rand(M, N, generator=gen) < 0.001] *= 100
     # rotate over buffer sets so that > 512 MB is touched between reuses (the 256 MB Infinity Cache stays cold)
-    nset = 12
+    nset = max(4, min(12, (640 << 20) // (M * N * 2) + 1))
     xs = [x.bfloat16().to(dev).clone() for _ in range(nset)]
     state = {"i": 0}
     fn = fp8_quantize_transpose if transpose else fp8_quantize
@@ -81,9 +82,9 @@ def make_quantize_workload(dev, torch, transpose):
         state["i"] += 1
         fn(xs[state["i"] % nset], 16, "E4M3")
 
-    nbytes = 4096 * 4096 * 2 + (2 if transpose else 1) * (4096 * 4096 + 4096 * 256 * 2)
+    nbytes = M * N * 2 + (2 if transpose else 1) * (M * N + M * N // 16 * 2)
     name = "fp8_quantize_transpose" if transpose else "fp8_quantize"
-    return step, nbytes, {"workload": f"{name} bf16 [4096,4096] QB16 e4m3, {nset} rotating inputs", "numel": 4096 * 4096,
+    return step, nbytes, {"workload": f"{name} bf16 [{M},{N}] QB16 e4m3, {nset} rotating inputs", "numel": M * N,
                           "kernel": "k_quantize_transpose" if transpose else "k_quantize_pg"}
 
 
@@ -328,6 +329,27 @@ def make_layernorm_workload(dev, torch):
                           "M": M, "N": N, "kernel": "k_layernorm_fwd, k_division_transpose, k_layernorm_bwd"}
 
 
+def make_hbm_probe_workload(dev, torch, kind):
+    """What this box's HBM delivers to simple kernels on 1 GiB: "copy" (torch's device copy: 1 GiB read + 1 GiB written),
+    "read" (this library's absmax reduction over bf16: read only), "fill" (torch's fill kernel: write only).  These are the
+    practical ceilings the streaming kernels are compared with next to the nominal 8 TB/s."""
+    from coat_amd import _hip
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+    if kind == "copy":
+        dst = torch.empty_like(src)
+        return (lambda: dst.copy_(src)), 2 * n, {"workload": "hbm_probe copy: torch device copy of 1 GiB", "kernel": "copy"}
+    if kind == "fill":
+        return (lambda: src.fill_(3)), n, {"workload": "hbm_probe fill: torch fill of 1 GiB", "kernel": "fill"}
+    x = src.view(torch.bfloat16)
+    amax = torch.zeros((), dtype=torch.float32, device=dev)
+
+    def step():
+        _hip.check(_hip.lib().coat_absmax(_hip.ptr(x), _hip.dt(x), _hip.ptr(amax), x.numel(), _hip.stream(dev)), "absmax")
+
+    return step, n, {"workload": "hbm_probe read: coat_absmax over 1 GiB of bf16", "kernel": "k_absmax"}
+
+
 def make_division_workload(dev, torch, stochastic):
     """Per-tensor division bf16 [8192,4096] -> e5m2 with a given scale, deterministic or with the reference's stochastic
     rounding (coat/activation/real_quantization/_division.py:153-207): 2 bytes read + 1 written per element."""
@@ -511,8 +533,11 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adamw", choices=["adamw", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
-                             "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr", "olmo_block", "layer_7b", "layer_13b"])
+                             "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr", "olmo_block",
+                             "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--shape", type=int, nargs=2, default=[4096, 4096], metavar=("M", "N"),
+                    help="input shape of the quantize / quantize_transpose workloads (default: the headline [4096, 4096])")
     ap.add_argument("--grad-format", default="e5m2", choices=["e5m2", "e4m3"],
                     help="FP8 format of the gradient operand of gemm_dgrad / gemm_wgrad (the reference's default is e5m2)")
     ap.add_argument("--ramp-seconds", type=float, default=1.5,
@@ -547,6 +572,8 @@ def main():
         step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1], args.grad_format)
     elif args.workload == "cross_entropy":
         step, nbytes, cfg = make_cross_entropy_workload(dev, torch)
+    elif args.workload.startswith("hbm_"):
+        step, nbytes, cfg = make_hbm_probe_workload(dev, torch, args.workload.split("_")[1])
     elif args.workload == "layernorm":
         step, nbytes, cfg = make_layernorm_workload(dev, torch)
     elif args.workload in ("division", "division_sr"):
@@ -556,7 +583,7 @@ def main():
     elif args.workload == "rmsnorm":
         step, nbytes, cfg = make_rmsnorm_workload(dev, torch)
     else:
-        step, nbytes, cfg = make_quantize_workload(dev, torch, args.workload == "quantize_transpose")
+        step, nbytes, cfg = make_quantize_workload(dev, torch, args.workload == "quantize_transpose", tuple(args.shape))
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -595,14 +622,14 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8" if is_gemm else "f32", "data": "synthetic", "config": cfg,
         "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload) if args.shape == [4096, 4096] else None,
                      ("algorithmic_flops_per_launch" if is_gemm else "algorithmic_bytes_per_launch"): nbytes, "kernel_ms_avg": round(avg_ms, 5),
                      "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
                      "kernel_ms_p20": round(kern_ms[len(kern_ms) // 5], 5), "kernel_ms_p80": round(kern_ms[(4 * len(kern_ms)) // 5], 5)},
     }
     if args.workload == "adamw" and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_adamw(torch)
-    elif args.workload in ("quantize", "quantize_transpose") and not args.no_cpu_baseline:
+    elif args.workload in ("quantize", "quantize_transpose") and not args.no_cpu_baseline and args.shape == [4096, 4096]:
         out["cpu_baseline"] = cpu_baseline_quantize(torch, args.workload == "quantize_transpose", nbytes)
     else:
         out["cpu_baseline"] = None
