@@ -287,22 +287,38 @@ __global__ __launch_bounds__(256) void k_division_transpose(const void* __restri
         r = 1.0f / s;
         fast = s >= kMinFastDivScale && s < 0x1p100f;
     }
-    // phase 1: each job converts 16 consecutive elements of one row into 4 dwords of the tile
+    // phase 1: each job converts 16 consecutive elements of one row into 4 dwords of the tile.  All loads of the
+    // thread's jobs are issued before the first conversion.
     constexpr int JOBS = TM * (kTileN / 16);
-    for (int job = threadIdx.x; job < JOBS; job += 256) {
-        int row = job / (kTileN / 16), c16 = job % (kTileN / 16);
-        int64_t m = m0 + row, n = n0 + c16 * 16;
+    static_assert(JOBS % 256 == 0, "whole iterations");
+    constexpr int NIT = JOBS / 256;
+    constexpr int VEC = VecOf<XDT>::kVec;
+    constexpr int LPJ = RAW ? 1 : 16 / VEC;        // 16-byte loads per job
+    constexpr int ESIZE = RAW ? 1 : 16 / VEC;      // bytes per input element
+    uint4 raw[NIT][LPJ];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * 256;
+        const int64_t m = m0 + job / (kTileN / 16), n = n0 + (job % (kTileN / 16)) * 16;
+        const bool ok = m < M && n < N;
+#pragma unroll
+        for (int h = 0; h < LPJ; h++)
+            raw[it][h] = ok ? *(const uint4*)((const uint8_t*)x + (m * N + n) * ESIZE + h * 16) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * 256;
+        const int row = job / (kTileN / 16), c16 = job % (kTileN / 16);
+        const int64_t m = m0 + row, n = n0 + c16 * 16;
         uint32_t c[4] = {0, 0, 0, 0};
         if (m < M && n < N) {
             if (RAW) {
-                uint4 t = *(const uint4*)((const uint8_t*)x + m * N + n);
-                c[0] = t.x; c[1] = t.y; c[2] = t.z; c[3] = t.w;
+                c[0] = raw[it][0].x; c[1] = raw[it][0].y; c[2] = raw[it][0].z; c[3] = raw[it][0].w;
             } else {
-                constexpr int VEC = VecOf<XDT>::kVec;
 #pragma unroll
                 for (int h = 0; h < 16 / VEC; h++) {
                     float v[VEC];
-                    load_vec<XDT>(x, m * N + n + h * VEC, v);
+                    unpack_vec<XDT>(raw[it][RAW ? 0 : h], v);
                     if (SR) quantize_vec_sr<KIND, VEC>(v, s, r, fast, (uint32_t)(m * N + n + h * VEC), k0, k1, c + h * (VEC / 4));
                     else if (fast) quantize_vec<KIND, VEC>(v, s, r, c + h * (VEC / 4));
                     else quantize_vec_slow<KIND, VEC>(v, s, c + h * (VEC / 4));
