@@ -355,7 +355,12 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
     // whole bands of rows of x and q (long contiguous runs for the memory controllers) and the hardware balances the
     // rest.  Measured on bf16 [8192, 11008] against pairs of tiles walked down the columns per XCD with register
     // prefetch: 89 us instead of 118 us; more tiles per block were slower (4: 105 us, 8: 117 us).
-    const int64_t tm = (int64_t)blockIdx.x / tiles_n, tn = (int64_t)blockIdx.x % tiles_n;
+    // tile rows are padded to a multiple of 8 blocks: blocks go round-robin over the 8 XCDs, so the tiles of one tile
+    // column then share an XCD and the 8-byte pieces they write into the same line of the transposed scales meet in one
+    // L2 (2 % on [8192, 11008], where a tile row has 86 tiles)
+    const int64_t tn_pad = (tiles_n + 7) & ~(int64_t)7;
+    const int64_t tm = (int64_t)blockIdx.x / tn_pad, tn = (int64_t)blockIdx.x % tn_pad;
+    if (tn >= tiles_n) return;
     const int64_t m0 = tm * TM, n0 = tn * TN;
 
     // phase-1 jobs: VEC consecutive elements (16 bytes); a row of the tile is TN/VEC jobs (a multiple of LPG)
@@ -613,7 +618,7 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
     hipStream_t st = (hipStream_t)stream;
     // 64 x 128 tiles for QB <= 64 (33 KiB of LDS: four blocks per CU), 128 x 128 for QB = 128
     const int TMh = QB == 128 ? 128 : 64, TNh = 128;
-    const int64_t blocks = ((M + TMh - 1) / TMh) * ((N + TNh - 1) / TNh);  // one tile per block, row-major
+    const int64_t blocks = ((M + TMh - 1) / TMh) * ((((N + TNh - 1) / TNh) + 7) & ~(int64_t)7);  // one tile per block, row-major
     if (blocks >= ((int64_t)1 << 31)) return COAT_ESHAPE;
 #define LAUNCH_QT(QBV, TMV, TNV)                                                                                     \
     DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                 \
