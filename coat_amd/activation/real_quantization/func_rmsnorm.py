@@ -30,10 +30,25 @@ def fp8_rmsnorm_forward(x, s_x, w, QB, eps, transpose_output_2d=False):
 
 
 def fp8_rmsnorm_backward(x, s_x, g, w, v, QB, num_warps):
-    """Returns (dx bf16, dw in w's dtype); ``v`` is the rstd saved by the forward."""
+    """Returns (dx bf16, dw in w's dtype); ``v`` is the rstd saved by the forward.
+
+    ``g`` may also be a tuple of two or three bf16 gradients of the normalised tensor: the kernel then uses
+    ``g[0] + g[1] (+ g[2])`` with the roundings of that chain of bf16 additions (what the reference's modules compute
+    before the call, coat/models/coat_llama.py:328 and :742), without the separate passes over the tensors."""
     x, s_x, batch = prep_pg(x, s_x)
+    extra = [None, None]
+    if isinstance(g, (tuple, list)):
+        if not 1 <= len(g) <= 3:
+            raise ValueError("fp8_rmsnorm_backward takes one to three gradients")
+        more = [prep_bf16(t) for t in g[1:]]
+        g = g[0]
+        for i, t in enumerate(more):
+            extra[i] = t
     g = prep_bf16(g)
     M, N = g.shape
+    for t in extra:
+        if t is not None and t.shape != g.shape:
+            raise ValueError("the gradients must have the same shape")
     w = _hip.dense(w)
     rstd = _hip.dense(v.to(torch.float32))
     dx = torch.empty_like(g, dtype=torch.bfloat16)
@@ -41,6 +56,7 @@ def fp8_rmsnorm_backward(x, s_x, g, w, v, QB, num_warps):
     nparts = min(_DW_PARTIALS, M)
     partial = torch.empty((nparts, N), dtype=torch.float32, device=w.device)
     _hip.check(_hip.lib().coat_fp8_rmsnorm_backward(
-        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(g), _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd),
+        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(g), _hip.ptr(extra[0]), _hip.ptr(extra[1]),
+        _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd),
         _hip.ptr(dx), _hip.ptr(dw), _hip.ptr(partial), nparts, M, N, QB, _hip.stream(x.device)), "fp8_rmsnorm_backward")
     return restore(dx, batch), dw

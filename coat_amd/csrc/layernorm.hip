@@ -26,17 +26,6 @@ template <int WMODE> __device__ __forceinline__ void load_wb16(const void* w, in
         load_w16<WMODE == kNoParam ? kF32 : WMODE>(w, col, o);
     }
 }
-__device__ __forceinline__ void load_bf16_16(const void* p, int64_t off, float* v) {
-    const uint4* src = (const uint4*)((const uint16_t*)p + off);
-    uint4 a = src[0], b = src[1];
-    uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-        v[2 * k] = bf16lo(u[k]);
-        v[2 * k + 1] = bf16hi(u[k]);
-    }
-}
-
 // Forward: y = (x - mean) * rstd (* w + b) in fp32, mean[row], rstd[row], row scale (max|y| + 1e-10)/fp8max (bf16),
 // tensor max of the row scales.
 template <int KIND, int WMODE, int ITERS>

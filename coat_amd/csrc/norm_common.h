@@ -58,6 +58,16 @@ template <int WDT> __device__ __forceinline__ void load_w16(const void* w, int c
         }
     }
 }
+__device__ __forceinline__ void load_bf16_16(const void* p, int64_t off, float* v) {
+    const uint4* src = (const uint4*)((const uint16_t*)p + off);
+    const uint4 a = src[0], b = src[1];
+    const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        v[2 * k] = bf16lo(u[k]);
+        v[2 * k + 1] = bf16hi(u[k]);
+    }
+}
 __device__ __forceinline__ void store_bf16_16(void* p, int64_t off, const float* v) {
     uint32_t w[8];
 #pragma unroll

@@ -65,7 +65,8 @@ __global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__
 // Backward: dx = bf16((w*dy - xhat * mean(xhat*w*dy)) * rstd); per-block partial of dw = sum_rows dy * xhat.
 template <int KIND, int WDT, int ITERS>
 __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
-                                                      const void* __restrict__ dy, const void* __restrict__ w,
+                                                      const void* __restrict__ dy, const void* __restrict__ dy2,
+                                                      const void* __restrict__ dy3, const void* __restrict__ w,
                                                       const float* __restrict__ rstd_in, void* __restrict__ dx,
                                                       float* __restrict__ dw_partial, int64_t M, int N, int qb) {
     __shared__ float smem[4];
@@ -86,14 +87,18 @@ __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__
                 float xv[16], wv[16], gv[16];
                 dequant16<KIND>(q, s, s_dt, row_off, srow_off, col, qb, xv);
                 load_w16<WDT>(w, col, wv);
-                {
-                    const uint4* src = (const uint4*)((const uint16_t*)dy + row_off + col);
-                    uint4 a = src[0], b = src[1];
-                    uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+                load_bf16_16(dy, row_off + col, gv);
+                // optional further gradients of the same tensor, summed the way a chain of bf16 tensor additions
+                // would: (dy + dy2) rounded to bf16, then + dy3 rounded to bf16 (block-uniform branches)
+                if (dy2) {
+                    float g2[16];
+                    load_bf16_16(dy2, row_off + col, g2);
 #pragma unroll
-                    for (int k = 0; k < 8; k++) {
-                        gv[2 * k] = bf16lo(u[k]);
-                        gv[2 * k + 1] = bf16hi(u[k]);
+                    for (int i = 0; i < 16; i++) gv[i] = round_to<kBF16>(gv[i] + g2[i]);
+                    if (dy3) {
+                        load_bf16_16(dy3, row_off + col, g2);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) gv[i] = round_to<kBF16>(gv[i] + g2[i]);
                     }
                 }
 #pragma unroll
@@ -174,16 +179,19 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
 }
 
 extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
-                                         const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
-                                         float* dw_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream) {
+                                         const void* dy2, const void* dy3, const void* w, int w_dtype, const float* rstd,
+                                         void* dx, void* dw, float* dw_partial, int n_partial, int64_t M, int64_t N,
+                                         int QB, void* stream) {
     if (int e = rms_check(M, N, QB)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x || !s_x || !dy || !w || !rstd || !dx || !dw || !dw_partial || n_partial <= 0) return COAT_EINVAL;
-    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(dy) || !coat_aligned16(dx) || !coat_aligned16(dw_partial))
+    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(dy) || !coat_aligned16(dx) || !coat_aligned16(dw_partial) ||
+        !coat_aligned16(dy2) || !coat_aligned16(dy3))
         return COAT_EALIGN;
+    if (dy3 && !dy2) return COAT_EINVAL;
     hipStream_t st = (hipStream_t)stream;
     const int64_t grid = n_partial < M ? n_partial : M;
-    RMS_DISPATCH(k_rmsnorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, rstd, dx, dw_partial, M, (int)N, QB)
+    RMS_DISPATCH(k_rmsnorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB)
     if (int e = coat_launch_status()) return e;
     const int cols_blocks = (int)((N + 31) / 32);
     switch (w_dtype) {

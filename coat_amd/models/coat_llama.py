@@ -182,8 +182,8 @@ class _CoatLlamaBeforeAttentionResidual(torch.autograd.Function):
             dx, dw = fp8_linear_backward(ln_x_t, ln_s, g8, gs, g8_t, w_t, w_s, group_size)
             dgrads.append(dx)
             wgrads.append(dw)
-        fc1_g = dgrads[0] + dgrads[1] + dgrads[2]
-        in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, fc1_g, rms_weight, rstd, group_size, num_warps)
+        # fc1_g = dgrads[0] + dgrads[1] + dgrads[2] (reference :328), summed inside the kernel with the same roundings
+        in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, tuple(dgrads), rms_weight, rstd, group_size, num_warps)
         re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],
                                                                 stochastic=False)
         # the per-group scale tensor is returned as the "gradient" of the forward scales so that shapes match;
@@ -316,8 +316,8 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
         w2_t = _backward_weight_t(w2_saved, w2_s, qargs, fwobits)
         fc1_g, weight1_grad = fp8_linear_backward(ln_x_t, ln_s, silu_g, silu_gs, silu_g_t, w1_t, w1_s, group_size)
         fc2_g, weight2_grad = fp8_linear_backward(ln_x_t, ln_s, mul_g2, mul_gs2, mul_g2_t, w2_t, w2_s, group_size)
-        fc_g = fc1_g + fc2_g
-        in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, fc_g, rms_weight, rstd, group_size, num_warps)
+        # fc_g = fc1_g + fc2_g (reference :742), summed inside the kernel
+        in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, (fc1_g, fc2_g), rms_weight, rstd, group_size, num_warps)
         re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],
                                                                 stochastic=False)
         return (re_g, in_g.view(E4M3), in_sg_g16,

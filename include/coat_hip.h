@@ -139,10 +139,12 @@ int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtyp
                              void* stream);
 /* rq/func_rmsnorm.py:281 fp8_rmsnorm_backward (kernels :121-196, :200-220): dx bf16 [M,N], dw [N] in w's dtype.
  * dw_partial: caller-provided fp32 workspace [n_partial, N]; the kernel uses min(n_partial, M) blocks and sums their
- * partial rows in block order (deterministic, unlike the reference's lock-ordered accumulation). */
-int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* w,
-                              int w_dtype, const float* rstd, void* dx, void* dw, float* dw_partial, int n_partial,
-                              int64_t M, int64_t N, int QB, void* stream);
+ * partial rows in block order (deterministic, unlike the reference's lock-ordered accumulation).
+ * dy2 / dy3 (NULL or bf16 [M,N]): further gradients of the same tensor; the kernel uses bf16(bf16(dy + dy2) + dy3), which
+ * is what the reference's callers compute with tensor additions before the call (coat/models/coat_llama.py:328, :742). */
+int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
+                              const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
+                              float* dw_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream);
 
 /* rq/func_layernorm_noparam.py:193 fp8_layernorm_noparam_forward (kernel :53-115) and rq/func_layernorm_param.py:258
  * fp8_layernorm_param_forward (kernel :51-125): y fp32 [M,N] = (x - mean) * rstd (* w + b); mean, rstd [M] fp32;

@@ -245,6 +245,22 @@ def test_fused_silu_mul_on_column_slices_and_joined_backward(dev, QBv):
     assert gs_.item() == ds_.item() and torch.equal(b(gq), b(dq)) and torch.equal(b(uqt), b(eqt))
 
 
+def test_rmsnorm_backward_sums_gradients_like_bf16_additions(dev):
+    """g given as a tuple: identical to adding the bf16 tensors first (the reference's callers do that with torch)."""
+    rq = _rq()
+    M, N = 96, 1024
+    x = rand(50, shape=(M, N))
+    w = (1 + 0.1 * rand(51, shape=(N,)).float()).bfloat16()
+    g1, g2, g3 = rand(52, 0.01, shape=(M, N)), rand(53, 0.01, shape=(M, N)), rand(54, 0.02, shape=(M, N))
+    q, s = rq.fp8_quantize(x.to(dev), 16, "E4M3")
+    _, _, _, (_, rstd, nw) = rq.fp8_rmsnorm_forward(q, s, w.to(dev), 16, 1e-5, transpose_output_2d=True)
+    d1, d2, d3 = g1.to(dev), g2.to(dev), g3.to(dev)
+    for gs, summed in (((d1, d2), d1 + d2), ((d1, d2, d3), d1 + d2 + d3), ((d1,), d1)):
+        dx_t, dw_t = rq.fp8_rmsnorm_backward(q, s, gs, w.to(dev), rstd, 16, nw)
+        dx_s, dw_s = rq.fp8_rmsnorm_backward(q, s, summed, w.to(dev), rstd, 16, nw)
+        assert torch.equal(dx_t, dx_s) and torch.equal(dw_t, dw_s)
+
+
 def test_larger_groups_and_float32_scales(dev):
     rq = _rq()
     x1, x2 = rand(13, shape=(128, 512)), rand(14, shape=(128, 512))
