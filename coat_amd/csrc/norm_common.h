@@ -81,15 +81,16 @@ __device__ __forceinline__ void store_bf16_16(void* p, int64_t off, const float*
 template <int WDT>
 __global__ __launch_bounds__(256) void k_norm_colsum(const float* __restrict__ partial, void* __restrict__ dw, int nblocks,
                                                      int N) {
-    // 32 columns per block, the partial rows split over 8 thread slices (fixed order: deterministic), 8 loads in flight
-    __shared__ float red[8][32];
-    const int c = threadIdx.x & 31, slice = threadIdx.x >> 5;
-    const int col = blockIdx.x * 32 + c;
+    // 16 columns per block (256 blocks for N = 4096, one per CU), the partial rows split over 16 thread slices in a fixed
+    // order (deterministic), 8 loads in flight per thread
+    __shared__ float red[16][16];
+    const int c = threadIdx.x & 15, slice = threadIdx.x >> 4;
+    const int col = blockIdx.x * 16 + c;
     float acc[8];
 #pragma unroll
     for (int u = 0; u < 8; u++) acc[u] = 0.0f;
     if (col < N) {
-        for (int b0 = slice * 8; b0 < nblocks; b0 += 64) {
+        for (int b0 = slice * 8; b0 < nblocks; b0 += 128) {
 #pragma unroll
             for (int u = 0; u < 8; u++)
                 if (b0 + u < nblocks) acc[u] += partial[(int64_t)(b0 + u) * N + col];
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(256) void k_norm_colsum(const float* __restrict__ p
     if (slice == 0 && col < N) {
         float s = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 8; k++) s += red[k][c];
+        for (int k = 0; k < 16; k++) s += red[k][c];
         store_from_f32<WDT>(dw, col, s);
     }
 }

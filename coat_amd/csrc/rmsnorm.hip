@@ -193,7 +193,7 @@ extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x
     const int64_t grid = n_partial < M ? n_partial : M;
     RMS_DISPATCH(k_rmsnorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB)
     if (int e = coat_launch_status()) return e;
-    const int cols_blocks = (int)((N + 31) / 32);
+    const int cols_blocks = (int)((N + 15) / 16);
     switch (w_dtype) {
         case COAT_F32: hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
         case COAT_BF16: hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
