@@ -12,3 +12,23 @@ static inline int coat_launch_status() {
 }
 // Kernels move 16 bytes per lane; NULL (an optional output that is absent) counts as aligned.
 static inline bool coat_aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// The current device's index, bounded for the per-device caches below (a process normally drives one GPU).
+constexpr int kCoatMaxDevices = 64;
+static inline int coat_device_index() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kCoatMaxDevices) return -1;
+    return dev;
+}
+// Raises a kernel's dynamic-LDS limit once per device (the attribute is per device, the kernels are templates: each
+// instantiation passes its own flag array).
+template <typename K> static inline int coat_allow_lds(K kernel, int bytes, bool* done_per_device) {
+    const int dev = coat_device_index();
+    if (dev < 0) return COAT_EINVAL;
+    if (!done_per_device[dev]) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return (int)e;
+        done_per_device[dev] = true;
+    }
+    return COAT_OK;
+}

@@ -400,25 +400,23 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     G.tiles_m = (int)((M + BM - 1) / BM);
     G.tiles_n = (int)((N + BN - 1) / BN);
     const int ntiles = G.tiles_m * G.tiles_n;
-    static int n_cu = 0;  // persistent grid: one block per CU (the block's LDS ring takes a whole CU's LDS)
-    if (n_cu == 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 8)
-            return COAT_EINVAL;
-        n_cu = v & ~7;
+    // persistent grid: one block per CU (the block's LDS ring takes a whole CU's LDS); CU count cached per device
+    static int n_cu_dev[kCoatMaxDevices] = {};
+    const int dev = coat_device_index();
+    if (dev < 0) return COAT_EINVAL;
+    if (n_cu_dev[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 8) return COAT_EINVAL;
+        n_cu_dev[dev] = v & ~7;
     }
+    const int n_cu = n_cu_dev[dev];
     const int grid = min(((ntiles + 7) / 8) * 8, n_cu);
     const size_t lds_bytes = kLdsBytes;
     hipStream_t st = (hipStream_t)stream;
 #define GEMM_LAUNCH_V(FA, FB, EP, V16)                                                                                  \
     {                                                                                                              \
-        static bool attr_set = false;                                                                              \
-        if (!attr_set) {                                                                                           \
-            hipError_t e = hipFuncSetAttribute((const void*)k_fp8_gemm<FA, FB, EP, V16>,                 \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);        \
-            if (e != hipSuccess) return (int)e;                                                                    \
-            attr_set = true;                                                                                       \
-        }                                                                                                          \
+        static bool lds_ok[kCoatMaxDevices] = {};                                                                  \
+        if (int e = coat_allow_lds(k_fp8_gemm<FA, FB, EP, V16>, (int)lds_bytes, lds_ok)) return e;                 \
         hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, V16>), dim3(grid), dim3(512), lds_bytes, st, G); \
         return coat_launch_status();                                                                               \
     }
