@@ -424,6 +424,90 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
     }
 }
 
+// K2 for 16-bit inputs (bf16 / fp16): the tile is parked in LDS as the raw 16-bit input (exact, half the footprint of
+// fp32), which makes a 128 x 128 tile fit four times per CU: q, q^T and both scale tensors are then written in whole
+// 128-byte lines / 16-byte scale pieces.  Phase 2 reads one dword = two neighbouring columns of one row, so a lane owns
+// a column pair over a 16-row chunk (two 16-byte stores into neighbouring q^T rows); chunks vary fastest over the
+// lanes, so 8 neighbouring lanes complete one 128-byte q^T line.
+template <int XDT, int SDT, int KIND, int QB>
+__global__ __launch_bounds__(256) void k_quantize_transpose16(const void* __restrict__ x, void* __restrict__ q,
+                                                               void* __restrict__ s_out, void* __restrict__ qt,
+                                                               void* __restrict__ st_out, int64_t M, int64_t N) {
+    static_assert(XDT != kF32, "16-bit inputs only");
+    constexpr int T = 128;            // tile edge
+    constexpr int PDW = T / 2 + 1;    // row pitch in dwords (odd: column reads spread over the banks)
+    constexpr int LPG = QB / 8;       // lanes per row-direction group (8 elements per lane)
+    __shared__ uint32_t tile[T * PDW];
+    enable_fp8_saturation();
+    const int64_t tiles_n = (N + T - 1) / T;
+    const int64_t SN = N / QB, SM = M / QB;
+    const int64_t tn_pad = (tiles_n + 7) & ~(int64_t)7;  // see k_quantize_transpose
+    const int64_t tm = (int64_t)blockIdx.x / tn_pad, tn = (int64_t)blockIdx.x % tn_pad;
+    if (tn >= tiles_n) return;
+    const int64_t m0 = tm * T, n0 = tn * T;
+
+    // phase 1: 16 jobs of 8 elements per row, 8 jobs per thread; all loads first
+    constexpr int JPR = T / 8, NIT = T * JPR / 256;
+    uint4 raw[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * 256;
+        const int64_t m = m0 + job / JPR, n = n0 + (job % JPR) * 8;
+        raw[it] = (m < M && n < N) ? *(const uint4*)((const uint16_t*)x + m * N + n) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * 256;
+        const int row = job / JPR, cv = job % JPR;
+        const int64_t m = m0 + row, n = n0 + cv * 8;
+        const bool ok = m < M && n < N;  // N % QB == 0: a group is inside or outside as a whole
+        float v[8];
+        unpack_vec<XDT>(raw[it], v);
+        const float amax = cluster_max<LPG>(vec_amax<8>(v));
+        const float s = group_scale<KIND>(amax);
+        const float r = 1.0f / s;
+        uint32_t c[2];
+        quantize_vec<KIND, 8>(v, s, r, c);
+        if (ok) {
+            store_codes<8>(q, m * N + n, c);
+            if ((threadIdx.x % LPG) == 0) store_from_f32<SDT>(s_out, m * SN + n / QB, s);
+        }
+        uint32_t* dst = tile + row * PDW + cv * 4;
+        dst[0] = raw[it].x; dst[1] = raw[it].y; dst[2] = raw[it].z; dst[3] = raw[it].w;
+    }
+    __syncthreads();
+
+    // phase 2: job = (column pair cp, 16-row chunk mc), mc fastest; groups of QB rows are QB/16 neighbouring lanes
+    constexpr int MC = T / 16, LPG_T = QB / 16, JOBS2 = MC * (T / 2);
+#pragma unroll
+    for (int j0 = 0; j0 < JOBS2; j0 += 256) {
+        const int job = j0 + threadIdx.x;
+        const int mc = job % MC, cp = job / MC;
+        const int64_t m = m0 + mc * 16, n = n0 + 2 * cp;
+        const bool ok = m < M && n < N;  // M % QB == 0 and N even: whole groups, whole pairs
+        float v0[16], v1[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const uint32_t w = tile[(mc * 16 + i) * PDW + cp];
+            v0[i] = XDT == kBF16 ? bf16lo(w) : f16lo(w);
+            v1[i] = XDT == kBF16 ? bf16hi(w) : f16hi(w);
+        }
+        const float s0 = group_scale<KIND>(cluster_max<LPG_T>(vec_amax<16>(v0)));
+        const float s1 = group_scale<KIND>(cluster_max<LPG_T>(vec_amax<16>(v1)));
+        uint32_t c0[4], c1[4];
+        quantize_vec<KIND, 16>(v0, s0, 1.0f / s0, c0);
+        quantize_vec<KIND, 16>(v1, s1, 1.0f / s1, c1);
+        if (ok) {
+            *(uint4*)((uint8_t*)qt + n * M + m) = make_uint4(c0[0], c0[1], c0[2], c0[3]);
+            *(uint4*)((uint8_t*)qt + (n + 1) * M + m) = make_uint4(c1[0], c1[1], c1[2], c1[3]);
+            if ((mc % LPG_T) == 0) {
+                store_from_f32<SDT>(st_out, n * SM + m / QB, s0);
+                store_from_f32<SDT>(st_out, (n + 1) * SM + m / QB, s1);
+            }
+        }
+    }
+}
+
 }  // namespace coat
 
 // ================================================================================================ C ABI
@@ -631,6 +715,29 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
                            kLds, st, x, q, s, qt, st_out, M, N);                                                     \
         return coat_launch_status();                                                                                 \
     })))
+    if (x_dtype != COAT_F32) {  // 16-bit inputs: 128 x 128 tiles parked in LDS as 16-bit values
+        const int64_t tn16 = (N + 127) / 128;
+        const int64_t blocks16 = ((M + 127) / 128) * ((tn16 + 7) & ~(int64_t)7);
+        if (blocks16 >= ((int64_t)1 << 31)) return COAT_ESHAPE;
+#define LAUNCH_QT16(XD, QBV)                                                                                          \
+    DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                                        \
+        hipLaunchKernelGGL((k_quantize_transpose16<XD, SDT, KIND, QBV>), dim3((unsigned)blocks16), dim3(256), 0, st, x, q, \
+                           s, qt, st_out, M, N);                                                                      \
+        return coat_launch_status();                                                                                  \
+    }))
+#define LAUNCH_QT16_QB(XD)                                  \
+    switch (QB) {                                           \
+        case 16: LAUNCH_QT16(XD, 16); break;                \
+        case 32: LAUNCH_QT16(XD, 32); break;                \
+        case 64: LAUNCH_QT16(XD, 64); break;                \
+        case 128: LAUNCH_QT16(XD, 128); break;              \
+        default: return COAT_ESHAPE;                        \
+    }
+        if (x_dtype == COAT_BF16) { LAUNCH_QT16_QB(kBF16) } else if (x_dtype == COAT_F16) { LAUNCH_QT16_QB(kF16) }
+#undef LAUNCH_QT16_QB
+#undef LAUNCH_QT16
+        return COAT_EDTYPE;
+    }
     switch (QB) {
         case 16: LAUNCH_QT(16, 64, 128); break;
         case 32: LAUNCH_QT(32, 64, 128); break;
