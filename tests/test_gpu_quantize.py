@@ -73,7 +73,7 @@ def test_fp8_quantize_3d_and_scale_dtype(dev):
         rq.fp8_quantize(torch.zeros(4, 40, dtype=torch.bfloat16, device=dev), 16, "E4M3")  # N % QB != 0
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("fp8,QB,M,N", [("E4M3", 16, 128, 192), ("E5M2", 16, 64, 64), ("E4M3", 32, 96, 160),
                                         ("E4M3", 64, 128, 128), ("E4M3", 16, 16, 16), ("E4M3", 16, 208, 80),
                                         ("E4M3", 128, 384, 640), ("E5M2", 128, 128, 128)])
