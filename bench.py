@@ -369,7 +369,7 @@ def make_division_workload(dev, torch, stochastic):
                             "kernel": "k_division"}
 
 
-def make_layer_workload(dev, torch, size):
+def make_layer_workload(dev, torch, size, cache_weights=False):
     """COAT Llama decoder layer fwd+bwd, batch 4 x seq 2048, random init N(0, 0.02)."""
     from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
     from coat_amd.models.coat_llama import CoatLlamaConfig, CoatLlamaDecoderLayer
@@ -378,7 +378,10 @@ def make_layer_workload(dev, torch, size):
     H, heads, I = (4096, 32, 11008) if size == "7b" else (5120, 40, 13824)
     B, S = 4, 2048
     torch.manual_seed(0)
-    cfg = CoatLlamaConfig(hidden_size=H, intermediate_size=I, num_attention_heads=heads)
+    # cache_weights: weight_memory_efficient=False, i.e. FP8 weights and their transposes are kept from the first
+    # micro-batch on (coat/utils/_fp8_weightcache.py:11-37) instead of being re-quantized in every forward and backward
+    cfg = CoatLlamaConfig(hidden_size=H, intermediate_size=I, num_attention_heads=heads,
+                          coat_fp8_args={"weight_memory_efficient": not cache_weights})
     layer = CoatLlamaDecoderLayer(cfg, 0)
     for p in layer.parameters():
         if p.dim() == 2:
@@ -409,7 +412,8 @@ def make_layer_workload(dev, torch, size):
     gemm_flops = 3 * 2 * B * S * (4 * H * H + 3 * H * I)
     return step_fp8, step_bf16, gemm_flops, {
         "workload": f"CoatLlamaDecoderLayer fwd+bwd, Llama-2-{size.upper()} shape (H {H}, heads {heads}, I {I}), "
-                    f"batch {B} x seq {S}, FP8 linears/activations/norms, bf16 SDPA attention",
+                    f"batch {B} x seq {S}, FP8 linears/activations/norms, bf16 SDPA attention"
+                    + (", FP8 weights cached across micro-batches" if cache_weights else ""),
         "tokens": B * S, "gemm_flops": gemm_flops}
 
 
@@ -490,7 +494,7 @@ def bench_layer(args, dev, torch):
     elif args.workload == "olmo_block":
         step_fp8, step_bf16, gemm_flops, cfg = make_olmo_workload(dev, torch)
     else:
-        step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1])
+        step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1], args.cache_weights)
 
     def time_it(fn):
         ramp_clocks(fn, args.ramp_seconds, torch)
@@ -538,6 +542,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", type=int, nargs=2, default=[4096, 4096], metavar=("M", "N"),
                     help="input shape of the quantize / quantize_transpose workloads (default: the headline [4096, 4096])")
+    ap.add_argument("--cache-weights", action="store_true",
+                    help="layer workloads: weight_memory_efficient=False (FP8 weights cached after the first micro-batch)")
     ap.add_argument("--grad-format", default="e5m2", choices=["e5m2", "e4m3"],
                     help="FP8 format of the gradient operand of gemm_dgrad / gemm_wgrad (the reference's default is e5m2)")
     ap.add_argument("--ramp-seconds", type=float, default=1.5,
