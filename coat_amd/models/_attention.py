@@ -6,7 +6,6 @@ calls ``torch.nn.functional.scaled_dot_product_attention``.  On this ROCm build 
 default; for the shapes of the decoder layers (batch 4, 32 heads, 2048 tokens, head dimension 128, causal) its
 "memory-efficient" backend runs forward + backward in 1.40 ms against 2.66 ms, so that one is tried first and the
 others stay as fallbacks for arguments it does not take.  The mathematics is the same."""
-import torch
 import torch.nn.functional as F
 from torch.nn.attention import SDPBackend, sdpa_kernel
 

@@ -15,7 +15,6 @@ is the tensor's scale.
 This file does not depend on the ``transformers`` package: the configuration is a plain attribute holder and the
 rotary embedding / causal SDPA are written out here.  Whole-model classes (CausalLM, HF registration) are out of scope.
 """
-import math
 from typing import Optional, Tuple
 
 import torch
@@ -25,9 +24,8 @@ import torch.nn.functional as F
 from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt, fp8_division,
                                             fp8_division_transpose, fp8_linear_backward, fp8_linear_forward,
-                                            fp8_mul_backward, fp8_mul_forward, fp8_quantize_pertensor,
-                                            fp8_quantize_pertensor_transpose, fp8_rmsnorm_backward,
-                                            fp8_rmsnorm_forward, fp8_silu_backward, fp8_silu_forward, fp8_silu_mul_backward,
+                                            fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
+                                            fp8_rmsnorm_backward, fp8_rmsnorm_forward, fp8_silu_mul_backward,
                                             fp8_silu_mul_forward, fp8_transpose)
 from ..utils._fp8_quantization_config import QuantizationConfig
 from ..utils._fp8_weightcache import FP8CacheWeightModule

@@ -1,6 +1,5 @@
 """GPU parity: stochastic-rounding division (the reference's coat/activation/real_quantization/_division.py:96-150
 branch) against the CPU oracle, bit for bit: same Philox stream, same perturbation, same FP8 codes."""
-import numpy as np
 import pytest
 import torch
 

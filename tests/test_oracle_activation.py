@@ -1,5 +1,4 @@
 """Pins oracle/activation_ref.py by closed forms, invariants and torch.nn.functional + autograd."""
-import math
 
 import pytest
 import torch

@@ -3,8 +3,6 @@ the reference test's own torch definition of the step (restated in oracle/adamw_
 torch.optim.AdamW, and the invariants of Dynamic Range Expansion."""
 import math
 
-import numpy as np
-import pytest
 import torch
 
 from oracle import adamw_ref as A
