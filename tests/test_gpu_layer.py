@@ -218,3 +218,67 @@ def test_attention_backend_choice_matches_fp32_math(dev):
     rq, rk, rv = torch.autograd.grad(ref, (qf, kf, vf), go.float())
     for a, b in ((out, ref), (gq, rq), (gk, rk), (gv, rv)):
         assert ((a.float() - b).norm() / b.norm()).item() < 1e-2
+
+
+def test_training_steps_with_coat_adamw_reduce_the_loss(dev):
+    """End to end: FP8 decoder layer + FP8-state optimizer on a fixed batch.  fp32 master weights (the optimizer kernels
+    take fp32 parameters, coat/optimizer/fp8_adamw.py:128), bf16 compute copy refreshed after every step; the loss of a
+    fixed regression target must fall, and follow the same layer trained in plain fp32 torch with torch.optim.AdamW."""
+    from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
+    from coat_amd.optimizer.fp8_adamw import CoatAdamW
+    from coat_amd.utils._fp8_quantization_config import QuantizationConfig
+    from coat_amd.utils._fp8manager import FP8Manager
+    layer, cfg = build(dev, H=256, heads=4, I=512)
+    layer.train()
+    B, S, H = 2, 64, 256
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(B, S, H, generator=g).to(dev)
+    target = torch.randn(B, S, H, generator=g).to(dev) * 0.5
+    bgn, end = Coat_quantize_bgn(layer.qargs).to(dev), Coat_quantize_end(layer.qargs).to(dev)
+    master = [p.detach().float().clone().requires_grad_(True) for p in layer.parameters()]
+    opt = CoatAdamW(master, lr=2e-3, betas=(0.9, 0.95), weight_decay=0.0, qargs=QuantizationConfig())
+    ref_params = [m.detach().clone().requires_grad_(True) for m in master]
+    names = [n for n, _ in layer.named_parameters()]
+    ref_opt = torch.optim.AdamW(ref_params, lr=2e-3, betas=(0.9, 0.95), weight_decay=0.0)
+
+    def ref_forward(xin):
+        W = dict(zip(names, ref_params))
+        B_, S_, H_ = xin.shape
+        nh = layer.self_attn.num_heads
+        hd = H_ // nh
+        from coat_amd.models.coat_llama import apply_rotary_pos_emb, rotary_cos_sin
+        h = F.rms_norm(xin, (H_,), W["input_layernorm.weight"], 1e-5)
+        q, k, v = ((h @ W[f"BeforeAttention.{n}_proj.weight"].t()).view(B_, S_, nh, hd).transpose(1, 2) for n in "qkv")
+        cos, sin = rotary_cos_sin(torch.arange(S_, device=xin.device).unsqueeze(0).expand(B_, -1), hd, 10000.0, torch.float32)
+        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(B_, S_, H_)
+        x1 = xin + a @ W["AfterAttention.o_proj.weight"].t()
+        h2 = F.rms_norm(x1, (H_,), W["post_attention_layernorm.weight"], 1e-5)
+        m = F.silu(h2 @ W["MLPResidual.gate_proj.weight"].t()) * (h2 @ W["MLPResidual.up_proj.weight"].t())
+        return x1 + m @ W["MLPResidual.down_proj.weight"].t()
+
+    losses, ref_losses = [], []
+    for step in range(25):
+        FP8Manager.is_first_microbatch = True
+        with torch.no_grad():
+            for p, m in zip(layer.parameters(), master):
+                p.copy_(m)
+        layer.zero_grad(set_to_none=True)
+        h, q, s = bgn(x.bfloat16().requires_grad_(True))
+        (h, q, s), = layer(h, q, s)
+        loss = F.mse_loss(end(h, q, s).float(), target)
+        loss.backward()
+        for p, m in zip(layer.parameters(), master):
+            m.grad = p.grad.float()
+        opt.step()
+        losses.append(loss.item())
+        ref_opt.zero_grad(set_to_none=True)
+        rl = F.mse_loss(ref_forward(x), target)
+        rl.backward()
+        ref_opt.step()
+        ref_losses.append(rl.item())
+    assert all(torch.isfinite(torch.tensor(losses)))
+    assert losses[-1] < 0.8 * losses[0], (losses[0], losses[-1])
+    # the FP8 run tracks the fp32 run: same loss within 5 % at every step
+    for a, b in zip(losses, ref_losses):
+        assert abs(a - b) <= 0.05 * b, (losses, ref_losses)
