@@ -15,7 +15,7 @@ namespace coat {
 __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab,
                                                     const int64_t* __restrict__ pos, int64_t rows, int seq_len, int heads,
-                                                    int head_dim, float sign) {
+                                                    int head_dim, float sign, int64_t x_pitch, int64_t y_pitch) {
     const int half = head_dim >> 1;
     const int cpr = half >> 3;                      // 16-byte chunks per half row
     const int64_t total = rows * heads * cpr;       // one job = 8 pairs
@@ -24,7 +24,8 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
         const int64_t rh = job / cpr;               // row * heads + head
         const int64_t row = rh / heads;
         const int64_t p = pos ? pos[row] : row % seq_len;
-        const uint16_t* src = x + rh * head_dim + c * 8;
+        const int head = (int)(rh - row * heads);
+        const uint16_t* src = x + row * x_pitch + head * head_dim + c * 8;
         const uint4 a = *(const uint4*)src, b = *(const uint4*)(src + half);
         const float4* ct = (const float4*)(cos_tab + p * half + c * 8);
         const float4* st = (const float4*)(sin_tab + p * half + c * 8);
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
             o1[k] = pack_bf16x2(x1l * cs[2 * k] - x2l * sl, x1h * cs[2 * k + 1] - x2h * sh);
             o2[k] = pack_bf16x2(x2l * cs[2 * k] + x1l * sl, x2h * cs[2 * k + 1] + x1h * sh);
         }
-        uint16_t* dst = y + rh * head_dim + c * 8;
+        uint16_t* dst = y + row * y_pitch + head * head_dim + c * 8;
         *(uint4*)dst = make_uint4(o1[0], o1[1], o1[2], o1[3]);
         *(uint4*)(dst + half) = make_uint4(o2[0], o2[1], o2[2], o2[3]);
     }
@@ -51,9 +52,15 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
 using namespace coat;
 
 extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, const int64_t* pos,
-                              int64_t rows, int seq_len, int heads, int head_dim, int inverse, void* stream) {
+                              int64_t rows, int seq_len, int heads, int head_dim, int inverse, int64_t x_pitch,
+                              int64_t y_pitch, void* stream) {
     if (rows < 0 || heads <= 0 || head_dim <= 0 || seq_len <= 0) return COAT_EINVAL;
     if (head_dim % 16 != 0) return COAT_ESHAPE;  // 8 pairs per lane
+    // row pitches in elements (0 = contiguous): x or y may be a column slice of a wider tensor (a fused q/k/v projection)
+    const int64_t width = (int64_t)heads * head_dim;
+    if (x_pitch == 0) x_pitch = width;
+    if (y_pitch == 0) y_pitch = width;
+    if (x_pitch < width || y_pitch < width || x_pitch % 8 != 0 || y_pitch % 8 != 0) return COAT_ESHAPE;
     if (rows == 0) return COAT_OK;
     if (!x || !y || !cos_tab || !sin_tab) return COAT_EINVAL;
     if (!coat_aligned16(x) || !coat_aligned16(y) || !coat_aligned16(cos_tab) || !coat_aligned16(sin_tab)) return COAT_EALIGN;
@@ -61,6 +68,6 @@ extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, cons
     int64_t blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;
     hipLaunchKernelGGL(k_rope_bf16, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
-                       (uint16_t*)y, cos_tab, sin_tab, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f);
+                       (uint16_t*)y, cos_tab, sin_tab, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f, x_pitch, y_pitch);
     return coat_launch_status();
 }

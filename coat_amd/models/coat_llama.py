@@ -378,7 +378,7 @@ class _FusedRoPE(torch.autograd.Function):
         x = _hip.dense(x)
         y = torch.empty_like(x)
         _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(x), _hip.ptr(y), _hip.ptr(cos_tab), _hip.ptr(sin_tab), _hip.ptr(pos),
-                                             B * S, S, heads, head_dim, 0, _hip.stream(x.device)), "rope forward")
+                                             B * S, S, heads, head_dim, 0, 0, 0, _hip.stream(x.device)), "rope forward")
         ctx.save_for_backward(cos_tab, sin_tab, pos)
         ctx.dims = (B, S, heads, head_dim)
         return y.view(B, S, heads, head_dim).transpose(1, 2)
@@ -391,8 +391,61 @@ class _FusedRoPE(torch.autograd.Function):
         g = _hip.dense(g.transpose(1, 2).to(torch.bfloat16))  # physically [B, S, heads, head_dim]
         dx = torch.empty_like(g)
         _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(g), _hip.ptr(dx), _hip.ptr(cos_tab), _hip.ptr(sin_tab), _hip.ptr(pos),
-                                             B * S, S, heads, head_dim, 1, _hip.stream(g.device)), "rope backward")
+                                             B * S, S, heads, head_dim, 1, 0, 0, _hip.stream(g.device)), "rope backward")
         return dx.view(B, S, heads * head_dim), None, None, None, None, None
+
+
+class _FusedQKVRoPE(torch.autograd.Function):
+    """qkv bf16 [B, S, Dq + 2 Dkv] (a fused projection's output) -> rotated q [B, heads, S, hd], rotated k
+    [B, kv_heads, S, hd] and v [B, kv_heads, S, hd] (a view of qkv).  The kernels read the q / k column slices where
+    they lie; the backward writes the two inverse rotations and dv straight into one [B, S, Dq + 2 Dkv] gradient, so
+    neither the ``.contiguous()`` copies of the slices nor the concatenation of the three gradients are needed."""
+
+    @staticmethod
+    def forward(ctx, qkv, cos_tab, sin_tab, heads, kv_heads, head_dim):
+        from .. import _hip
+        B, S, W = qkv.shape
+        Dq, Dkv = heads * head_dim, kv_heads * head_dim
+        assert W == Dq + 2 * Dkv and Dq % 8 == 0 and Dkv % 8 == 0
+        qkv = _hip.dense(qkv)
+        flat = qkv.view(B * S, W)
+        q = torch.empty((B, S, Dq), dtype=qkv.dtype, device=qkv.device)
+        k = torch.empty((B, S, Dkv), dtype=qkv.dtype, device=qkv.device)
+        lib, st = _hip.lib(), _hip.stream(qkv.device)
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, :Dq]), _hip.ptr(q), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
+                                      B * S, S, heads, head_dim, 0, W, 0, st), "rope forward (q of qkv)")
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, Dq:Dq + Dkv]), _hip.ptr(k), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
+                                      B * S, S, kv_heads, head_dim, 0, W, 0, st), "rope forward (k of qkv)")
+        ctx.save_for_backward(cos_tab, sin_tab)
+        ctx.dims = (B, S, heads, kv_heads, head_dim)
+        v = qkv[..., Dq + Dkv:].view(B, S, kv_heads, head_dim).transpose(1, 2)
+        return (q.view(B, S, heads, head_dim).transpose(1, 2), k.view(B, S, kv_heads, head_dim).transpose(1, 2), v)
+
+    @staticmethod
+    def backward(ctx, gq, gk, gv):
+        from .. import _hip
+        cos_tab, sin_tab = ctx.saved_tensors
+        B, S, heads, kv_heads, head_dim = ctx.dims
+        Dq, Dkv = heads * head_dim, kv_heads * head_dim
+        W = Dq + 2 * Dkv
+        gq = _hip.dense(gq.transpose(1, 2).to(torch.bfloat16))  # physically [B, S, heads, head_dim]
+        gk = _hip.dense(gk.transpose(1, 2).to(torch.bfloat16))
+        dqkv = torch.empty((B, S, W), dtype=torch.bfloat16, device=gq.device)
+        flat = dqkv.view(B * S, W)
+        lib, st = _hip.lib(), _hip.stream(gq.device)
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(gq), _hip.ptr(flat[:, :Dq]), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
+                                      B * S, S, heads, head_dim, 1, 0, W, st), "rope backward (q of qkv)")
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(gk), _hip.ptr(flat[:, Dq:Dq + Dkv]), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
+                                      B * S, S, kv_heads, head_dim, 1, 0, W, st), "rope backward (k of qkv)")
+        dqkv[..., Dq + Dkv:].copy_(gv.transpose(1, 2).reshape(B, S, Dkv))
+        return dqkv, None, None, None, None, None
+
+
+def fused_qkv_rotary(qkv, heads, kv_heads, head_dim, theta):
+    """RoPE on the q and k parts of a fused projection output qkv [B, S, (heads + 2 kv_heads) * head_dim] (bf16, GPU);
+    returns (q [B, heads, S, hd], k [B, kv_heads, S, hd], v [B, kv_heads, S, hd])."""
+    cos_tab, sin_tab = rotary_tables(qkv.shape[1], head_dim, theta, qkv.device)
+    return _FusedQKVRoPE.apply(qkv, cos_tab, sin_tab, heads, kv_heads, head_dim)
 
 
 def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=None):

@@ -22,7 +22,7 @@ from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_If
                                             fp8_silu_mul_backward_joined, fp8_silu_mul_forward, fp8_transpose)
 from ..utils._fp8_quantization_config import QuantizationConfig
 from .coat_llama import (E4M3, _as_e4m3_input, _as_e5m2_grad, _backward_weight_t, _forward_weight, _ResidualBase,
-                         apply_rotary_pos_emb, fused_rotary, rotary_cos_sin)
+                         apply_rotary_pos_emb, fused_qkv_rotary, fused_rotary, rotary_cos_sin)
 
 __all__ = ["CoatOLMoConfig", "CoatOLMoBeforeAttentionResidual", "CoatOLMoAfterAttentionResidual",
            "CoatOLMoMLPResidual", "CoatOLMoSequentialBlock"]
@@ -291,8 +291,18 @@ class CoatOLMoSequentialBlock(nn.Module):
         x, qkv = self.BeforeAttention(x, qx, sx)
         if self.config.clip_qkv is not None:
             qkv = qkv.clamp(min=-self.config.clip_qkv, max=self.config.clip_qkv)
-        q, k, v = qkv.split(self.fused_dims, dim=-1)
-        att = self.attention(q, k, v, attention_bias)
+        if self.config.rope and qkv.is_cuda and qkv.dtype == torch.bfloat16:
+            # RoPE reads the q / k column slices of the fused projection where they lie, and its backward writes into the
+            # fused gradient (the reference splits, copies, and concatenates the gradients again, :1003-1006)
+            B, T, _ = qkv.shape
+            C = self.fused_dims[0]
+            hd = C // self.config.n_heads
+            q, k, v = fused_qkv_rotary(qkv, self.config.n_heads, self.config.effective_n_kv_heads, hd,
+                                       self.config.rope_theta)
+            att = self._sdpa(q, k, v, attention_bias, B, T, C)
+        else:
+            q, k, v = qkv.split(self.fused_dims, dim=-1)
+            att = self.attention(q, k, v, attention_bias)
         x, qx, sx = self.AfterAttention(x, att)
         x, qx, sx = self.MLPResidual(x, qx, sx)
         return x, qx, sx, None

@@ -167,9 +167,11 @@ int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_d
  * RotaryEmbedding at coat/models/coat_olmo.py:862-863).  x, y bf16 [rows, heads, head_dim], rows = batch * seq;
  * cos_tab / sin_tab fp32 [n_pos, head_dim / 2]; pos int64 [rows] or NULL (position = row % seq_len);
  * y1 = x1 cos - x2 sin, y2 = x2 cos + x1 sin on the (d, d + head_dim/2) pairs; inverse != 0 negates the angle, which
- * is the backward pass.  head_dim % 16 == 0. */
+ * is the backward pass.  head_dim % 16 == 0.  x_pitch / y_pitch: row pitches in elements, 0 = contiguous; a multiple
+ * of 8 (16-byte rows), for x or y that is a column slice of a fused q/k/v tensor (coat/models/coat_olmo.py:1003-1006). */
 int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, const int64_t* pos,
-                   int64_t rows, int seq_len, int heads, int head_dim, int inverse, void* stream);
+                   int64_t rows, int seq_len, int heads, int head_dim, int inverse, int64_t x_pitch, int64_t y_pitch,
+                   void* stream);
 
 /* ---- GEMM -------------------------------------------------------------------------------------------
  * rq/linear.py:172 fp8matmul (kernel :61-169): C[M,N] = (A[M,K] . B[N,K]^T) * (float(*scale_a) * float(*scale_b))

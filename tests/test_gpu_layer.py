@@ -282,3 +282,26 @@ def test_training_steps_with_coat_adamw_reduce_the_loss(dev):
     # the FP8 run tracks the fp32 run: same loss within 5 % at every step
     for a, b in zip(losses, ref_losses):
         assert abs(a - b) <= 0.05 * b, (losses, ref_losses)
+
+
+def test_fused_qkv_rope_matches_the_separate_path(dev):
+    """fused_qkv_rotary on a fused projection output against split + fused_rotary per tensor: same q, k, v and the same
+    gradient of the fused tensor, bit for bit (the kernels are the same, only the addressing differs)."""
+    from coat_amd.models.coat_llama import fused_qkv_rotary, fused_rotary
+    B, S, nh, nkv, hd = 2, 48, 8, 4, 64
+    g = torch.Generator().manual_seed(21)
+    qkv = torch.randn(B, S, (nh + 2 * nkv) * hd, generator=g).bfloat16().to(dev)
+    gq = torch.randn(B, nh, S, hd, generator=g).bfloat16().to(dev)
+    gk = torch.randn(B, nkv, S, hd, generator=g).bfloat16().to(dev)
+    gv = torch.randn(B, nkv, S, hd, generator=g).bfloat16().to(dev)
+    a = qkv.clone().requires_grad_(True)
+    q, k, v = fused_qkv_rotary(a, nh, nkv, hd, 10000.0)
+    torch.autograd.backward((q, k, v), (gq, gk, gv))
+    b = qkv.clone().requires_grad_(True)
+    q2, k2, v2 = b.split((nh * hd, nkv * hd, nkv * hd), dim=-1)
+    q2 = fused_rotary(q2.contiguous(), nh, hd, 10000.0)
+    k2 = fused_rotary(k2.contiguous(), nkv, hd, 10000.0)
+    v2 = v2.view(B, S, nkv, hd).transpose(1, 2)
+    torch.autograd.backward((q2, k2, v2), (gq, gk, gv))
+    assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(v, v2)
+    assert torch.equal(a.grad, b.grad)
