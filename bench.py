@@ -7,7 +7,8 @@ weight [11008, 4096], grads N(0, 1e-3), lr 3e-4, betas (0.9, 0.95), wd 0.1, eps 
 moment state produced by nine untimed steps.  A "step" is one pass of the fused kernel over the whole tensor.
 Prints ONE JSON line.  `value` is algorithmic GB/s: every distinct input read once + every output written once
 (in-place tensors count read + write) divided by the wall-clock per step with inputs resident in HBM.
-`roofline.achieved` uses the kernel's average launch duration measured with HIP events on the launch stream.
+`roofline.achieved` uses the kernel's average launch duration: HIP events on the launch stream around the K
+back-to-back launches of the timed region, divided by K (per-launch event pairs of a second pass give the spread).
 `cpu_baseline` times the plain-C oracle (one thread) on a bounded sample of the same workload.
 """
 import argparse
@@ -601,10 +602,23 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    # HIP events around every launch, on the stream the kernels are launched on (torch's current stream)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     prepare = getattr(step, "prepare", None)
-    t0 = time.perf_counter()
+    # (1) the timed region: exactly K steps between two synchronisations, nothing else in the loop
+    wall = region_ms = None
+    if not prepare:
+        ra, rb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        ra.record()
+        for _ in range(args.steps):
+            step()
+        rb.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        region_ms = ra.elapsed_time(rb)  # HIP events over the timed region: K launches back to back
+    # (2) the same K steps again with HIP events around every launch, on the stream the kernels are launched on (torch's
+    # current stream): the kernel's own duration for the roofline (event records inside loop (1) would add their gaps
+    # to the wall clock)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     for a, b in evs:
         if prepare:
             prepare()
@@ -612,9 +626,10 @@ def main():
         step()
         b.record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     kern_ms = sorted(a.elapsed_time(b) for a, b in evs)
-    avg_ms = sum(kern_ms) / len(kern_ms)
+    # average launch duration: the event pair over the timed region divided by K; the per-launch pairs (which include
+    # the event records' own gaps) give the spread
+    avg_ms = sum(kern_ms) / len(kern_ms) if prepare else region_ms / args.steps
     ms_per_step = avg_ms if prepare else wall * 1e3 / args.steps
     value = nbytes / (ms_per_step * 1e-3) / 1e9
     achieved = nbytes / (avg_ms * 1e-3) / 1e9
@@ -631,6 +646,7 @@ def main():
                      "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload) if args.shape == [4096, 4096] else None,
                      ("algorithmic_flops_per_launch" if is_gemm else "algorithmic_bytes_per_launch"): nbytes, "kernel_ms_avg": round(avg_ms, 5),
                      "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
+                     "kernel_ms_per_launch_events_avg": round(sum(kern_ms) / len(kern_ms), 5),
                      "kernel_ms_p20": round(kern_ms[len(kern_ms) // 5], 5), "kernel_ms_p80": round(kern_ms[(4 * len(kern_ms)) // 5], 5)},
     }
     if args.workload == "adamw" and not args.no_cpu_baseline:
