@@ -16,7 +16,10 @@ def absmax_scale(x, fp8type):
     return (amax.to(x.dtype) + SCALE_MIN_THRES) / FP8_MAX_VALUE[fp8type]
 
 
-def _division(x, fp8type, s_y, want_q, want_qt, what, stochastic=False):
+def _division(x, fp8type, s_y, want_q, want_qt, what, stochastic=False, max_as=None):
+    """q and / or q^T of x divided by a per-tensor scale.  ``max_as`` (a torch dtype): ``s_y`` is the fp32 device
+    scalar into which a producer kernel merged the maximum of its group scales; the division kernel rounds it to that
+    dtype itself and writes the rounded scale, which is returned (no separate conversion launch)."""
     M, N = x.shape
     if s_y is None:
         s_y = absmax_scale(x, fp8type)
@@ -25,6 +28,16 @@ def _division(x, fp8type, s_y, want_q, want_qt, what, stochastic=False):
     s_dev = s_y if s_y.is_cuda else s_y.to(x.device)
     y = torch.empty_like(x, dtype=fp8type) if want_q else None
     y_t = torch.empty((N, M), dtype=fp8type, device=x.device) if want_qt else None
+    if max_as is not None and not stochastic and M * N > 0:
+        if s_dev.dtype != torch.float32:
+            raise ValueError(f"{what}: the running maximum must be fp32")
+        s_out = torch.empty((), dtype=max_as, device=x.device)
+        _hip.check(_hip.lib().coat_fp8_division_from_max(
+            _hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.ptr(s_out), _hip.dt(s_out), _hip.ptr(y), _hip.ptr(y_t), M, N,
+            _hip.fp8(fp8type), _hip.stream(x.device)), what)
+        return y, s_out, y_t
+    if max_as is not None:
+        s_y = s_dev = s_dev.to(max_as)
     if stochastic:
         _hip.check(_hip.lib().coat_fp8_division_stochastic(
             _hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.dt(s_dev), _hip.ptr(y), _hip.ptr(y_t), M, N,

@@ -8,17 +8,16 @@ from .common import convert_str_to_fp8, flatten_2d, new_max, restore
 
 
 def group_scales_and_max(x, QB, fp8type, scale_dtype=torch.bfloat16, want_pg=True):
-    """(s_pg [M, N/QB] or None, max scale as a 0-dim tensor of scale_dtype) in one pass over x.
+    """(s_pg [M, N/QB] or None, maximum of the fp32 group scales as a 0-dim fp32 tensor) in one pass over x.
 
-    The kernel takes the maximum of the fp32 group scales; rounding to scale_dtype is monotone, so rounding
-    the maximum equals the reference's ``s_y.max()`` over the rounded scales (reference :139)."""
+    Rounding to scale_dtype is monotone, so rounding the maximum (which the division pass does) equals the reference's ``s_y.max()`` over the rounded scales (reference :139)."""
     M, N = x.shape
     s_pg = torch.empty((M, N // QB), dtype=scale_dtype, device=x.device) if want_pg else None
     s_max = new_max(x.device)
     _hip.check(_hip.lib().coat_fp8_group_scales(_hip.ptr(x), _hip.dt(x), _hip.ptr(s_pg), _hip.dt(scale_dtype),
                                                 _hip.ptr(s_max), M, N, QB, _hip.fp8(fp8type), _hip.stream(x.device)),
                "fp8_group_scales")
-    return s_pg, s_max.to(scale_dtype)
+    return s_pg, s_max
 
 
 def fp8_quantize_pertensor(x, QB, fp8type, stochastic=False, scale_dtype=torch.bfloat16):
@@ -27,5 +26,6 @@ def fp8_quantize_pertensor(x, QB, fp8type, stochastic=False, scale_dtype=torch.b
     x = _hip.dense(x)
     fp8type = convert_str_to_fp8[fp8type]  # the reference accepts only the string here (:118)
     s_y, s_y_max = group_scales_and_max(x, QB, fp8type, scale_dtype)
-    y, s_y_max, _ = _division(x, fp8type, s_y_max, True, False, "fp8_quantize_pertensor", stochastic)
+    y, s_y_max, _ = _division(x, fp8type, s_y_max, True, False, "fp8_quantize_pertensor", stochastic,
+                                max_as=scale_dtype)
     return restore(y, batch), s_y_max, restore(s_y, batch)

@@ -18,7 +18,7 @@ def fp8_quantize_pertensor_transpose(x, QB, fp8type, transpose_output_2d=False, 
     fp8type = convert_str_to_fp8[fp8type]
     _, s_y_max = group_scales_and_max(x, QB, fp8type, scale_dtype, want_pg=False)
     qy, s_y_max, qy_t = _division(x, fp8type, s_y_max, True, True, "fp8_quantize_pertensor_transpose",
-                                   stochastic)
+                                   stochastic, max_as=scale_dtype)
     if batch is not None and not transpose_output_2d:
         qy_t = qy_t.reshape(batch, -1, qy_t.shape[-1])
     return restore(qy, batch), s_y_max, qy_t

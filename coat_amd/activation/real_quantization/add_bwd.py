@@ -24,6 +24,6 @@ def fp8_add_Ifp_Ifp_Ofp_Opt(x1, x2, QB, fp8type, stochastic=False):
     s_max = new_max(x1.device)
     _hip.check(_hip.lib().coat_fp8_add_bwd(_hip.ptr(x1), _hip.ptr(x2), _hip.ptr(y1), _hip.ptr(s_y2), _hip.ptr(s_max),
                                            _hip.fp8(fp8type), M, N, QB, _hip.stream(x1.device)), "fp8_add_Ifp_Ifp_Ofp_Opt")
-    qy2, s_y2_max, _ = _division(y1, fp8type, s_max.to(torch.bfloat16), True, False, "fp8_add_Ifp_Ifp_Ofp_Opt",
-                                 stochastic)
+    qy2, s_y2_max, _ = _division(y1, fp8type, s_max, True, False, "fp8_add_Ifp_Ifp_Ofp_Opt", stochastic,
+                                 max_as=torch.bfloat16)
     return restore(y1, batch), (restore(qy2, batch), s_y2_max, restore(s_y2, batch))

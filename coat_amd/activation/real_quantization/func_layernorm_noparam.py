@@ -20,7 +20,7 @@ def _forward(x, s_x, w, b, QB, eps, transpose_output_2d, who):
         _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.ptr(b),
         -1 if w is None else _hip.dt(w), _hip.ptr(y), _hip.ptr(s_row), _hip.ptr(mean), _hip.ptr(rstd), _hip.ptr(s_max),
         M, N, QB, float(eps), _hip.stream(x.device)), who)
-    qy, s_y_max, qy_t = _division(y, x.dtype, s_max.to(torch.bfloat16), True, True, who)
+    qy, s_y_max, qy_t = _division(y, x.dtype, s_max, True, True, who, max_as=torch.bfloat16)
     if batch is not None and not transpose_output_2d:
         qy_t = qy_t.reshape(batch, -1, N)
     return restore(qy, batch), s_y_max, qy_t, mean, rstd

@@ -22,7 +22,7 @@ def fp8_rmsnorm_forward(x, s_x, w, QB, eps, transpose_output_2d=False):
     _hip.check(_hip.lib().coat_fp8_rmsnorm_forward(
         _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.dt(w), _hip.ptr(y), _hip.ptr(s_row),
         _hip.ptr(rstd), _hip.ptr(s_max), M, N, QB, float(eps), _hip.stream(x.device)), "fp8_rmsnorm_forward")
-    qy, s_y_max, qy_t = _division(y, x.dtype, s_max.to(torch.bfloat16), True, True, "fp8_rmsnorm_forward")
+    qy, s_y_max, qy_t = _division(y, x.dtype, s_max, True, True, "fp8_rmsnorm_forward", max_as=torch.bfloat16)
     if batch is not None and not transpose_output_2d:
         qy_t = qy_t.reshape(batch, -1, N)
     num_warps = 8  # kept in the tuple for signature compatibility; the HIP kernels do not use it

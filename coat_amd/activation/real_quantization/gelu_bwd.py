@@ -18,5 +18,5 @@ def fp8_gelu_backward(x, s_x, g, QB, fp8type):
     _hip.check(_hip.lib().coat_fp8_gelu_backward(
         _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(g), _hip.ptr(y), None, _hip.ptr(s_max),
         _hip.fp8(fp8type), M, N, QB, _hip.stream(x.device)), "fp8_gelu_backward")
-    qy, s_y_max, _ = _division(y, fp8type, s_max.to(torch.bfloat16), True, False, "fp8_gelu_backward")
+    qy, s_y_max, _ = _division(y, fp8type, s_max, True, False, "fp8_gelu_backward", max_as=torch.bfloat16)
     return restore(qy, batch), s_y_max

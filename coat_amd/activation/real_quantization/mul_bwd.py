@@ -32,5 +32,5 @@ def fp8_mul_backward(x1, s_x1, x2, s_x2, g, QB, fp8type, stochastic=False, outpu
         _hip.stream(x1.device)), "fp8_mul_backward")
     if want_pg:
         return restore(y1, batch), (restore(y2, batch), restore(s_y2, batch))
-    qy2, s_y2_max, qy2_t = _division(y2, fp8type, s_max.to(torch.bfloat16), True, True, "fp8_mul_backward")
+    qy2, s_y2_max, qy2_t = _division(y2, fp8type, s_max, True, True, "fp8_mul_backward", max_as=torch.bfloat16)
     return restore(y1, batch), (restore(qy2, batch), s_y2_max, qy2_t)

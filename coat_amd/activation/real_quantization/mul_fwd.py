@@ -22,7 +22,7 @@ def fp8_mul_forward(x1, s_x1, x2, s_x2, QB, transpose_output_2d=False):
     _hip.check(_hip.lib().coat_fp8_mul_forward(
         _hip.ptr(x1), _hip.ptr(s_x1), _hip.ptr(x2), _hip.ptr(s_x2), _hip.fp8(x1.dtype), _hip.dt(s_x1), _hip.ptr(y),
         None, _hip.ptr(s_max), M, N, QB, _hip.stream(x1.device)), "fp8_mul_forward")
-    qy, s_y_max, qy_t = _division(y, x2.dtype, s_max.to(s_x1.dtype), True, True, "fp8_mul_forward")
+    qy, s_y_max, qy_t = _division(y, x2.dtype, s_max, True, True, "fp8_mul_forward", max_as=s_x1.dtype)
     if batch is not None and not transpose_output_2d:
         qy_t = qy_t.reshape(batch, -1, qy.shape[-1])
     return restore(qy, batch), s_y_max, qy_t

@@ -23,5 +23,5 @@ def fp8_silu_backward(x, s_x, g, QB, fp8type, stochastic=False, output_quantized
         _hip.ptr(s_max), _hip.fp8(fp8type), M, N, QB, _hip.stream(x.device)), "fp8_silu_backward")
     if want_pg:
         return restore(y, batch), restore(s_y, batch)
-    qy, s_y_max, qy_t = _division(y, fp8type, s_max.to(torch.bfloat16), True, True, "fp8_silu_backward")
+    qy, s_y_max, qy_t = _division(y, fp8type, s_max, True, True, "fp8_silu_backward", max_as=torch.bfloat16)
     return restore(qy, batch), s_y_max, qy_t

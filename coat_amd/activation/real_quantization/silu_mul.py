@@ -48,7 +48,7 @@ def fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, QB, transpose_output_2d=Fal
         _hip.ptr(gate_x), _hip.ptr(gate_s), _hip.ptr(up_x), _hip.ptr(up_s), _hip.fp8(gate_x.dtype), _hip.dt(gate_s),
         _hip.ptr(silu_x), _hip.ptr(silu_s), _hip.ptr(y), _hip.ptr(s_max), M, N, QB, in_pitch, s_pitch,
         _hip.stream(gate_x.device)), "fp8_silu_mul_forward")
-    mul_x, mul_s, mul_x_t = _division(y, up_x.dtype, s_max.to(torch.bfloat16), True, True, "fp8_silu_mul_forward")
+    mul_x, mul_s, mul_x_t = _division(y, up_x.dtype, s_max, True, True, "fp8_silu_mul_forward", max_as=torch.bfloat16)
     if batch is not None and not transpose_output_2d:
         mul_x_t = mul_x_t.reshape(batch, -1, N)
     return restore(silu_x, batch), restore(silu_s, batch), restore(mul_x, batch), mul_s, mul_x_t
@@ -69,7 +69,8 @@ def _silu_mul_backward_values(gate_x, gate_s, up_x, up_s, silu_x, silu_s, g, QB,
         y_up, y_gate, y_pitch = both[:, :N], both[:, N:], 2 * N
     else:
         y_gate, y_up, y_pitch = torch.empty_like(g), torch.empty_like(g), 0
-    m_gate, m_up = new_max(g.device), new_max(g.device)
+    m_gate = new_max(g.device)
+    m_up = m_gate if joined else new_max(g.device)  # joined: one maximum over both halves
     _hip.check(_hip.lib().coat_fp8_silu_mul_backward(
         _hip.ptr(gate_x), _hip.ptr(gate_s), _hip.ptr(up_x), _hip.ptr(up_s), _hip.ptr(silu_x), _hip.ptr(silu_s),
         _hip.fp8(gate_x.dtype), _hip.dt(gate_s), _hip.ptr(g), _hip.ptr(y_gate), _hip.ptr(m_gate), _hip.ptr(y_up),
@@ -86,8 +87,8 @@ def fp8_silu_mul_backward(gate_x, gate_s, up_x, up_s, silu_x, silu_s, g, QB, fp8
     fp8type = as_fp8_dtype(fp8type)
     y_gate, y_up, m_gate, m_up, batch, _ = _silu_mul_backward_values(gate_x, gate_s, up_x, up_s, silu_x, silu_s, g, QB,
                                                                      fp8type, False)
-    gq, gs, gq_t = _division(y_gate, fp8type, m_gate.to(torch.bfloat16), True, True, "fp8_silu_mul_backward")
-    uq, us, uq_t = _division(y_up, fp8type, m_up.to(torch.bfloat16), True, True, "fp8_silu_mul_backward")
+    gq, gs, gq_t = _division(y_gate, fp8type, m_gate, True, True, "fp8_silu_mul_backward", max_as=torch.bfloat16)
+    uq, us, uq_t = _division(y_up, fp8type, m_up, True, True, "fp8_silu_mul_backward", max_as=torch.bfloat16)
     return (restore(gq, batch), gs, gq_t), (restore(uq, batch), us, uq_t)
 
 
@@ -101,6 +102,6 @@ def fp8_silu_mul_backward_joined(gate_x, gate_s, up_x, up_s, silu_x, silu_s, g, 
     fp8type = as_fp8_dtype(fp8type)
     _, _, m_gate, m_up, batch, both = _silu_mul_backward_values(gate_x, gate_s, up_x, up_s, silu_x, silu_s, g, QB,
                                                                 fp8type, True)
-    s = torch.maximum(m_up, m_gate).to(torch.bfloat16)  # rounding is monotone: the max of the bf16 group scales
-    q, s, q_t = _division(both, fp8type, s, True, True, "fp8_silu_mul_backward_joined")
+    # rounding is monotone: the rounded maximum is the maximum of the bf16 group scales
+    q, s, q_t = _division(both, fp8type, m_gate, True, True, "fp8_silu_mul_backward_joined", max_as=torch.bfloat16)
     return restore(q, batch), s, q_t

@@ -158,16 +158,27 @@ __global__ __launch_bounds__(256) void k_absmax(const void* __restrict__ x, floa
     block_atomic_max_nonneg(amax, m, smem_max);
 }
 
+// The per-tensor scale of a division kernel.  s_out == NULL: *s_ptr is the scale, an element of dtype SDT.  Otherwise
+// *s_ptr is the fp32 maximum of the group scales left by the producer kernel's atomics: it is rounded to SDT here (what
+// the reference's ``s.max()`` over the stored scales gives, rounding being monotone) and the first thread of the grid
+// stores the rounded value to s_out for the consumers, which saves a separate conversion launch per tensor.
+template <int SDT> __device__ __forceinline__ float load_scale_or_max(const void* s_ptr, void* s_out) {
+    if (!s_out) return load_as_f32<SDT>(s_ptr, 0);
+    const float s = round_to<SDT>(((const float*)s_ptr)[0]);
+    if (blockIdx.x == 0 && threadIdx.x == 0) store_from_f32<SDT>(s_out, 0, s);
+    return s;
+}
+
 // ------------------------------------------------------------------------------------------------
 // K4: per-tensor division over the flat array, q = fp8(x / float(*s)).  SR: stochastic rounding with the
 // Philox key (k0, k1) (the reference's branch, coat/activation/real_quantization/_division.py:96-112).
 template <int XDT, int SDT, int KIND, int UNROLL, bool SR>
 __global__ __launch_bounds__(256) void k_division(const void* __restrict__ x, const void* __restrict__ s_ptr,
                                                    void* __restrict__ q, int64_t nvec, int64_t numel, uint32_t k0,
-                                                   uint32_t k1) {
+                                                   uint32_t k1, void* __restrict__ s_out) {
     constexpr int VEC = VecOf<XDT>::kVec;
     enable_fp8_saturation();
-    const float s = load_as_f32<SDT>(s_ptr, 0);
+    const float s = load_scale_or_max<SDT>(s_ptr, s_out);
     const float r = 1.0f / s;
     const bool fast = s >= kMinFastDivScale && s < 0x1p100f;  // uniform across the grid
     const int64_t base = ((int64_t)blockIdx.x * UNROLL) * 256 + threadIdx.x;
@@ -275,7 +286,7 @@ __device__ __forceinline__ void store_tile_transposed(const uint32_t* tile, void
 template <int XDT, int SDT, int KIND, bool RAW, bool WRITE_Q, int TM, bool SR>
 __global__ __launch_bounds__(256) void k_division_transpose(const void* __restrict__ x, const void* __restrict__ s_ptr,
                                                              void* __restrict__ q, void* __restrict__ qt, int64_t M,
-                                                             int64_t N, uint32_t k0, uint32_t k1) {
+                                                             int64_t N, uint32_t k0, uint32_t k1, void* __restrict__ s_out) {
     __shared__ uint32_t tile[TM * kPitchDw];
     enable_fp8_saturation();
     const int64_t tiles_n = (N + kTileN - 1) / kTileN;
@@ -283,7 +294,7 @@ __global__ __launch_bounds__(256) void k_division_transpose(const void* __restri
     float s = 1.0f, r = 1.0f;
     bool fast = true;
     if (!RAW) {
-        s = load_as_f32<SDT>(s_ptr, 0);
+        s = load_scale_or_max<SDT>(s_ptr, s_out);
         r = 1.0f / s;
         fast = s >= kMinFastDivScale && s < 0x1p100f;
     }
@@ -614,7 +625,7 @@ extern "C" int coat_absmax(const void* x, int x_dtype, float* amax, int64_t nume
 
 template <bool SR>
 static int division_launch(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M, int64_t N,
-                           int fp8, uint64_t seed, void* stream) {
+                           int fp8, uint64_t seed, void* stream, void* s_out = nullptr) {
     if (M < 0 || N < 0) return COAT_EINVAL;
     if (M * N == 0) return COAT_OK;
     if (!x || !s || (!q && !qt)) return COAT_EINVAL;
@@ -627,7 +638,7 @@ static int division_launch(const void* x, int x_dtype, const void* s, int s_dtyp
             int64_t numel = M * N, nvec = numel / VEC;
             int64_t blocks = (nvec + 256 * 4 - 1) / (256 * 4);
             if (blocks == 0) blocks = 1;
-            hipLaunchKernelGGL((k_division<XDT, SDT, KIND, 4, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, nvec, numel, k0, k1);
+            hipLaunchKernelGGL((k_division<XDT, SDT, KIND, 4, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, nvec, numel, k0, k1, s_out);
             return coat_launch_status();
         })));
         return COAT_EINVAL;
@@ -637,12 +648,12 @@ static int division_launch(const void* x, int x_dtype, const void* s, int s_dtyp
     int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
     if (q) {
         DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
-            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, true, TM, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N, k0, k1);
+            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, true, TM, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N, k0, k1, s_out);
             return coat_launch_status();
         })));
     } else {
         DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {
-            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, false, TM, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N, k0, k1);
+            hipLaunchKernelGGL((k_division_transpose<XDT, SDT, KIND, false, false, TM, SR>), dim3((unsigned)blocks), dim3(256), 0, st, x, s, q, qt, M, N, k0, k1, s_out);
             return coat_launch_status();
         })));
     }
@@ -652,6 +663,12 @@ static int division_launch(const void* x, int x_dtype, const void* s, int s_dtyp
 extern "C" int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
                                  int64_t N, int fp8, void* stream) {
     return division_launch<false>(x, x_dtype, s, s_dtype, q, qt, M, N, fp8, 0, stream);
+}
+
+extern "C" int coat_fp8_division_from_max(const void* x, int x_dtype, const float* s_max, void* s_out, int s_dtype, void* q,
+                                          void* qt, int64_t M, int64_t N, int fp8, void* stream) {
+    if ((M > 0 && N > 0) && !s_out) return COAT_EINVAL;
+    return division_launch<false>(x, x_dtype, s_max, s_dtype, q, qt, M, N, fp8, 0, stream, s_out);
 }
 
 extern "C" int coat_fp8_division_stochastic(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt,
@@ -670,7 +687,7 @@ extern "C" int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, 
     constexpr int TM = 128;
     int64_t blocks = ((M + TM - 1) / TM) * ((N + kTileN - 1) / kTileN);
     hipLaunchKernelGGL((k_division_transpose<kBF16, kBF16, kE4M3, true, false, TM, false>), dim3((unsigned)blocks), dim3(256), 0,
-                       (hipStream_t)stream, x, nullptr, nullptr, y, M, N, 0u, 0u);
+                       (hipStream_t)stream, x, nullptr, nullptr, y, M, N, 0u, 0u, nullptr);
     return coat_launch_status();
 }
 

@@ -66,6 +66,13 @@ int coat_absmax(const void* x, int x_dtype, float* amax, int64_t numel, void* st
 int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
                       int64_t N, int fp8, void* stream);
 
+/* The same division fed with the producer kernel's fp32 maximum of the group scales (the word that
+ * coat_fp8_group_scales and the fused kernels merge their atomics into): the kernel rounds *s_max to s_dtype, divides by
+ * that value and stores it to s_out (one element of s_dtype) for the consumers.  Replaces "convert the maximum to bf16 on
+ * the host side, then divide" (the reference's s_y.max() at rq/_quantize_pertensor.py:139 and the like) by one launch. */
+int coat_fp8_division_from_max(const void* x, int x_dtype, const float* s_max, void* s_out, int s_dtype, void* q, void* qt,
+                               int64_t M, int64_t N, int fp8, void* stream);
+
 /* The same two entry points with stochastic=True (rq/_division.py:96-112 and :130-150 _stochastic_rounding;
  * rq/_division_transpose.py:103-119): the quotient of element i (linear index in x) is moved up by
  * noise_i * (one FP8 step of its binade), clamped to the binade, then rounded to nearest.  noise_i is Triton's

@@ -192,3 +192,26 @@ def test_default_division_scale_is_the_device_expression(dev, dtype):
             ws = R.absmax_scale(x, fp8)
             assert s.dtype == dtype and torch.equal(s.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
                                                     ws.view(torch.int16 if dtype != torch.float32 else torch.int32))
+
+
+@pytest.mark.parametrize("sdtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(64, 128), (7, 37)])
+def test_division_from_fp32_max_equals_division_by_rounded_scale(dev, sdtype, shape):
+    """coat_fp8_division_from_max rounds the fp32 maximum to the scale dtype, divides by that value and stores it."""
+    from coat_amd import _hip
+    M, N = shape
+    x = make_x(M, N, 11, torch.bfloat16).to(dev)
+    for m in (0.0123456789, 3.1e-7, 1.0):
+        s_max = torch.tensor(m, dtype=torch.float32, device=dev)
+        want_s = s_max.to(sdtype)
+        tr = M % 16 == 0 and N % 16 == 0
+        q, qt = torch.empty((M, N), dtype=torch.uint8, device=dev), torch.empty((N, M), dtype=torch.uint8, device=dev)
+        wq, wqt = torch.empty_like(q), torch.empty_like(qt)
+        s_out = torch.zeros((), dtype=sdtype, device=dev)
+        _hip.check(_hip.lib().coat_fp8_division_from_max(
+            _hip.ptr(x), _hip.dt(x), _hip.ptr(s_max), _hip.ptr(s_out), _hip.dt(s_out), _hip.ptr(q),
+            _hip.ptr(qt) if tr else None, M, N, 0, _hip.stream(x.device)), "from_max")
+        _hip.check(_hip.lib().coat_fp8_division(
+            _hip.ptr(x), _hip.dt(x), _hip.ptr(want_s), _hip.dt(want_s), _hip.ptr(wq), _hip.ptr(wqt) if tr else None,
+            M, N, 0, _hip.stream(x.device)), "division")
+        assert s_out.item() == want_s.item() and torch.equal(q, wq) and (not tr or torch.equal(qt, wqt))
