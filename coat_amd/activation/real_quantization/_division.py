@@ -48,6 +48,35 @@ def _division(x, fp8type, s_y, want_q, want_qt, what, stochastic=False, max_as=N
     return y, s_y, y_t
 
 
+def _outputs_for(x, fp8type):
+    M, N = x.shape
+    return (torch.empty((M, N), dtype=fp8type, device=x.device), torch.empty((N, M), dtype=fp8type, device=x.device),
+            torch.empty((), dtype=torch.bfloat16, device=x.device))
+
+
+def _rmsnorm_division(x, s_x, w, rstd, s_max, QB, what):
+    """(q, s, q_t) of bf16(x * rstd * w) divided by the bf16-rounded ``s_max``, with the tensor recomputed tile by tile
+    from the norm's inputs instead of being stored and read back (same codes as ``_division`` on the stored tensor)."""
+    M, N = x.shape
+    q, q_t, s_out = _outputs_for(x, x.dtype)
+    _hip.check(_hip.lib().coat_fp8_rmsnorm_division(
+        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd),
+        _hip.ptr(s_max), _hip.ptr(s_out), _hip.ptr(q), _hip.ptr(q_t), M, N, QB, _hip.stream(x.device)), what)
+    return q, s_out, q_t
+
+
+def _product_division(a, s_a, b, s_b, b_pitch, sb_pitch, s_max, QB, what):
+    """(q, s, q_t) of bf16(dequant(a) * dequant(b)) divided by the bf16-rounded ``s_max``, recomputed from the factors.
+    ``b`` may be a column slice (row pitches in codes / scales, 0 = dense)."""
+    M, N = a.shape
+    q, q_t, s_out = _outputs_for(a, a.dtype)
+    _hip.check(_hip.lib().coat_fp8_product_division(
+        _hip.ptr(a), _hip.ptr(s_a), _hip.dt(s_a), _hip.ptr(b), _hip.ptr(s_b), _hip.dt(s_b), _hip.fp8(a.dtype),
+        _hip.ptr(s_max), _hip.ptr(s_out), _hip.ptr(q), _hip.ptr(q_t), M, N, QB, b_pitch, sb_pitch,
+        _hip.stream(a.device)), what)
+    return q, s_out, q_t
+
+
 def fp8_division(x, QB, fp8type, s_y=None, stochastic=False):
     """x -> (y fp8, s_y); y = fp8(x / float(s_y)); s_y defaults to (absmax + 1e-10) / fp8max.
     stochastic: the reference's noise-then-round branch (reference :96-112, :130-150), same Philox stream."""

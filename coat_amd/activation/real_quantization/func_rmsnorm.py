@@ -3,7 +3,7 @@ Reference: coat/activation/real_quantization/func_rmsnorm.py:223-335."""
 import torch
 
 from ... import _hip
-from ._division import _division
+from ._division import _division, _rmsnorm_division
 from ._fused import new_max, prep_bf16, prep_pg
 from .common import restore
 
@@ -15,14 +15,20 @@ def fp8_rmsnorm_forward(x, s_x, w, QB, eps, transpose_output_2d=False):
     x, s_x, batch = prep_pg(x, s_x)
     M, N = x.shape
     w = _hip.dense(w)
-    y = torch.empty_like(x, dtype=torch.bfloat16)
+    # the division recomputes y from x, rstd and w tile by tile, so y is not stored (needs whole 16 x 16 blocks,
+    # which the transposed output needs anyway)
+    recompute = M % 16 == 0 and M > 0
+    y = None if recompute else torch.empty_like(x, dtype=torch.bfloat16)
     s_row = torch.empty((M,), dtype=torch.bfloat16, device=x.device)
     rstd = torch.empty((M,), dtype=torch.float32, device=x.device)
     s_max = new_max(x.device)
     _hip.check(_hip.lib().coat_fp8_rmsnorm_forward(
         _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.dt(w), _hip.ptr(y), _hip.ptr(s_row),
         _hip.ptr(rstd), _hip.ptr(s_max), M, N, QB, float(eps), _hip.stream(x.device)), "fp8_rmsnorm_forward")
-    qy, s_y_max, qy_t = _division(y, x.dtype, s_max, True, True, "fp8_rmsnorm_forward", max_as=torch.bfloat16)
+    if recompute:
+        qy, s_y_max, qy_t = _rmsnorm_division(x, s_x, w, rstd, s_max, QB, "fp8_rmsnorm_forward")
+    else:
+        qy, s_y_max, qy_t = _division(y, x.dtype, s_max, True, True, "fp8_rmsnorm_forward", max_as=torch.bfloat16)
     if batch is not None and not transpose_output_2d:
         qy_t = qy_t.reshape(batch, -1, N)
     num_warps = 8  # kept in the tuple for signature compatibility; the HIP kernels do not use it

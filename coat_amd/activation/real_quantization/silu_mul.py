@@ -5,7 +5,7 @@ gradient."""
 import torch
 
 from ... import _hip
-from ._division import _division
+from ._division import _division, _product_division
 from ._fused import new_max, prep_bf16, prep_pg
 from .common import as_fp8_dtype, restore
 
@@ -42,13 +42,19 @@ def fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, QB, transpose_output_2d=Fal
     M, N = gate_x.shape
     silu_x = torch.empty((M, N), dtype=gate_x.dtype, device=gate_x.device)
     silu_s = torch.empty(gate_s.shape, dtype=torch.bfloat16, device=gate_x.device)
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=gate_x.device)
+    # the division recomputes the product from the SiLU codes just written and from up, so the bf16 product is not stored
+    recompute = M % 16 == 0 and M > 0 and N > 0
+    y = None if recompute else torch.empty((M, N), dtype=torch.bfloat16, device=gate_x.device)
     s_max = new_max(gate_x.device)
     _hip.check(_hip.lib().coat_fp8_silu_mul_forward(
         _hip.ptr(gate_x), _hip.ptr(gate_s), _hip.ptr(up_x), _hip.ptr(up_s), _hip.fp8(gate_x.dtype), _hip.dt(gate_s),
         _hip.ptr(silu_x), _hip.ptr(silu_s), _hip.ptr(y), _hip.ptr(s_max), M, N, QB, in_pitch, s_pitch,
         _hip.stream(gate_x.device)), "fp8_silu_mul_forward")
-    mul_x, mul_s, mul_x_t = _division(y, up_x.dtype, s_max, True, True, "fp8_silu_mul_forward", max_as=torch.bfloat16)
+    if recompute:
+        mul_x, mul_s, mul_x_t = _product_division(silu_x, silu_s, up_x, up_s, in_pitch, s_pitch, s_max, QB,
+                                                  "fp8_silu_mul_forward")
+    else:
+        mul_x, mul_s, mul_x_t = _division(y, up_x.dtype, s_max, True, True, "fp8_silu_mul_forward", max_as=torch.bfloat16)
     if batch is not None and not transpose_output_2d:
         mul_x_t = mul_x_t.reshape(batch, -1, N)
     return restore(silu_x, batch), restore(silu_s, batch), restore(mul_x, batch), mul_s, mul_x_t

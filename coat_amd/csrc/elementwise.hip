@@ -237,7 +237,7 @@ __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
             dequant_words<KIND_IN>(w, round_bf16(s), d);
 #pragma unroll
             for (int i = 0; i < 16; i++) v[i] = d[i] * b[i];
-            if (ok) store_bf16x16(A.y, c, v);
+            if (ok && A.y) store_bf16x16(A.y, c, v);  // NULL: maximum only (the division recomputes the product)
             const float s2 = group_scale<KIND_IN>(cluster_max_rt(amax16(v), lpg));
             tmax = fmaxf(tmax, ok ? s2 : 0.0f);
         } else {
@@ -415,7 +415,7 @@ static int silu_mul_launch(SiluMulArgs& A, bool bwd, int fp8_in, int fp8_out, in
 extern "C" int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
                                          int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M,
                                          int64_t N, int QB, int64_t in_pitch, int64_t s_pitch, void* stream) {
-    if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !q_silu || !s_silu || !y || !s_max)) return COAT_EINVAL;
+    if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !q_silu || !s_silu || !s_max)) return COAT_EINVAL;  // y may be NULL
     SiluMulArgs A = {gate, s_gate, up, s_up, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr, 0, 0, 0};
     return silu_mul_launch(A, false, fp8, fp8, M, N, QB, s_dtype, in_pitch, s_pitch, 0, (hipStream_t)stream);
 }

@@ -9,6 +9,7 @@
 //     with neighbouring lanes writing neighbouring chunks of one output row.
 #include "coat_device.h"
 #include "coat_host.h"
+#include "norm_common.h"
 
 namespace coat {
 
@@ -336,6 +337,119 @@ __global__ __launch_bounds__(256) void k_division_transpose(const void* __restri
                 }
                 if (WRITE_Q) *(uint4*)((uint8_t*)q + m * N + n) = make_uint4(c[0], c[1], c[2], c[3]);
             }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) tile[row * kPitchDw + c16 * 4 + k] = c[k];
+    }
+    __syncthreads();
+    store_tile_transposed<TM>(tile, qt, M, N, m0, n0);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Division + transpose of a bf16 tensor that is never stored: the tile's values are recomputed from the inputs of
+// the kernel that produced the tensor's statistics (same expressions, same roundings, so the codes equal those of
+// "write the bf16 tensor, then divide it"), which trades a bf16 write and read for a second read of FP8 inputs.
+// A source provides  struct Raw,  load(m, n, Raw&)  (16 elements of row m from column n, loads only) and
+// value(Raw, float v[16])  (the 16 values, already rounded to bf16).
+
+// bf16((x * rstd[row]) * w[col]) of k_rmsnorm_fwd (coat/activation/real_quantization/func_rmsnorm.py:92-108)
+template <int KIND, int WDT> struct RmsNormSource {
+    const uint8_t* q; const void* s; const void* w; const float* rstd;
+    int s_dt, qb; int64_t N;
+    struct Raw { uint4 codes; float sc, rstd; uint4 w[WDT == kF32 ? 4 : 2]; };
+    __device__ __forceinline__ void load(int64_t m, int64_t n, Raw& r) const {
+        r.codes = *(const uint4*)(q + m * N + n);
+        r.sc = load_rt_f32(s, m * (N / qb) + n / qb, s_dt);
+        r.rstd = rstd[m];
+        const uint4* wp = (const uint4*)((const uint8_t*)w + n * (WDT == kF32 ? 4 : 2));
+#pragma unroll
+        for (int i = 0; i < (WDT == kF32 ? 4 : 2); i++) r.w[i] = wp[i];
+    }
+    __device__ __forceinline__ void value(const Raw& r, float* v) const {
+        const uint32_t c[4] = {r.codes.x, r.codes.y, r.codes.z, r.codes.w};
+        float wv[16];
+        if constexpr (WDT == kF32) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                wv[4 * i] = u2f(r.w[i].x); wv[4 * i + 1] = u2f(r.w[i].y); wv[4 * i + 2] = u2f(r.w[i].z); wv[4 * i + 3] = u2f(r.w[i].w);
+            }
+        } else {
+            const uint32_t u[8] = {r.w[0].x, r.w[0].y, r.w[0].z, r.w[0].w, r.w[1].x, r.w[1].y, r.w[1].z, r.w[1].w};
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                wv[2 * k] = WDT == kBF16 ? bf16lo(u[k]) : f16lo(u[k]);
+                wv[2 * k + 1] = WDT == kBF16 ? bf16hi(u[k]) : f16hi(u[k]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float f[4];
+            fp8x4_to_f32<KIND>(c[k], f);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[4 * k + i] = round_to<kBF16>(((f[i] * r.sc) * r.rstd) * wv[4 * k + i]);
+        }
+    }
+};
+
+// bf16(dequant(a) * dequant(b)) of two per-group FP8 tensors: the product of k_silu_mul's forward
+// (coat/activation/real_quantization/mul_fwd.py:136-150).  a is dense [M, N]; b may be a column slice of a wider tensor
+// (row pitches in elements / scales).
+template <int KIND> struct ProductSource {
+    const uint8_t* a; const void* sa; const uint8_t* b; const void* sb;
+    int sa_dt, sb_dt, qb; int64_t N, b_pitch, sb_pitch;
+    struct Raw { uint4 ca, cb; float fa, fb; };
+    __device__ __forceinline__ void load(int64_t m, int64_t n, Raw& r) const {
+        r.ca = *(const uint4*)(a + m * N + n);
+        r.cb = *(const uint4*)(b + m * b_pitch + n);
+        r.fa = load_rt_f32(sa, m * (N / qb) + n / qb, sa_dt);
+        r.fb = load_rt_f32(sb, m * sb_pitch + n / qb, sb_dt);
+    }
+    __device__ __forceinline__ void value(const Raw& r, float* v) const {
+        const uint32_t ca[4] = {r.ca.x, r.ca.y, r.ca.z, r.ca.w}, cb[4] = {r.cb.x, r.cb.y, r.cb.z, r.cb.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float fa[4], fb[4];
+            fp8x4_to_f32<KIND>(ca[k], fa);
+            fp8x4_to_f32<KIND>(cb[k], fb);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[4 * k + i] = round_to<kBF16>((fa[i] * r.fa) * (fb[i] * r.fb));
+        }
+    }
+};
+
+// q = fp8(value / bf16(*s_max)) and its transpose; the rounded scale goes to s_out (bf16).  M % 16 == 0, N % 16 == 0.
+template <typename SRC, int KIND>
+__global__ __launch_bounds__(256) void k_produced_division_transpose(SRC src, const float* __restrict__ s_max,
+                                                                      void* __restrict__ s_out, void* __restrict__ q,
+                                                                      void* __restrict__ qt, int64_t M, int64_t N) {
+    constexpr int TM = 128;
+    __shared__ uint32_t tile[TM * kPitchDw];
+    enable_fp8_saturation();
+    const int64_t tiles_n = (N + kTileN - 1) / kTileN;
+    const int64_t m0 = (blockIdx.x / tiles_n) * TM, n0 = (blockIdx.x % tiles_n) * kTileN;
+    const float s = load_scale_or_max<kBF16>(s_max, s_out);
+    const float r = 1.0f / s;
+    const bool fast = s >= kMinFastDivScale && s < 0x1p100f;
+    constexpr int NIT = TM * (kTileN / 16) / 256;
+    typename SRC::Raw raw[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * 256;
+        const int64_t m = m0 + job / (kTileN / 16), n = n0 + (job % (kTileN / 16)) * 16;
+        if (m < M && n < N) src.load(m, n, raw[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * 256;
+        const int row = job / (kTileN / 16), c16 = job % (kTileN / 16);
+        const int64_t m = m0 + row, n = n0 + c16 * 16;
+        uint32_t c[4] = {0, 0, 0, 0};
+        if (m < M && n < N) {
+            float v[16];
+            src.value(raw[it], v);
+            if (fast) quantize_vec<KIND, 16>(v, s, r, c);
+            else quantize_vec_slow<KIND, 16>(v, s, c);
+            *(uint4*)((uint8_t*)q + m * N + n) = make_uint4(c[0], c[1], c[2], c[3]);
         }
 #pragma unroll
         for (int k = 0; k < 4; k++) tile[row * kPitchDw + c16 * 4 + k] = c[k];
@@ -676,6 +790,64 @@ extern "C" int coat_fp8_division_stochastic(const void* x, int x_dtype, const vo
     // the noise counter is the 32-bit linear element index, as in the reference's int32 offset arithmetic
     if (M > 0 && N > 0 && M * N > ((int64_t)1 << 32)) return COAT_ESHAPE;
     return division_launch<true>(x, x_dtype, s, s_dtype, q, qt, M, N, fp8, seed, stream);
+}
+
+// The division (+ transpose) that follows coat_fp8_rmsnorm_forward, fed with that kernel's inputs instead of its bf16
+// output (which the caller then need not store: y = NULL there).
+extern "C" int coat_fp8_rmsnorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype,
+                                         const float* rstd, const float* s_max, void* s_out, void* q, void* qt, int64_t M,
+                                         int64_t N, int QB, void* stream) {
+    if (int e = check_mn(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (M % 16 != 0 || N % 16 != 0 || QB % 16 != 0) return COAT_ESHAPE;
+    if (!x || !s_x || !w || !rstd || !s_max || !s_out || !q || !qt) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(q) || !coat_aligned16(qt)) return COAT_EALIGN;
+    if (s_dtype < 0 || s_dtype > 2) return COAT_EDTYPE;
+    const int64_t blocks = ((M + 127) / 128) * ((N + kTileN - 1) / kTileN);
+    if (blocks >= ((int64_t)1 << 31)) return COAT_ESHAPE;
+    hipStream_t st = (hipStream_t)stream;
+#define RMS_DIV(KINDV, WDTV)                                                                                        \
+    {                                                                                                               \
+        RmsNormSource<KINDV, WDTV> src{(const uint8_t*)x, s_x, w, rstd, s_dtype, QB, N};                             \
+        hipLaunchKernelGGL((k_produced_division_transpose<RmsNormSource<KINDV, WDTV>, KINDV>), dim3((unsigned)blocks), \
+                           dim3(256), 0, st, src, s_max, s_out, q, qt, M, N);                                       \
+        return coat_launch_status();                                                                                \
+    }
+    DISPATCH_KIND(fp8, {
+        if (w_dtype == COAT_BF16) RMS_DIV(KIND, kBF16)
+        if (w_dtype == COAT_F32) RMS_DIV(KIND, kF32)
+        if (w_dtype == COAT_F16) RMS_DIV(KIND, kF16)
+        return COAT_EDTYPE;
+    });
+#undef RMS_DIV
+    return COAT_EINVAL;
+}
+
+// The division (+ transpose) of the product of two per-group FP8 tensors (what coat_fp8_silu_mul_forward and
+// coat_fp8_mul_forward leave in their bf16 output), recomputed from the two factors.  a [M, N] dense with scales
+// [M, N / QB]; b with row pitch b_pitch codes and sb_pitch scales (0 = dense).
+extern "C" int coat_fp8_product_division(const void* a, const void* s_a, int sa_dtype, const void* b, const void* s_b,
+                                         int sb_dtype, int fp8, const float* s_max, void* s_out, void* q, void* qt,
+                                         int64_t M, int64_t N, int QB, int64_t b_pitch, int64_t sb_pitch, void* stream) {
+    if (int e = check_mn(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (M % 16 != 0 || N % 16 != 0 || QB % 16 != 0) return COAT_ESHAPE;
+    if (!a || !s_a || !b || !s_b || !s_max || !s_out || !q || !qt) return COAT_EINVAL;
+    if (b_pitch == 0) b_pitch = N;
+    if (sb_pitch == 0) sb_pitch = N / QB;
+    if (b_pitch < N || b_pitch % 16 != 0 || sb_pitch < N / QB) return COAT_ESHAPE;
+    if (!coat_aligned16(a) || !coat_aligned16(b) || !coat_aligned16(q) || !coat_aligned16(qt)) return COAT_EALIGN;
+    if (sa_dtype < 0 || sa_dtype > 2 || sb_dtype < 0 || sb_dtype > 2) return COAT_EDTYPE;
+    const int64_t blocks = ((M + 127) / 128) * ((N + kTileN - 1) / kTileN);
+    if (blocks >= ((int64_t)1 << 31)) return COAT_ESHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_KIND(fp8, {
+        ProductSource<KIND> src{(const uint8_t*)a, s_a, (const uint8_t*)b, s_b, sa_dtype, sb_dtype, QB, N, b_pitch, sb_pitch};
+        hipLaunchKernelGGL((k_produced_division_transpose<ProductSource<KIND>, KIND>), dim3((unsigned)blocks), dim3(256), 0,
+                           st, src, s_max, s_out, q, qt, M, N);
+        return coat_launch_status();
+    });
+    return COAT_EINVAL;
 }
 
 extern "C" int coat_fp8_transpose(const void* x, void* y, int64_t M, int64_t N, void* stream) {

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__
                 yv[i] = (x[it][i] * rstd) * wv[i];
                 amax = fmaxf(amax, fabsf(yv[i]));
             }
-            store_bf16_16(y, row_off + col, yv);
+            if (y) store_bf16_16(y, row_off + col, yv);  // NULL: statistics only (the division recomputes y)
         }
     }
     amax = block_max_256(amax, smem);
@@ -171,7 +171,7 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
                                         float eps, void* stream) {
     if (int e = rms_check(M, N, QB)) return e;
     if (M * N == 0) return COAT_OK;
-    if (!x || !s_x || !w || !y || !s_row || !rstd || !s_max) return COAT_EINVAL;
+    if (!x || !s_x || !w || !s_row || !rstd || !s_max) return COAT_EINVAL;  // y may be NULL
     if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(y)) return COAT_EALIGN;
     hipStream_t st = (hipStream_t)stream;
     RMS_DISPATCH(k_rmsnorm_fwd, M, (const uint8_t*)x, s_x, s_dtype, w, y, s_row, rstd, s_max, (int)N, QB, eps)

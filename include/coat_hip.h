@@ -125,7 +125,8 @@ int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s_y, float* 
  * (forward: rq/silu_fwd.py:152 then rq/mul_fwd.py:191) and round-trip the bf16 gradient of the product (backward:
  * rq/mul_bwd.py:221 then rq/silu_bwd.py:170).  No single counterpart in the reference; used by the MLP module.
  * forward: q_silu / s_silu = per-group FP8 SiLU(gate) with bf16 scales (saved for backward), y = bf16 product of the
- * dequantized SiLU and up, *s_max = max of the product's fp32 group scales (fp8 = format of gate / up / silu). */
+ * dequantized SiLU and up (may be NULL: the maximum alone, for coat_fp8_product_division), *s_max = max of the product's
+ * fp32 group scales (fp8 = format of gate / up / silu). */
 int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
                               int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M, int64_t N,
                               int QB, int64_t in_pitch, int64_t s_pitch, void* stream);
@@ -140,10 +141,26 @@ int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, const void*
                                int QB, int64_t in_pitch, int64_t s_pitch, int64_t y_pitch, void* stream);
 
 /* rq/func_rmsnorm.py:223 fp8_rmsnorm_forward (kernel :54-111): y = bf16(x * rstd * w); s_row [M] bf16 row scales
- * (max|y| + 1e-10) / fp8max; rstd [M] fp32; s_max as above.  N <= 16384, N % 16 == 0. */
+ * (max|y| + 1e-10) / fp8max; rstd [M] fp32; s_max as above.  N <= 16384, N % 16 == 0.  y may be NULL (statistics
+ * only, for coat_fp8_rmsnorm_division). */
 int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype, void* y,
                              void* s_row, float* rstd, float* s_max, int64_t M, int64_t N, int QB, float eps,
                              void* stream);
+/* The per-tensor division + transpose that ends rq/func_rmsnorm.py:223 (its fp8_division_transpose call at :269),
+ * fed with the norm's inputs: every tile of y = bf16(x * rstd * w) is recomputed in registers with the forward kernel's
+ * expressions, so q / qt equal those of coat_fp8_division_from_max on the stored y, and y is never written or read.
+ * s_max: the fp32 maximum left by coat_fp8_rmsnorm_forward; s_out: one bf16 element, the rounded scale.
+ * M % 16 == 0, N % 16 == 0, QB % 16 == 0; q / qt in the format of x. */
+int coat_fp8_rmsnorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype,
+                              const float* rstd, const float* s_max, void* s_out, void* q, void* qt, int64_t M, int64_t N,
+                              int QB, void* stream);
+/* The same for the product of two per-group FP8 tensors, y = bf16(dequant(a) * dequant(b)) (kernel rq/mul_fwd.py:136-150;
+ * the division is its fp8_division_transpose call at :243): a [M, N] dense (the SiLU output that
+ * coat_fp8_silu_mul_forward just wrote, or x1 of fp8_mul_forward), b with row pitches b_pitch codes / sb_pitch scales
+ * (0 = dense). */
+int coat_fp8_product_division(const void* a, const void* s_a, int sa_dtype, const void* b, const void* s_b, int sb_dtype,
+                              int fp8, const float* s_max, void* s_out, void* q, void* qt, int64_t M, int64_t N, int QB,
+                              int64_t b_pitch, int64_t sb_pitch, void* stream);
 /* rq/func_rmsnorm.py:281 fp8_rmsnorm_backward (kernels :121-196, :200-220): dx bf16 [M,N], dw [N] in w's dtype.
  * dw_partial: caller-provided fp32 workspace [n_partial, N]; the kernel uses min(n_partial, M) blocks and sums their
  * partial rows in block order (deterministic, unlike the reference's lock-ordered accumulation).

@@ -269,3 +269,76 @@ def test_larger_groups_and_float32_scales(dev):
     qy, s, qyt = rq.fp8_mul_forward(q1.to(dev), s1.to(dev), q2.to(dev), s2.to(dev), 64)
     wq, ws, wqt = R.fp8_mul_forward(q1, s1, q2, s2, 64)
     assert s.item() == ws.item() and torch.equal(b(qy), b(wq)) and torch.equal(b(qyt), b(wqt))
+
+
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("shape,QBv", [((48, 176), 16), ((256, 4096), 32), ((144, 8192 + 64), 16)])
+def test_rmsnorm_division_recomputed_equals_division_of_the_stored_tensor(dev, wdtype, shape, QBv):
+    """coat_fp8_rmsnorm_division recomputes y from the norm's inputs: same codes, transpose and scale as dividing the
+    bf16 tensor that coat_fp8_rmsnorm_forward stores."""
+    from coat_amd import _hip
+    M, N = shape
+    x = rand(41, 1.0, shape)
+    q, s = R.fp8_quantize(x, QBv, "E4M3")
+    q, s = q.to(dev), s.to(dev)
+    w = (torch.ones(N) + 0.1 * torch.randn(N, generator=torch.Generator().manual_seed(5))).to(wdtype).to(dev)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    s_row = torch.empty((M,), dtype=torch.bfloat16, device=dev)
+    rstd = torch.empty((M,), dtype=torch.float32, device=dev)
+    s_max = torch.zeros((), dtype=torch.float32, device=dev)
+    lib, st = _hip.lib(), _hip.stream(q.device)
+    _hip.check(lib.coat_fp8_rmsnorm_forward(_hip.ptr(q), 0, _hip.ptr(s), _hip.dt(s), _hip.ptr(w), _hip.dt(w), _hip.ptr(y),
+                                            _hip.ptr(s_row), _hip.ptr(rstd), _hip.ptr(s_max), M, N, QBv, 1e-5, st), "fwd")
+    # statistics-only call: same rstd, row scales and maximum without the bf16 output
+    s_row2, rstd2, s_max2 = torch.empty_like(s_row), torch.empty_like(rstd), torch.zeros_like(s_max)
+    _hip.check(lib.coat_fp8_rmsnorm_forward(_hip.ptr(q), 0, _hip.ptr(s), _hip.dt(s), _hip.ptr(w), _hip.dt(w), None,
+                                            _hip.ptr(s_row2), _hip.ptr(rstd2), _hip.ptr(s_max2), M, N, QBv, 1e-5, st), "stats")
+    assert torch.equal(s_row.view(torch.int16), s_row2.view(torch.int16)) and torch.equal(rstd, rstd2)
+    assert torch.equal(s_max, s_max2)
+    outs = []
+    for fused in (False, True):
+        qy, qyt = torch.empty((M, N), dtype=torch.uint8, device=dev), torch.empty((N, M), dtype=torch.uint8, device=dev)
+        s_out = torch.zeros((), dtype=torch.bfloat16, device=dev)
+        if fused:
+            _hip.check(lib.coat_fp8_rmsnorm_division(_hip.ptr(q), 0, _hip.ptr(s), _hip.dt(s), _hip.ptr(w), _hip.dt(w),
+                                                     _hip.ptr(rstd), _hip.ptr(s_max), _hip.ptr(s_out), _hip.ptr(qy),
+                                                     _hip.ptr(qyt), M, N, QBv, st), "rmsnorm_division")
+        else:
+            _hip.check(lib.coat_fp8_division_from_max(_hip.ptr(y), _hip.dt(y), _hip.ptr(s_max), _hip.ptr(s_out),
+                                                      _hip.dt(s_out), _hip.ptr(qy), _hip.ptr(qyt), M, N, 0, st), "division")
+        outs.append((qy, qyt, s_out))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert outs[0][2].item() == outs[1][2].item() and outs[0][2].item() > 0
+    assert torch.equal(outs[1][1], outs[1][0].t().contiguous())
+
+
+@pytest.mark.parametrize("fp8", ["E4M3", "E5M2"])
+@pytest.mark.parametrize("sliced", [False, True])
+def test_product_division_recomputed_equals_division_of_the_stored_product(dev, fp8, sliced):
+    """coat_fp8_product_division against coat_fp8_mul_forward's stored bf16 product followed by the division, with the
+    second factor dense or a column slice of a wider tensor."""
+    from coat_amd import _hip
+    M, N = 208, 352
+    kind = 0 if fp8 == "E4M3" else 1
+    a, sa = R.fp8_quantize(rand(51, 1.0, (M, N)), QB, fp8)
+    wide, swide = R.fp8_quantize(rand(52, 1.0, (M, 2 * N)), QB, fp8)
+    a, sa, wide, swide = a.to(dev), sa.to(dev), wide.to(dev), swide.to(dev)
+    if sliced:
+        bq, sb, b_pitch, sb_pitch = wide[:, N:], swide[:, N // QB:], 2 * N, 2 * N // QB
+    else:
+        bq, sb, b_pitch, sb_pitch = wide[:, N:].contiguous(), swide[:, N // QB:].contiguous(), 0, 0
+    bd, sbd = wide[:, N:].contiguous(), swide[:, N // QB:].contiguous()
+    lib, st = _hip.lib(), _hip.stream(a.device)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    s_max = torch.zeros((), dtype=torch.float32, device=dev)
+    _hip.check(lib.coat_fp8_mul_forward(_hip.ptr(a), _hip.ptr(sa), _hip.ptr(bd), _hip.ptr(sbd), kind, _hip.dt(sa),
+                                        _hip.ptr(y), None, _hip.ptr(s_max), M, N, QB, st), "mul_forward")
+    want_q, want_qt = torch.empty((M, N), dtype=torch.uint8, device=dev), torch.empty((N, M), dtype=torch.uint8, device=dev)
+    want_s = torch.zeros((), dtype=torch.bfloat16, device=dev)
+    _hip.check(lib.coat_fp8_division_from_max(_hip.ptr(y), _hip.dt(y), _hip.ptr(s_max), _hip.ptr(want_s), _hip.dt(want_s),
+                                              _hip.ptr(want_q), _hip.ptr(want_qt), M, N, kind, st), "division")
+    got_q, got_qt, got_s = torch.empty_like(want_q), torch.empty_like(want_qt), torch.zeros_like(want_s)
+    _hip.check(lib.coat_fp8_product_division(_hip.ptr(a), _hip.ptr(sa), _hip.dt(sa), _hip.ptr(bq), _hip.ptr(sb), _hip.dt(sb),
+                                             kind, _hip.ptr(s_max), _hip.ptr(got_s), _hip.ptr(got_q), _hip.ptr(got_qt), M, N,
+                                             QB, b_pitch, sb_pitch, st), "product_division")
+    assert torch.equal(got_q, want_q) and torch.equal(got_qt, want_qt) and got_s.item() == want_s.item() > 0
