@@ -331,24 +331,20 @@ def make_layernorm_workload(dev, torch):
 
 
 def make_hbm_probe_workload(dev, torch, kind):
-    """What this box's HBM delivers to simple kernels on 1 GiB: "copy" (torch's device copy: 1 GiB read + 1 GiB written),
-    "read" (this library's absmax reduction over bf16: read only), "fill" (torch's fill kernel: write only).  These are the
-    practical ceilings the streaming kernels are compared with next to the nominal 8 TB/s."""
+    """What this box's HBM delivers to the simplest kernels on 1 GiB (coat_hbm_probe: one 16-byte access per lane,
+    streaming loads): "copy" (1 GiB read + 1 GiB written), "read", "fill".  These are the practical ceilings the
+    streaming kernels are compared with next to the nominal 8 TB/s."""
     from coat_amd import _hip
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
-    if kind == "copy":
-        dst = torch.empty_like(src)
-        return (lambda: dst.copy_(src)), 2 * n, {"workload": "hbm_probe copy: torch device copy of 1 GiB", "kernel": "copy"}
-    if kind == "fill":
-        return (lambda: src.fill_(3)), n, {"workload": "hbm_probe fill: torch fill of 1 GiB", "kernel": "fill"}
-    x = src.view(torch.bfloat16)
-    amax = torch.zeros((), dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src) if kind != "read" else torch.zeros(16, dtype=torch.uint8, device=dev)
+    code = {"copy": 0, "read": 1, "fill": 2}[kind]
 
     def step():
-        _hip.check(_hip.lib().coat_absmax(_hip.ptr(x), _hip.dt(x), _hip.ptr(amax), x.numel(), _hip.stream(dev)), "absmax")
+        _hip.check(_hip.lib().coat_hbm_probe(code, _hip.ptr(src), _hip.ptr(dst), n, _hip.stream(dev)), "hbm_probe")
 
-    return step, n, {"workload": "hbm_probe read: coat_absmax over 1 GiB of bf16", "kernel": "k_absmax"}
+    return step, (2 * n if kind == "copy" else n), {"workload": f"hbm_probe {kind}: coat_hbm_probe on 1 GiB",
+                                                      "kernel": "k_hbm_probe"}
 
 
 def make_division_workload(dev, torch, stochastic):

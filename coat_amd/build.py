@@ -22,7 +22,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
-]
+] + os.environ.get("COAT_HIPCC_FLAGS", "").split()  # extra flags (e.g. -D tuning switches) for experiments
 
 
 def sources():
@@ -36,7 +36,8 @@ def _compile(src):
     return src, obj, r.returncode, r.stdout + r.stderr
 
 
-def build(verbose=True, jobs=None):
+def build(verbose=True, jobs=None, lib=None):
+    lib = lib or os.environ.get("COAT_LIB_OUT") or LIB
     os.makedirs(OBJ, exist_ok=True)
     srcs = sources()
     jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")))
@@ -53,13 +54,13 @@ def build(verbose=True, jobs=None):
                 for l in warn[:10]:
                     print("   ", l)
             objs.append(obj)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
     if verbose:
-        print(f"[coat_amd.build] linked {LIB}")
-    return LIB
+        print(f"[coat_amd.build] linked {lib}")
+    return lib
 
 
 if __name__ == "__main__":

@@ -84,10 +84,10 @@ template <int PDT> struct PVec { static constexpr int kBytes = (PDT == kF32) ? 1
 template <int PDT> __device__ __forceinline__ void load4(const void* base, int64_t e, int64_t numel, float* o) {
     if (e + 3 < numel) {
         if (PDT == kF32) {
-            float4 t = *(const float4*)((const float*)base + e);
-            o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+            const uint4 t = ld_stream16((const float*)base + e);
+            o[0] = u2f(t.x); o[1] = u2f(t.y); o[2] = u2f(t.z); o[3] = u2f(t.w);
         } else {
-            uint2 t = *(const uint2*)((const uint16_t*)base + e);
+            const uint2 t = ld_stream8((const uint16_t*)base + e);
             o[0] = PDT == kBF16 ? bf16lo(t.x) : f16lo(t.x);
             o[1] = PDT == kBF16 ? bf16hi(t.x) : f16hi(t.x);
             o[2] = PDT == kBF16 ? bf16lo(t.y) : f16lo(t.y);
@@ -110,7 +110,7 @@ template <int PDT> __device__ __forceinline__ void store4(void* base, int64_t e,
     }
 }
 __device__ __forceinline__ uint32_t load_codes4(const uint8_t* base, int64_t e, int64_t numel) {
-    if (e + 3 < numel) return *(const uint32_t*)(base + e);
+    if (e + 3 < numel) return ld_stream4(base + e);
     uint32_t w = 0;
 #pragma unroll
     for (int i = 0; i < 4; i++)

@@ -44,6 +44,23 @@ __device__ __forceinline__ float f16lo(uint32_t w) { return (float)__builtin_bit
 __device__ __forceinline__ float f16hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
 __device__ __forceinline__ uint32_t f2f16(float f) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f); }
 
+// Streaming (non-temporal) global loads for data that a kernel reads once and no later kernel reads again soon (the
+// optimizer state, the logits of the loss): the caches treat such lines as first candidates for replacement.  On 1 GiB
+// probes: read 7.1 instead of 6.5 TB/s, copy 6.2-6.6 instead of 5.8-6.2 TB/s; the AdamW step gains 8 %, the cross-entropy
+// kernel 6 %.  Not used where a following kernel re-reads the tensor from the cache (the norms lose 16-26 % with it),
+// nor for stores (the in-place AdamW update loses 9 % with streaming stores).
+typedef uint32_t coat_u4v __attribute__((ext_vector_type(4)));
+typedef uint32_t coat_u2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 ld_stream16(const void* p) {
+    const coat_u4v v = __builtin_nontemporal_load((const coat_u4v*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 ld_stream8(const void* p) {
+    const coat_u2v v = __builtin_nontemporal_load((const coat_u2v*)p);
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t ld_stream4(const void* p) { return __builtin_nontemporal_load((const uint32_t*)p); }
+
 // Typed scalar load / store used for scale tensors and ragged tails.
 template <int DT> __device__ __forceinline__ float load_as_f32(const void* p, int64_t i) {
     if (DT == kF32) return ((const float*)p)[i];
@@ -90,11 +107,18 @@ template <int KIND, int SEL> __device__ __forceinline__ float fp8_to_f32(uint32_
     if (KIND == kE4M3) return __builtin_amdgcn_cvt_f32_fp8(w, SEL);
     return __builtin_amdgcn_cvt_f32_bf8(w, SEL);
 }
+// four codes of one dword: two packed conversions (v_cvt_pk_f32_fp8 / _bf8 convert a 16-bit half each)
+typedef float coat_f2v __attribute__((ext_vector_type(2)));
 template <int KIND> __device__ __forceinline__ void fp8x4_to_f32(uint32_t w, float* o) {
-    o[0] = fp8_to_f32<KIND, 0>(w);
-    o[1] = fp8_to_f32<KIND, 1>(w);
-    o[2] = fp8_to_f32<KIND, 2>(w);
-    o[3] = fp8_to_f32<KIND, 3>(w);
+    coat_f2v lo, hi;
+    if (KIND == kE4M3) {
+        lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+        hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+    } else {
+        lo = __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+        hi = __builtin_amdgcn_cvt_pk_f32_bf8(w, true);
+    }
+    o[0] = lo.x; o[1] = lo.y; o[2] = hi.x; o[3] = hi.y;
 }
 
 // ------------------------------------------------------------------------------------------------ exact division

@@ -34,10 +34,11 @@ template <int XDT, int VEC> __device__ __forceinline__ void load_chunk(const voi
     const int64_t e0 = j * VEC;
     if (VEC > 1 && e0 + VEC <= V) {
         if (XDT == kF32) {
-            const float4 t = *(const float4*)((const float*)row + e0);
+            const uint4 tu = ld_stream16((const float*)row + e0);
+            const float4 t = make_float4(u2f(tu.x), u2f(tu.y), u2f(tu.z), u2f(tu.w));
             v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
         } else {
-            const uint4 t = *(const uint4*)((const uint16_t*)row + e0);
+            const uint4 t = ld_stream16((const uint16_t*)row + e0);
             const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
             for (int i = 0; i < 4; i++) {

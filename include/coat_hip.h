@@ -35,6 +35,9 @@ enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.f
 
 const char* coat_version(void);
 const char* coat_status_string(int status);
+/* Memory-bandwidth probe for the benchmarks (no counterpart in the reference): kind 0 copies bytes from src to dst,
+ * 1 reads src (dst: 4 writable bytes), 2 fills dst; one 16-byte access per lane, bytes % 16 == 0. */
+int coat_hbm_probe(int kind, const void* src, void* dst, int64_t bytes, void* stream);
 
 /* ---- quantize family -------------------------------------------------------------------------- */
 
