@@ -274,7 +274,7 @@ using namespace coat;
 
 template <int OP> static int launch_ew(const EwArgs& A, int kind_in, int kind_out, hipStream_t st) {
     int64_t blocks = (A.nchunk + 255) / 256;
-    if (blocks > 2048) blocks = 2048;  // 8 blocks per CU; the kernel strides over the rest
+    if (blocks > 2048) blocks = 2048;  // 8 blocks per CU; the kernel strides over the rest (8192 blocks or no cap: slower)
 #define EW_LAUNCH(KI, KO)                                                                                   \
     hipLaunchKernelGGL((k_elementwise<OP, KI, KO>), dim3((unsigned)blocks), dim3(256), 0, st, A); \
     return coat_launch_status();
