@@ -347,9 +347,10 @@ def make_hbm_probe_workload(dev, torch, kind):
                                                       "kernel": "k_hbm_probe"}
 
 
-def make_division_workload(dev, torch, stochastic):
+def make_division_workload(dev, torch, stochastic, transpose=False):
     """Per-tensor division bf16 [8192,4096] -> e5m2 with a given scale, deterministic or with the reference's stochastic
-    rounding (coat/activation/real_quantization/_division.py:153-207): 2 bytes read + 1 written per element."""
+    rounding (coat/activation/real_quantization/_division.py:153-207): 2 bytes read + 1 written per element; with
+    ``transpose`` the transposed copy is written too (_division_transpose.py:147-210, 2 + 2 bytes)."""
     import coat_amd.activation.real_quantization as rq
 
     M, N = 8192, 4096
@@ -360,10 +361,15 @@ def make_division_workload(dev, torch, stochastic):
 
     def step():
         it["i"] = (it["i"] + 1) % len(xs)
-        rq.fp8_division(xs[it["i"]], 16, "E5M2", scale, stochastic=stochastic)
+        if transpose:
+            rq.fp8_division_transpose(xs[it["i"]], 16, "E5M2", scale)
+        else:
+            rq.fp8_division(xs[it["i"]], 16, "E5M2", scale, stochastic=stochastic)
 
-    return step, 3 * M * N, {"workload": f"fp8_division bf16 [{M},{N}] -> e5m2, stochastic={stochastic}", "M": M, "N": N,
-                            "kernel": "k_division"}
+    name = "fp8_division_transpose" if transpose else "fp8_division"
+    return step, (4 if transpose else 3) * M * N, {
+        "workload": f"{name} bf16 [{M},{N}] -> e5m2, stochastic={stochastic}", "M": M, "N": N,
+        "kernel": "k_division_transpose" if transpose else "k_division"}
 
 
 def make_layer_workload(dev, torch, size, cache_weights=False):
@@ -534,7 +540,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adamw", choices=["adamw", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
-                             "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr", "olmo_block",
+                             "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr", "division_transpose", "olmo_block",
                              "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", type=int, nargs=2, default=[4096, 4096], metavar=("M", "N"),
@@ -579,8 +585,9 @@ def main():
         step, nbytes, cfg = make_hbm_probe_workload(dev, torch, args.workload.split("_")[1])
     elif args.workload == "layernorm":
         step, nbytes, cfg = make_layernorm_workload(dev, torch)
-    elif args.workload in ("division", "division_sr"):
-        step, nbytes, cfg = make_division_workload(dev, torch, args.workload == "division_sr")
+    elif args.workload in ("division", "division_sr", "division_transpose"):
+        step, nbytes, cfg = make_division_workload(dev, torch, args.workload == "division_sr",
+                                                   transpose=args.workload == "division_transpose")
     elif args.workload == "silu_mul":
         step, nbytes, cfg = make_silu_mul_workload(dev, torch)
     elif args.workload == "rmsnorm":
