@@ -477,7 +477,7 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
     static_assert(QB <= TN && TM % QB == 0, "tile must hold whole groups in both directions");
     extern __shared__ float tile[];  // TM x PITCH fp32 (dynamic: 65 KiB for the 128 x 128 tile of QB = 128)
     enable_fp8_saturation();
-    const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
+    const int64_t tiles_n = (N + TN - 1) / TN;
     const int64_t SN = N / QB, SM = M / QB;
     // One tile per block, tiles taken in row-major order: the blocks resident at any time then read and write a few
     // whole bands of rows of x and q (long contiguous runs for the memory controllers) and the hardware balances the
