@@ -65,6 +65,18 @@ def _rmsnorm_division(x, s_x, w, rstd, s_max, QB, what):
     return q, s_out, q_t
 
 
+def _layernorm_division(x, s_x, w, b, mean, rstd, s_max, QB, what):
+    """(q, s, q_t) of the fp32 tensor (x - mean) * rstd (* w + b) divided by the bf16-rounded ``s_max``, recomputed tile
+    by tile from the norm's inputs (same codes as ``_division`` on the stored fp32 tensor)."""
+    M, N = x.shape
+    q, q_t, s_out = _outputs_for(x, x.dtype)
+    _hip.check(_hip.lib().coat_fp8_layernorm_division(
+        _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.ptr(b),
+        -1 if w is None else _hip.dt(w), _hip.ptr(mean), _hip.ptr(rstd), _hip.ptr(s_max), _hip.ptr(s_out), _hip.ptr(q),
+        _hip.ptr(q_t), M, N, QB, _hip.stream(x.device)), what)
+    return q, s_out, q_t
+
+
 def _product_division(a, s_a, b, s_b, b_pitch, sb_pitch, s_max, QB, what):
     """(q, s, q_t) of bf16(dequant(a) * dequant(b)) divided by the bf16-rounded ``s_max``, recomputed from the factors.
     ``b`` may be a column slice (row pitches in codes / scales, 0 = dense)."""

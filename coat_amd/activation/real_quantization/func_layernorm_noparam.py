@@ -3,7 +3,7 @@ Reference: coat/activation/real_quantization/func_layernorm_noparam.py:193-297."
 import torch
 
 from ... import _hip
-from ._division import _division
+from ._division import _division, _layernorm_division
 from ._fused import new_max, prep_bf16, prep_pg
 from .common import no_stochastic, restore
 
@@ -11,16 +11,24 @@ from .common import no_stochastic, restore
 def _forward(x, s_x, w, b, QB, eps, transpose_output_2d, who):
     x, s_x, batch = prep_pg(x, s_x)
     M, N = x.shape
-    y = torch.empty_like(x, dtype=torch.float32)  # the reference keeps the normalised tensor in fp32 (:205)
+    # the reference keeps the normalised tensor in fp32 (:205); here the division recomputes it tile by tile from x, mean
+    # and rstd, so it is only stored when the row count does not allow the tiled kernel
+    recompute = M % 16 == 0 and M > 0
+    y = None if recompute else torch.empty_like(x, dtype=torch.float32)
     s_row = torch.empty((M,), dtype=torch.bfloat16, device=x.device)
     mean = torch.empty((M,), dtype=torch.float32, device=x.device)
     rstd = torch.empty((M,), dtype=torch.float32, device=x.device)
     s_max = new_max(x.device)
+    if w is not None:
+        w, b = _hip.dense(w), _hip.dense(b)
     _hip.check(_hip.lib().coat_fp8_layernorm_forward(
         _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(w), _hip.ptr(b),
         -1 if w is None else _hip.dt(w), _hip.ptr(y), _hip.ptr(s_row), _hip.ptr(mean), _hip.ptr(rstd), _hip.ptr(s_max),
         M, N, QB, float(eps), _hip.stream(x.device)), who)
-    qy, s_y_max, qy_t = _division(y, x.dtype, s_max, True, True, who, max_as=torch.bfloat16)
+    if recompute:
+        qy, s_y_max, qy_t = _layernorm_division(x, s_x, w, b, mean, rstd, s_max, QB, who)
+    else:
+        qy, s_y_max, qy_t = _division(y, x.dtype, s_max, True, True, who, max_as=torch.bfloat16)
     if batch is not None and not transpose_output_2d:
         qy_t = qy_t.reshape(batch, -1, N)
     return restore(qy, batch), s_y_max, qy_t, mean, rstd

@@ -80,9 +80,11 @@ __global__ __launch_bounds__(256) void k_layernorm_fwd(const uint8_t* __restrict
                 yv[i] = v;
                 amax = fmaxf(amax, fabsf(v));
             }
-            float4* dst = (float4*)(y + row_off + col);
+            if (y) {  // NULL: statistics only (the division recomputes y)
+                float4* dst = (float4*)(y + row_off + col);
 #pragma unroll
-            for (int i = 0; i < 4; i++) dst[i] = make_float4(yv[4 * i], yv[4 * i + 1], yv[4 * i + 2], yv[4 * i + 3]);
+                for (int i = 0; i < 4; i++) dst[i] = make_float4(yv[4 * i], yv[4 * i + 1], yv[4 * i + 2], yv[4 * i + 3]);
+            }
         }
     }
     amax = block_max_256(amax, smem);
@@ -207,7 +209,7 @@ extern "C" int coat_fp8_layernorm_forward(const void* x, int fp8, const void* s_
                                           float* s_max, int64_t M, int64_t N, int QB, float eps, void* stream) {
     if (int e = ln_check(M, N, QB)) return e;
     if (M * N == 0) return COAT_OK;
-    if (!x || !s_x || !y || !s_row || !mean || !rstd || !s_max) return COAT_EINVAL;
+    if (!x || !s_x || !s_row || !mean || !rstd || !s_max) return COAT_EINVAL;  // y may be NULL
     if (w_dtype >= 0 && (!w || !b)) return COAT_EINVAL;
     if (s_dtype < 0 || s_dtype > 2) return COAT_EDTYPE;
     if (!coat_aligned16(x) || !coat_aligned16(y) || !coat_aligned16(w) || !coat_aligned16(b)) return COAT_EALIGN;

@@ -394,6 +394,60 @@ template <int KIND, int WDT> struct RmsNormSource {
     }
 };
 
+// (x - mean[row]) * rstd[row] (* w[col] + b[col]) of k_layernorm_fwd, kept in fp32 as the reference keeps it
+// (coat/activation/real_quantization/func_layernorm_noparam.py:85-100, func_layernorm_param.py:90-108).
+// WMODE: dtype of w and b, or 3 = no affine parameters.
+template <int KIND, int WMODE> struct LayerNormSource {
+    static constexpr int kNW = WMODE == 3 ? 1 : (WMODE == kF32 ? 4 : 2);  // 16-byte pieces of 16 weights
+    const uint8_t* q; const void* s; const void* w; const void* b; const float* mean; const float* rstd;
+    int s_dt, qb; int64_t N;
+    struct Raw { uint4 codes; float sc, mean, rstd; uint4 w[kNW], b[kNW]; };
+    __device__ __forceinline__ void load(int64_t m, int64_t n, Raw& r) const {
+        r.codes = *(const uint4*)(q + m * N + n);
+        r.sc = load_rt_f32(s, m * (N / qb) + n / qb, s_dt);
+        r.mean = mean[m];
+        r.rstd = rstd[m];
+        if constexpr (WMODE != 3) {
+            const uint4* wp = (const uint4*)((const uint8_t*)w + n * (WMODE == kF32 ? 4 : 2));
+            const uint4* bp = (const uint4*)((const uint8_t*)b + n * (WMODE == kF32 ? 4 : 2));
+#pragma unroll
+            for (int i = 0; i < kNW; i++) { r.w[i] = wp[i]; r.b[i] = bp[i]; }
+        }
+    }
+    static __device__ __forceinline__ void unpack16(const uint4* p, float* o) {
+        if constexpr (WMODE == kF32) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                o[4 * i] = u2f(p[i].x); o[4 * i + 1] = u2f(p[i].y); o[4 * i + 2] = u2f(p[i].z); o[4 * i + 3] = u2f(p[i].w);
+            }
+        } else if constexpr (WMODE != 3) {
+            const uint32_t u[8] = {p[0].x, p[0].y, p[0].z, p[0].w, p[1].x, p[1].y, p[1].z, p[1].w};
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                o[2 * k] = WMODE == kBF16 ? bf16lo(u[k]) : f16lo(u[k]);
+                o[2 * k + 1] = WMODE == kBF16 ? bf16hi(u[k]) : f16hi(u[k]);
+            }
+        }
+    }
+    __device__ __forceinline__ void value(const Raw& r, float* v) const {
+        const uint32_t c[4] = {r.codes.x, r.codes.y, r.codes.z, r.codes.w};
+        float wv[16], bv[16];
+        unpack16(r.w, wv);
+        unpack16(r.b, bv);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            float f[4];
+            fp8x4_to_f32<KIND>(c[k], f);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float t = ((f[i] * r.sc) - r.mean) * r.rstd;
+                if constexpr (WMODE != 3) t = t * wv[4 * k + i] + bv[4 * k + i];
+                v[4 * k + i] = t;
+            }
+        }
+    }
+};
+
 // bf16(dequant(a) * dequant(b)) of two per-group FP8 tensors: the product of k_silu_mul's forward
 // (coat/activation/real_quantization/mul_fwd.py:136-150).  a is dense [M, N]; b may be a column slice of a wider tensor
 // (row pitches in elements / scales).
@@ -818,6 +872,40 @@ extern "C" int coat_fp8_rmsnorm_division(const void* x, int fp8, const void* s_x
         return COAT_EDTYPE;
     });
 #undef RMS_DIV
+    return COAT_EINVAL;
+}
+
+// The same for coat_fp8_layernorm_forward (y = NULL there); w_dtype < 0: no affine parameters.
+extern "C" int coat_fp8_layernorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, const void* b,
+                                           int w_dtype, const float* mean, const float* rstd, const float* s_max,
+                                           void* s_out, void* q, void* qt, int64_t M, int64_t N, int QB, void* stream) {
+    if (int e = check_mn(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (M % 16 != 0 || N % 16 != 0 || QB % 16 != 0) return COAT_ESHAPE;
+    if (!x || !s_x || !mean || !rstd || !s_max || !s_out || !q || !qt) return COAT_EINVAL;
+    if (w_dtype >= 0 && (!w || !b)) return COAT_EINVAL;
+    if (w_dtype > 2) return COAT_EDTYPE;
+    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(b) || !coat_aligned16(q) || !coat_aligned16(qt))
+        return COAT_EALIGN;
+    if (s_dtype < 0 || s_dtype > 2) return COAT_EDTYPE;
+    const int64_t blocks = ((M + 127) / 128) * ((N + kTileN - 1) / kTileN);
+    if (blocks >= ((int64_t)1 << 31)) return COAT_ESHAPE;
+    hipStream_t st = (hipStream_t)stream;
+#define LN_DIV(KINDV, WM)                                                                                            \
+    {                                                                                                                \
+        LayerNormSource<KINDV, WM> src{(const uint8_t*)x, s_x, w, b, mean, rstd, s_dtype, QB, N};                    \
+        hipLaunchKernelGGL((k_produced_division_transpose<LayerNormSource<KINDV, WM>, KINDV>), dim3((unsigned)blocks), \
+                           dim3(kDivTThreads), 0, st, src, s_max, s_out, q, qt, M, N);                               \
+        return coat_launch_status();                                                                                 \
+    }
+    DISPATCH_KIND(fp8, {
+        if (w_dtype < 0) LN_DIV(KIND, 3)
+        if (w_dtype == COAT_BF16) LN_DIV(KIND, kBF16)
+        if (w_dtype == COAT_F32) LN_DIV(KIND, kF32)
+        if (w_dtype == COAT_F16) LN_DIV(KIND, kF16)
+        return COAT_EDTYPE;
+    });
+#undef LN_DIV
     return COAT_EINVAL;
 }
 

@@ -157,6 +157,12 @@ int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtyp
 int coat_fp8_rmsnorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype,
                               const float* rstd, const float* s_max, void* s_out, void* q, void* qt, int64_t M, int64_t N,
                               int QB, void* stream);
+/* The same for coat_fp8_layernorm_forward (rq/func_layernorm_noparam.py:193, rq/func_layernorm_param.py:258; y = NULL
+ * there): y = (x - mean) * rstd (* w + b) in fp32, as the reference keeps it, recomputed per tile.  w_dtype < 0: no affine
+ * parameters (w, b NULL). */
+int coat_fp8_layernorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, const void* b,
+                                int w_dtype, const float* mean, const float* rstd, const float* s_max, void* s_out, void* q,
+                                void* qt, int64_t M, int64_t N, int QB, void* stream);
 /* The same for the product of two per-group FP8 tensors, y = bf16(dequant(a) * dequant(b)) (kernel rq/mul_fwd.py:136-150;
  * the division is its fp8_division_transpose call at :243): a [M, N] dense (the SiLU output that
  * coat_fp8_silu_mul_forward just wrote, or x1 of fp8_mul_forward), b with row pitches b_pitch codes / sb_pitch scales

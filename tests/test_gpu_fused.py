@@ -342,3 +342,42 @@ def test_product_division_recomputed_equals_division_of_the_stored_product(dev, 
                                              kind, _hip.ptr(s_max), _hip.ptr(got_s), _hip.ptr(got_q), _hip.ptr(got_qt), M, N,
                                              QB, b_pitch, sb_pitch, st), "product_division")
     assert torch.equal(got_q, want_q) and torch.equal(got_qt, want_qt) and got_s.item() == want_s.item() > 0
+
+
+@pytest.mark.parametrize("wdtype", [None, torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("shape,QBv", [((48, 176), 16), ((272, 4096), 32)])
+def test_layernorm_division_recomputed_equals_division_of_the_stored_tensor(dev, wdtype, shape, QBv):
+    """coat_fp8_layernorm_division recomputes the fp32 y from the norm's inputs: same codes, transpose and scale as dividing
+    the fp32 tensor that coat_fp8_layernorm_forward stores (with and without affine parameters)."""
+    from coat_amd import _hip
+    M, N = shape
+    q, s = R.fp8_quantize(rand(61, 1.0, shape) + 0.25, QBv, "E4M3")
+    q, s = q.to(dev), s.to(dev)
+    w = b = None
+    if wdtype is not None:
+        gen = torch.Generator().manual_seed(7)
+        w = (torch.ones(N) + 0.1 * torch.randn(N, generator=gen)).to(wdtype).to(dev)
+        b = (0.05 * torch.randn(N, generator=gen)).to(wdtype).to(dev)
+    wd = -1 if w is None else _hip.dt(w)
+    y = torch.empty((M, N), dtype=torch.float32, device=dev)
+    s_row = torch.empty((M,), dtype=torch.bfloat16, device=dev)
+    mean, rstd = torch.empty((M,), dtype=torch.float32, device=dev), torch.empty((M,), dtype=torch.float32, device=dev)
+    s_max = torch.zeros((), dtype=torch.float32, device=dev)
+    lib, st = _hip.lib(), _hip.stream(q.device)
+    _hip.check(lib.coat_fp8_layernorm_forward(_hip.ptr(q), 0, _hip.ptr(s), _hip.dt(s), _hip.ptr(w), _hip.ptr(b), wd,
+                                              _hip.ptr(y), _hip.ptr(s_row), _hip.ptr(mean), _hip.ptr(rstd), _hip.ptr(s_max),
+                                              M, N, QBv, 1e-5, st), "fwd")
+    mean2, rstd2, s_max2 = torch.empty_like(mean), torch.empty_like(rstd), torch.zeros_like(s_max)
+    _hip.check(lib.coat_fp8_layernorm_forward(_hip.ptr(q), 0, _hip.ptr(s), _hip.dt(s), _hip.ptr(w), _hip.ptr(b), wd, None,
+                                              _hip.ptr(s_row), _hip.ptr(mean2), _hip.ptr(rstd2), _hip.ptr(s_max2), M, N, QBv,
+                                              1e-5, st), "stats")
+    assert torch.equal(mean, mean2) and torch.equal(rstd, rstd2) and torch.equal(s_max, s_max2)
+    want_q, want_qt = torch.empty((M, N), dtype=torch.uint8, device=dev), torch.empty((N, M), dtype=torch.uint8, device=dev)
+    want_s = torch.zeros((), dtype=torch.bfloat16, device=dev)
+    _hip.check(lib.coat_fp8_division_from_max(_hip.ptr(y), _hip.dt(y), _hip.ptr(s_max), _hip.ptr(want_s), _hip.dt(want_s),
+                                              _hip.ptr(want_q), _hip.ptr(want_qt), M, N, 0, st), "division")
+    got_q, got_qt, got_s = torch.empty_like(want_q), torch.empty_like(want_qt), torch.zeros_like(want_s)
+    _hip.check(lib.coat_fp8_layernorm_division(_hip.ptr(q), 0, _hip.ptr(s), _hip.dt(s), _hip.ptr(w), _hip.ptr(b), wd,
+                                               _hip.ptr(mean), _hip.ptr(rstd), _hip.ptr(s_max), _hip.ptr(got_s),
+                                               _hip.ptr(got_q), _hip.ptr(got_qt), M, N, QBv, st), "layernorm_division")
+    assert torch.equal(got_q, want_q) and torch.equal(got_qt, want_qt) and got_s.item() == want_s.item() > 0
