@@ -265,9 +265,11 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     const uint32_t q_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * G.N + wn * (TJ * 32) + 8 * half);
     const uint32_t s_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * (G.N >> 4) + wn * (TJ * 2)) * 2;
     const int q_n_lim = G.N - n0 - wn * (TJ * 32);          // a 16-column group at offset c exists iff c < q_n_lim
+    const bool pack_scales = (G.N & 63) == 0 && q_n_lim >= TJ * 32 && ((uintptr_t)G.Cs & 7) == 0;  // wave-uniform
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int m = m0 + wm * 128 + i * 32 + (lane & 31);
+        uint32_t spack[TJ] = {};
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const int nb = n0 + wn * (TJ * 32) + j * 32 + 4 * half;  // + 8*q + {0..3}
@@ -323,7 +325,10 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                     float amax = 0.0f;
 #pragma unroll
                     for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[8 * g2 + e]));
-                    amax = fmaxf(amax, lane_xor_f32(amax, 32));
+                    // the other half of the group sits in lane ^ 32: a swap of the value with itself leaves [lo, lo] and
+                    // [hi, hi] in the two results
+                    const auto am = __builtin_amdgcn_permlane32_swap(f2u(amax), f2u(amax), false, false);
+                    amax = fmaxf(u2f(am[0]), u2f(am[1]));
                     const float s = group_scale<KIND>(amax);
                     const float r = 1.0f / s;
                     const uint32_t w0 = cvt4_fp8<KIND>(div_by_scale(v[8 * g2], s, r), div_by_scale(v[8 * g2 + 1], s, r),
@@ -334,13 +339,20 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                     if (i * 32 < m_lim && j * 32 + 16 * g2 < q_n_lim) {
                         uint8_t* base = q_tile + ((int64_t)(i * 32) * G.N + j * 32 + 16 * g2);
                         *(uint2*)(base + q_lane_off) = make_uint2(sw[0], sw[1]);
-                        if (half == 0) {
+                        if (half == 0 && !pack_scales) {
                             uint8_t* sbase = s_tile + ((int64_t)(i * 32) * (G.N >> 4) + j * 2 + g2) * 2;
                             *(uint16_t*)(sbase + s_lane_off) = (uint16_t)f2bf16(s);
                         }
                     }
+                    spack[j] |= f2bf16(s) << (16 * g2);
                 }
             }
+        }
+        // the wave's four group scales of a row (64 columns) are 8 contiguous bytes: one store when they are all inside
+        // the matrix and the row's scales start 8-byte aligned
+        if (EPI != kEpiBf16 && pack_scales && half == 0 && i * 32 < m_lim) {
+            uint8_t* sbase = s_tile + (int64_t)(i * 32) * (G.N >> 4) * 2;
+            *(uint2*)(sbase + s_lane_off) = make_uint2(spack[0], spack[1]);
         }
     }
     }  // epilogue of tile it - 1
