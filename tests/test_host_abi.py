@@ -47,6 +47,52 @@ def test_argument_validation_without_gpu():
         _hip.check(-2, "x")
 
 
+def test_argument_validation_of_the_remaining_entry_points_without_gpu():
+    """Every entry point checks shapes, pointers, alignment and enums before it launches anything."""
+    from coat_amd import _hip
+
+    L = _hip.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+    odd = ctypes.c_void_p(p.value + 4)
+    EINVAL, ESHAPE, EDTYPE, EALIGN = -1, -2, -3, -5
+    # per-tensor division family
+    assert L.coat_fp8_division(p, 1, p, 1, p, p, 24, 64, 0, None) == ESHAPE            # transpose needs M % 16 == 0
+    assert L.coat_fp8_division(p, 1, p, 1, None, None, 16, 64, 0, None) == EINVAL      # no output at all
+    assert L.coat_fp8_division(p, 1, p, 1, odd, None, 16, 64, 0, None) == EALIGN
+    assert L.coat_fp8_division(p, 1, p, 9, p, None, 16, 64, 0, None) == EDTYPE         # unknown scale dtype
+    assert L.coat_fp8_division(p, 1, p, 1, p, None, 16, 64, 5, None) == EINVAL         # unknown fp8 kind
+    assert L.coat_fp8_division_from_max(p, 1, p, None, 1, p, None, 16, 64, 0, None) == EINVAL  # nowhere to put the scale
+    assert L.coat_fp8_division_stochastic(p, 1, p, 1, p, None, 1 << 17, 1 << 16, 0, 0, None) == ESHAPE  # > 2^32 noise indices
+    assert L.coat_fp8_dequantize(p, 0, p, 1, p, 4, 64, 24, None) == ESHAPE
+    # the divisions that recompute their input
+    assert L.coat_fp8_rmsnorm_division(p, 0, p, 1, p, 1, p, p, p, p, p, 24, 64, 16, None) == ESHAPE
+    assert L.coat_fp8_rmsnorm_division(p, 0, p, 1, p, 1, None, p, p, p, p, 16, 64, 16, None) == EINVAL
+    assert L.coat_fp8_rmsnorm_division(p, 0, p, 1, p, 7, p, p, p, p, p, 16, 64, 16, None) == EDTYPE
+    assert L.coat_fp8_layernorm_division(p, 0, p, 1, None, None, 1, p, p, p, p, p, p, 16, 64, 16, None) == EINVAL  # w, b missing
+    assert L.coat_fp8_layernorm_division(p, 0, p, 1, None, None, -1, p, p, p, p, p, odd, 16, 64, 16, None) == EALIGN
+    assert L.coat_fp8_product_division(p, p, 1, p, p, 1, 0, p, p, p, p, 16, 64, 16, 48, 0, None) == ESHAPE  # pitch < N
+    assert L.coat_fp8_product_division(p, p, 1, p, p, 4, 0, p, p, p, p, 16, 64, 16, 0, 0, None) == EDTYPE
+    # fused activations / norms
+    assert L.coat_fp8_silu_forward(p, 0, p, 1, p, p, 4, 40, 16, None) == ESHAPE
+    assert L.coat_fp8_silu_mul_forward(p, p, p, p, 0, 1, p, p, None, None, 4, 64, 16, 0, 0, None) == EINVAL  # no maximum word
+    assert L.coat_fp8_rmsnorm_forward(p, 0, p, 1, p, 1, None, p, p, p, 4, 32768, 16, 1e-5, None) == ESHAPE   # row too long
+    assert L.coat_fp8_rmsnorm_forward(p, 0, p, 1, p, 1, None, None, p, p, 4, 64, 16, 1e-5, None) == EINVAL
+    # GEMM
+    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 0, p, p, 1, None, 0, 64, 64, 24, 16, None) == ESHAPE    # K % 16
+    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 1, p, p, 1, None, 0, 64, 64, 64, 16, None) == ESHAPE    # quantized output without scales
+    assert L.coat_fp8_gemm(p, 3, p, 0, p, None, 0, p, p, 1, None, 0, 64, 64, 64, 16, None) == EINVAL    # unknown operand format
+    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 0, p, p, 1, None, 0, 0, 64, 64, 16, None) == 0          # empty
+    # RoPE, cross-entropy, probe
+    assert L.coat_rope_bf16(p, p, p, p, None, 8, 8, 2, 24, 0, 0, 0, None) == ESHAPE                      # head_dim % 16
+    assert L.coat_rope_bf16(p, p, p, p, None, 8, 8, 2, 32, 0, 48, 0, None) == ESHAPE                     # pitch < heads * head_dim
+    assert L.coat_cross_entropy_forward(p, 0, 8, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # stride < columns
+    assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # mean without a count
+    assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, p, 4, 16, -100, 0.0, 0.0, 7, 0.0, 0, None) == EINVAL
+    assert L.coat_hbm_probe(0, p, p, 40, None) == EINVAL                                                   # bytes % 16
+    assert L.coat_hbm_probe(3, p, p, 64, None) == EINVAL
+
+
 def test_quantization_config_defaults():
     from coat_amd.utils._fp8_quantization_config import QuantizationConfig
 
