@@ -29,6 +29,7 @@ SIGNATURES = {
     "coat_fp8_division": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_rmsnorm_division": [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_layernorm_division": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _vp],
+    "coat_fp8_silu_mul_forward_bf16": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_product_division": [_vp, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i64, _i64, _vp],
     "coat_hbm_probe": [_i, _vp, _vp, _i64, _vp],
     "coat_fp8_division_from_max": [_vp, _i, _vp, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],

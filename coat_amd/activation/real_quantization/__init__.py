@@ -11,7 +11,8 @@ from .add_bwd import fp8_add_Ifp_Ifp_Ofp_Opt
 from .add_fwd import fp8_add_Ifp_Ifp_Ofp_Og16
 from .func_layernorm_noparam import fp8_layernorm_noparam_backward, fp8_layernorm_noparam_forward
 from .func_layernorm_param import fp8_layernorm_param_backward, fp8_layernorm_param_forward
-from .silu_mul import fp8_silu_mul_backward, fp8_silu_mul_backward_joined, fp8_silu_mul_forward
+from .silu_mul import (fp8_silu_mul_backward, fp8_silu_mul_backward_joined, fp8_silu_mul_forward,
+                       fp8_silu_mul_forward_from_bf16)
 from .func_rmsnorm import fp8_rmsnorm_backward, fp8_rmsnorm_forward
 from .gelu_bwd import fp8_gelu_backward
 from .gelu_fwd import fp8_gelu_forward

@@ -60,6 +60,39 @@ def fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, QB, transpose_output_2d=Fal
     return restore(silu_x, batch), restore(silu_s, batch), restore(mul_x, batch), mul_s, mul_x_t
 
 
+def fp8_silu_mul_forward_from_bf16(gate, up, QB, fp8type="E4M3", transpose_output_2d=False):
+    """``gate_x, gate_s = fp8_quantize(gate, QB, fp8type)``, ``up_x, up_s = fp8_quantize(up, QB, fp8type)`` and
+    ``fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, QB, transpose_output_2d)`` in one pass over the two bf16 tensors.
+    Returns (gate_x, gate_s, up_x, up_s, silu_x, silu_s, mul_x, mul_s, mul_x_t), bit-identical to that chain."""
+    fp8type = as_fp8_dtype(fp8type)
+    assert gate.shape == up.shape
+    batch = gate.shape[0] if gate.dim() == 3 else None
+    g2, u2 = prep_bf16(gate), prep_bf16(up)
+    M, N = g2.shape
+    dev = g2.device
+    if N % QB != 0:
+        raise ValueError(f"fp8_silu_mul_forward_from_bf16: the last dimension {N} is not a multiple of the group size {QB}")
+    outs = [torch.empty((M, N), dtype=fp8type, device=dev) for _ in range(3)]
+    scales = [torch.empty((M, N // QB), dtype=torch.bfloat16, device=dev) for _ in range(3)]
+    (gate_x, up_x, silu_x), (gate_s, up_s, silu_s) = outs, scales
+    recompute = M % 16 == 0 and M > 0 and N > 0
+    y = None if recompute else torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    s_max = new_max(dev)
+    _hip.check(_hip.lib().coat_fp8_silu_mul_forward_bf16(
+        _hip.ptr(g2), _hip.ptr(u2), _hip.fp8(fp8type), _hip.ptr(gate_x), _hip.ptr(gate_s), _hip.ptr(up_x), _hip.ptr(up_s),
+        _hip.ptr(silu_x), _hip.ptr(silu_s), _hip.ptr(y), _hip.ptr(s_max), M, N, QB, _hip.stream(dev)),
+        "fp8_silu_mul_forward_from_bf16")
+    if recompute:
+        mul_x, mul_s, mul_x_t = _product_division(silu_x, silu_s, up_x, up_s, 0, 0, s_max, QB, "fp8_silu_mul_forward_from_bf16")
+    else:
+        mul_x, mul_s, mul_x_t = _division(y, fp8type, s_max, True, True, "fp8_silu_mul_forward_from_bf16",
+                                          max_as=torch.bfloat16)
+    if batch is not None and not transpose_output_2d:
+        mul_x_t = mul_x_t.reshape(batch, -1, N)
+    r = lambda t: restore(t, batch)  # noqa: E731
+    return r(gate_x), r(gate_s), r(up_x), r(up_s), r(silu_x), r(silu_s), r(mul_x), mul_s, mul_x_t
+
+
 def _silu_mul_backward_values(gate_x, gate_s, up_x, up_s, silu_x, silu_s, g, QB, fp8type, joined):
     """Runs the fused backward kernel.  joined: the two bf16 gradients are written side by side, [up | gate], into one
     [M, 2N] tensor.  Returns (y_gate, y_up, m_gate, m_up, batch, joined tensor or None)."""

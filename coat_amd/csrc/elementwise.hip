@@ -171,6 +171,7 @@ struct SiluMulArgs {
     void* y;                                                // forward: bf16 product;  backward: bf16 gradient of gate
     void* y2;                                               // backward: bf16 gradient of up
     float *s_max, *s_max2;                                  // max of the fp32 group scales of y / y2
+    void *q_gate_out, *s_gate_out, *q_up_out, *s_up_out;    // forward from bf16 gate / up: their per-group FP8 codes and bf16 scales
     int64_t nchunk;
     int qb, s_dtype;
     // Row pitches, for gate / up taken as column slices of a wider tensor and y / y2 written into one (strided != 0):
@@ -196,7 +197,9 @@ __device__ __forceinline__ float amax16(const float* v) {
     return a;
 }
 
-template <bool BWD, int KIND_IN, int KIND_OUT>
+// FROM16 (forward only): gate / up are bf16 tensors; they are quantized per group here exactly as k_quantize_pg would
+// (codes and bf16 scales stored for the backward) and the rest of the kernel works on the dequantized values.
+template <bool BWD, int KIND_IN, int KIND_OUT, bool FROM16 = false>
 __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
     __shared__ float smem_max[4];
     enable_fp8_saturation();
@@ -215,8 +218,29 @@ __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
             cy = row * A.y_cpr + col;
         }
         float a[16], b[16];
-        load_fp8x16<KIND_IN>(A.gate, cin, load_scale_rt(A.s_gate, gin, A.s_dtype), a);
-        load_fp8x16<KIND_IN>(A.up, cin, load_scale_rt(A.s_up, gin, A.s_dtype), b);
+        if (FROM16) {
+            float raw[2][16];
+            load_bf16x16(A.gate, c, raw[0]);
+            load_bf16x16(A.up, c, raw[1]);
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const float s = group_scale<KIND_IN>(cluster_max_rt(amax16(raw[t]), lpg));
+                const float r = 1.0f / s;
+                uint32_t w[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    w[k] = cvt4_fp8<KIND_IN>(div_by_scale(raw[t][4 * k], s, r), div_by_scale(raw[t][4 * k + 1], s, r),
+                                             div_by_scale(raw[t][4 * k + 2], s, r), div_by_scale(raw[t][4 * k + 3], s, r));
+                if (ok) {
+                    *(uint4*)((uint8_t*)(t ? A.q_up_out : A.q_gate_out) + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+                    if ((threadIdx.x % lpg) == 0) ((uint16_t*)(t ? A.s_up_out : A.s_gate_out))[gidx] = (uint16_t)f2bf16(s);
+                }
+                dequant_words<KIND_IN>(w, round_bf16(s), t ? b : a);  // as the saved activation is read back
+            }
+        } else {
+            load_fp8x16<KIND_IN>(A.gate, cin, load_scale_rt(A.s_gate, gin, A.s_dtype), a);
+            load_fp8x16<KIND_IN>(A.up, cin, load_scale_rt(A.s_up, gin, A.s_dtype), b);
+        }
         if (!BWD) {
             float sv[16];
 #pragma unroll
@@ -386,7 +410,7 @@ static int silu_mul_launch(SiluMulArgs& A, bool bwd, int fp8_in, int fp8_out, in
     if (fp8_in != COAT_E4M3 && fp8_in != COAT_E5M2) return COAT_EINVAL;
     if (bwd && fp8_out != COAT_E4M3 && fp8_out != COAT_E5M2) return COAT_EINVAL;
     if (M * N == 0) return COAT_OK;
-    const void* ptrs[] = {A.gate, A.up, A.silu, A.g, A.q_silu, A.y, A.y2};
+    const void* ptrs[] = {A.gate, A.up, A.silu, A.g, A.q_silu, A.y, A.y2, A.q_gate_out, A.q_up_out};
     for (const void* p : ptrs)
         if (!coat_aligned16(p)) return COAT_EALIGN;
     if (s_pitch < N / QB) return COAT_ESHAPE;
@@ -401,7 +425,10 @@ static int silu_mul_launch(SiluMulArgs& A, bool bwd, int fp8_in, int fp8_out, in
     int64_t blocks = (A.nchunk + 255) / 256;
     if (blocks > 2048) blocks = 2048;
 #define SM_LAUNCH(B, KI, KO) hipLaunchKernelGGL((k_silu_mul<B, KI, KO>), dim3((unsigned)blocks), dim3(256), 0, st, A)
-    if (!bwd) {
+    if (!bwd && A.q_gate_out) {
+        if (fp8_in == COAT_E4M3) hipLaunchKernelGGL((k_silu_mul<false, kE4M3, kE4M3, true>), dim3((unsigned)blocks), dim3(256), 0, st, A);
+        else hipLaunchKernelGGL((k_silu_mul<false, kE5M2, kE5M2, true>), dim3((unsigned)blocks), dim3(256), 0, st, A);
+    } else if (!bwd) {
         if (fp8_in == COAT_E4M3) SM_LAUNCH(false, kE4M3, kE4M3); else SM_LAUNCH(false, kE5M2, kE5M2);
     } else if (fp8_in == COAT_E4M3) {
         if (fp8_out == COAT_E4M3) SM_LAUNCH(true, kE4M3, kE4M3); else SM_LAUNCH(true, kE4M3, kE5M2);
@@ -416,8 +443,21 @@ extern "C" int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, c
                                          int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M,
                                          int64_t N, int QB, int64_t in_pitch, int64_t s_pitch, void* stream) {
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !q_silu || !s_silu || !s_max)) return COAT_EINVAL;  // y may be NULL
-    SiluMulArgs A = {gate, s_gate, up, s_up, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr, 0, 0, 0};
+    SiluMulArgs A = {gate, s_gate, up, s_up, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr,
+                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
     return silu_mul_launch(A, false, fp8, fp8, M, N, QB, s_dtype, in_pitch, s_pitch, 0, (hipStream_t)stream);
+}
+
+// The forward from bf16 gate / up [M, N] (dense): additionally writes their per-group FP8 codes and bf16 scales (what
+// coat_fp8_quantize would give), so the three saved activations and the product's maximum come out of one pass.
+extern "C" int coat_fp8_silu_mul_forward_bf16(const void* gate, const void* up, int fp8, void* q_gate, void* s_gate,
+                                              void* q_up, void* s_up, void* q_silu, void* s_silu, void* y, float* s_max,
+                                              int64_t M, int64_t N, int QB, void* stream) {
+    if ((M > 0 && N > 0) && (!gate || !up || !q_gate || !s_gate || !q_up || !s_up || !q_silu || !s_silu || !s_max))
+        return COAT_EINVAL;  // y may be NULL
+    SiluMulArgs A = {gate, nullptr, up, nullptr, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr,
+                     q_gate, s_gate, q_up, s_up, 0, 0, 0};
+    return silu_mul_launch(A, false, fp8, fp8, M, N, QB, COAT_BF16, 0, 0, 0, (hipStream_t)stream);
 }
 
 extern "C" int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, const void* up, const void* s_up,
@@ -427,6 +467,7 @@ extern "C" int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, 
                                           int64_t y_pitch, void* stream) {
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !silu || !s_silu || !g || !y_gate || !s_max_gate || !y_up || !s_max_up))
         return COAT_EINVAL;
-    SiluMulArgs A = {gate, s_gate, up, s_up, silu, s_silu, g, nullptr, nullptr, y_gate, y_up, s_max_gate, s_max_up, 0, 0, 0};
+    SiluMulArgs A = {gate, s_gate, up, s_up, silu, s_silu, g, nullptr, nullptr, y_gate, y_up, s_max_gate, s_max_up,
+                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
     return silu_mul_launch(A, true, fp8_in, fp8_out, M, N, QB, s_dtype, in_pitch, s_pitch, y_pitch, (hipStream_t)stream);
 }

@@ -133,6 +133,12 @@ int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s_y, float* 
 int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
                               int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M, int64_t N,
                               int QB, int64_t in_pitch, int64_t s_pitch, void* stream);
+/* The same forward from bf16 gate / up [M, N] (dense): also writes their per-group FP8 codes and bf16 scales, bit for bit
+ * what coat_fp8_quantize gives (rq/_quantize.py:120), so that "quantize gate, quantize up, SiLU, multiply" is one pass over
+ * the two bf16 tensors.  No counterpart in the reference (its MLP receives gate / up quantized by the GEMM epilogue). */
+int coat_fp8_silu_mul_forward_bf16(const void* gate, const void* up, int fp8, void* q_gate, void* s_gate, void* q_up,
+                                   void* s_up, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M, int64_t N,
+                                   int QB, void* stream);
 /* backward: y_up = bf16(g * silu), y_gate = bf16(silu'(gate) * bf16(g * up)); *s_max_* = max of their fp32 group
  * scales for the format fp8_out (the per-tensor division that follows is coat_fp8_division).
  * Row pitches in elements, 0 = contiguous: in_pitch / s_pitch for gate, up and their scales when they are the two column

@@ -381,3 +381,25 @@ def test_layernorm_division_recomputed_equals_division_of_the_stored_tensor(dev,
                                                _hip.ptr(mean), _hip.ptr(rstd), _hip.ptr(s_max), _hip.ptr(got_s),
                                                _hip.ptr(got_q), _hip.ptr(got_qt), M, N, QBv, st), "layernorm_division")
     assert torch.equal(got_q, want_q) and torch.equal(got_qt, want_qt) and got_s.item() == want_s.item() > 0
+
+
+@pytest.mark.parametrize("fp8", ["E4M3", "E5M2"])
+@pytest.mark.parametrize("shape,QBv", [((BS, SL, C), 16), ((48, 352), 32), ((7, 64), 16)])
+def test_fused_silu_mul_from_bf16_equals_quantize_then_fused_forward(dev, fp8, shape, QBv):
+    """One pass over the bf16 gate / up gives the codes and scales of fp8_quantize and everything fp8_silu_mul_forward
+    returns, bit for bit (the last shape has no whole 16 x 16 blocks: it raises like the chain, which needs them for the
+    transposed output)."""
+    rq = _rq()
+    gate, up = rand(71, 1.0, shape).to(dev), rand(72, 1.0, shape).to(dev)
+    if shape[-2] % 16 != 0:
+        with pytest.raises(ValueError):
+            rq.fp8_silu_mul_forward_from_bf16(gate, up, QBv, fp8)
+        return
+    got = rq.fp8_silu_mul_forward_from_bf16(gate, up, QBv, fp8, transpose_output_2d=True)
+    gq, gs = rq.fp8_quantize(gate, QBv, fp8)
+    uq, us = rq.fp8_quantize(up, QBv, fp8)
+    want = (gq, gs, uq, us) + tuple(rq.fp8_silu_mul_forward(gq, gs, uq, us, QBv, transpose_output_2d=True))
+    assert len(got) == len(want) == 9
+    for i, (a, w) in enumerate(zip(got, want)):
+        assert a.shape == w.shape and a.dtype == w.dtype, i
+        assert torch.equal(a.view(torch.uint8) if a.dtype in (E4, E5) else a, w.view(torch.uint8) if w.dtype in (E4, E5) else w), i
