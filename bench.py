@@ -194,7 +194,7 @@ def make_rmsnorm_workload(dev, torch):
 
 def make_cross_entropy_workload(dev, torch):
     """LM-head loss of Llama-2 (vocabulary 32000) on 4 x 2048 tokens, fp32 logits as the reference computes it
-    (coat/activation/liger/cross_entropy.py:399-410).  One step = loss + in-place gradient, i.e. one read and one
+    (coat/activation/liger/cross_entropy.py:396-411).  One step = loss + in-place gradient, i.e. one read and one
     write of the logits: 8 bytes per logit."""
     from coat_amd.activation.liger.cross_entropy import cross_entropy_forward
     BT, V = 8192, 32000
@@ -311,7 +311,7 @@ def make_olmo_workload(dev, torch):
 
 def make_layernorm_workload(dev, torch):
     """Non-parametric LayerNorm on the FP8 block input [8192,4096] -> per-tensor FP8 (+ transpose), and its backward
-    (coat/activation/real_quantization/func_layernorm_noparam.py:193-297), as the OLMo block calls them."""
+    (coat/activation/real_quantization/func_layernorm_noparam.py:188-297), as the OLMo block calls them."""
     import coat_amd.activation.real_quantization as rq
 
     M, N, QB = 8192, 4096, 16

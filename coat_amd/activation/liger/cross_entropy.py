@@ -1,8 +1,8 @@
 """Fused cross-entropy of the LM head: loss and, in place of the logits, their gradient.
-Reference: coat/activation/liger/cross_entropy.py (kernel :24-222, host :240-410).  Same names, arguments, defaults
+Reference: coat/activation/liger/cross_entropy.py (kernel :24-198, host :212-411).  Same names, arguments, defaults
 and return values; the kernel underneath is coat_amd/csrc/cross_entropy.hip.  Two host synchronisations of the
-reference are gone: the count of non-ignored targets stays on the device (reference :262 calls ``.item()``), and the
-"is grad_output exactly 1" test of the backward (reference :304, ``torch.equal``) is made by the kernel itself."""
+reference are gone: the count of non-ignored targets stays on the device (reference :240 calls ``.item()``), and the
+"is grad_output exactly 1" test of the backward (reference :283, ``torch.equal``) is made by the kernel itself."""
 from typing import Optional
 
 import torch
@@ -22,7 +22,7 @@ def _check_input(_input):
 
 def cross_entropy_forward(_input, target, ignore_index, lse_square_scale, label_smoothing, reduction, softcap,
                           return_z_loss):
-    """Returns (loss, z_loss or None, _input); ``_input`` now holds d loss / d logits (reference :240-299)."""
+    """Returns (loss, z_loss or None, _input); ``_input`` now holds d loss / d logits (reference :212-278)."""
     if return_z_loss not in (True, False, 0, 1):
         raise AssertionError(f"return_z_loss must be True or False. Got: {return_z_loss}")
     if reduction not in _REDUCTION:
@@ -31,7 +31,7 @@ def cross_entropy_forward(_input, target, ignore_index, lse_square_scale, label_
     BT, V = _input.shape
     if target.shape != (BT,):
         raise ValueError(f"target must have shape ({BT},), got {tuple(target.shape)}")
-    # unreduced loss, in the logits' dtype as in the reference (:255-259); every row is written by the kernel
+    # unreduced loss, in the logits' dtype as in the reference (:234-238); every row is written by the kernel
     loss_1d = torch.empty(BT, dtype=_input.dtype, device=_input.device)
     z_loss_1d = torch.empty(BT, dtype=_input.dtype, device=_input.device) if return_z_loss else None
     target = target.to(device=_input.device, dtype=torch.int64).contiguous()
@@ -49,7 +49,7 @@ def cross_entropy_forward(_input, target, ignore_index, lse_square_scale, label_
 
 
 def cross_entropy_backward(_input, grad_output):
-    """_input *= grad_output in place (reference :302-325); untouched when grad_output is exactly 1."""
+    """_input *= grad_output in place (reference :281-302); untouched when grad_output is exactly 1."""
     _check_input(_input)
     BT, V = _input.shape
     if grad_output.numel() != 1:
@@ -64,7 +64,7 @@ def cross_entropy_backward(_input, grad_output):
 
 
 class LigerCrossEntropyFunction(torch.autograd.Function):
-    """autograd wrapper with the reference's signature (reference :328-387).  The logits are overwritten by their
+    """autograd wrapper with the reference's signature (reference :305-384).  The logits are overwritten by their
     gradient in the forward pass; the backward only rescales them."""
 
     @staticmethod
@@ -85,7 +85,7 @@ class LigerCrossEntropyFunction(torch.autograd.Function):
 
 
 def liger_fixed_cross_entropy(source, target, num_items_in_batch: int = None, ignore_index: int = -100, **kwargs):
-    """Reference :390-396."""
+    """Reference :387-393."""
     reduction = "sum" if num_items_in_batch is not None else "mean"
     loss, _ = LigerCrossEntropyFunction.apply(source, target, ignore_index, 0.0, 0.0, reduction)
     if reduction == "sum":
@@ -95,7 +95,7 @@ def liger_fixed_cross_entropy(source, target, num_items_in_batch: int = None, ig
 
 def LigerForCausalLMLoss(logits, labels, vocab_size: int, num_items_in_batch: int = None, ignore_index: int = -100,
                          **kwargs):
-    """Shifted next-token loss on fp32 logits (reference :399-410)."""
+    """Shifted next-token loss on fp32 logits (reference :396-411)."""
     logits = logits.float()
     shift_logits = logits[..., :-1, :].contiguous()
     shift_labels = labels[..., 1:].contiguous()

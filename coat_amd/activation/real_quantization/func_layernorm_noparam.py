@@ -1,5 +1,5 @@
 """FP8 LayerNorm without affine parameters, forward / backward.
-Reference: coat/activation/real_quantization/func_layernorm_noparam.py:193-297."""
+Reference: coat/activation/real_quantization/func_layernorm_noparam.py:188-297."""
 import torch
 
 from ... import _hip

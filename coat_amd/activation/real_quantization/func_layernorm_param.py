@@ -1,5 +1,5 @@
 """FP8 LayerNorm with weight and bias, forward / backward.
-Reference: coat/activation/real_quantization/func_layernorm_param.py:258-367."""
+Reference: coat/activation/real_quantization/func_layernorm_param.py:243-367."""
 import torch
 
 from ... import _hip

@@ -1,6 +1,6 @@
 // Softmax cross-entropy of the LM head: per-row loss and, written over the logits, the gradient of the reduced loss.
 //
-// Restates the reference's liger_cross_entropy_kernel (coat/activation/liger/cross_entropy.py:24-222) and
+// Restates the reference's liger_cross_entropy_kernel (coat/activation/liger/cross_entropy.py:24-198) and
 // element_mul_kernel (coat/activation/liger/utils.py) for gfx950.  One block owns one row of V logits:
 //   * V <= 512 * VEC * 16: the row is loaded once into registers (16-byte loads), reduced twice (max, then sum of
 //     exponentials) and overwritten once: 1 read + 1 write of the row, the algorithmic minimum;

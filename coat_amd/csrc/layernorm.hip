@@ -1,8 +1,8 @@
 // FP8 LayerNorm forward / backward for gfx950, without and with affine parameters.
 //
 // Reference: coat/activation/real_quantization/func_layernorm_noparam.py (_layer_norm_fwd_fused :53-115,
-// _layer_norm_bwd_dx_fused :125-190) and func_layernorm_param.py (_layer_norm_fwd_fused :51-125,
-// _layer_norm_bwd_dx_fused :134-226, _fp8_layer_norm_bwd_dwdb :229-255).
+// _layer_norm_bwd_dx_fused :122-185) and func_layernorm_param.py (_layer_norm_fwd_fused :52-119,
+// _layer_norm_bwd_dx_fused :128-209, _fp8_layer_norm_bwd_dwdb :214-240).
 //
 // Same organisation as the RMSNorm kernels: one 256-thread block per row, the dequantized row stays in registers
 // for the mean pass, the variance pass (two-pass variance, as the reference computes it) and the output pass.

@@ -395,7 +395,7 @@ template <int KIND, int WDT> struct RmsNormSource {
 };
 
 // (x - mean[row]) * rstd[row] (* w[col] + b[col]) of k_layernorm_fwd, kept in fp32 as the reference keeps it
-// (coat/activation/real_quantization/func_layernorm_noparam.py:85-100, func_layernorm_param.py:90-108).
+// (coat/activation/real_quantization/func_layernorm_noparam.py:93-113, func_layernorm_param.py:94-119).
 // WMODE: dtype of w and b, or 3 = no affine parameters.
 template <int KIND, int WMODE> struct LayerNormSource {
     static constexpr int kNW = WMODE == 3 ? 1 : (WMODE == kF32 ? 4 : 2);  // 16-byte pieces of 16 weights

@@ -163,7 +163,7 @@ int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtyp
 int coat_fp8_rmsnorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype,
                               const float* rstd, const float* s_max, void* s_out, void* q, void* qt, int64_t M, int64_t N,
                               int QB, void* stream);
-/* The same for coat_fp8_layernorm_forward (rq/func_layernorm_noparam.py:193, rq/func_layernorm_param.py:258; y = NULL
+/* The same for coat_fp8_layernorm_forward (rq/func_layernorm_noparam.py:188, rq/func_layernorm_param.py:243; y = NULL
  * there): y = (x - mean) * rstd (* w + b) in fp32, as the reference keeps it, recomputed per tile.  w_dtype < 0: no affine
  * parameters (w, b NULL). */
 int coat_fp8_layernorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, const void* b,
@@ -185,15 +185,15 @@ int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dty
                               const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
                               float* dw_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream);
 
-/* rq/func_layernorm_noparam.py:193 fp8_layernorm_noparam_forward (kernel :53-115) and rq/func_layernorm_param.py:258
- * fp8_layernorm_param_forward (kernel :51-125): y fp32 [M,N] = (x - mean) * rstd (* w + b); mean, rstd [M] fp32;
+/* rq/func_layernorm_noparam.py:188 fp8_layernorm_noparam_forward (kernel :53-115) and rq/func_layernorm_param.py:243
+ * fp8_layernorm_param_forward (kernel :52-119): y fp32 [M,N] = (x - mean) * rstd (* w + b); mean, rstd [M] fp32;
  * s_row [M] bf16 row scales (max|y| + 1e-10) / fp8max; s_max as above.  w_dtype < 0: no affine parameters (w, b
  * ignored); otherwise w and b share that dtype.  N <= 16384, N % 16 == 0. */
 int coat_fp8_layernorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, const void* b,
                                int w_dtype, float* y, void* s_row, float* mean, float* rstd, float* s_max, int64_t M,
                                int64_t N, int QB, float eps, void* stream);
-/* rq/func_layernorm_noparam.py:250 fp8_layernorm_noparam_backward (kernel :125-190) and
- * rq/func_layernorm_param.py:309 fp8_layernorm_param_backward (kernels :134-226, :229-255): dx bf16 [M,N]; with
+/* rq/func_layernorm_noparam.py:248 fp8_layernorm_noparam_backward (kernel :122-185) and
+ * rq/func_layernorm_param.py:305 fp8_layernorm_param_backward (kernels :128-209, :214-240): dx bf16 [M,N]; with
  * parameters also dw, db [N] in w's dtype through the caller-provided fp32 workspaces dw_partial, db_partial
  * [n_partial, N] (summed in block order; the reference accumulates under a spin lock in w's dtype). */
 int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* w,
@@ -241,19 +241,19 @@ int coat_fp8_adamw_step(void* params, const void* grads, int p_dtype, void* exp_
                         void* exp_avg_sq, float* scale_exp_avg_sq, float beta1, float beta2, float lr, float wd,
                         float eps, int step, int qgroup_size, int64_t numel, int64_t n_scale, void* stream);
 
-/* coat/activation/liger/cross_entropy.py:24-222 liger_cross_entropy_kernel as launched by cross_entropy_forward
- * (:240-299): softmax cross-entropy over x [n_rows, n_cols] (row pitch x_stride elements, fp32 / bf16 / fp16).
+/* coat/activation/liger/cross_entropy.py:24-198 liger_cross_entropy_kernel as launched by cross_entropy_forward
+ * (:212-278): softmax cross-entropy over x [n_rows, n_cols] (row pitch x_stride elements, fp32 / bf16 / fp16).
  * On return x holds the gradient of the reduced loss w.r.t. the logits, loss[row] (and z_loss[row] when z_loss is
  * not NULL) the row's contribution, both in x's dtype; rows whose target equals ignore_index get zeros.
  * target: int64 [n_rows].  reduction: 0 "none", 1 "mean", 2 "sum"; for "mean" the divisor is read from
  * *n_non_ignore (one int64 in device memory: the number of targets != ignore_index), so the host never waits for it
- * (the reference calls .item(), :262).  has_softcap != 0: logits pass through softcap * tanh(x / softcap) first. */
+ * (the reference calls .item(), :240).  has_softcap != 0: logits pass through softcap * tanh(x / softcap) first. */
 int coat_cross_entropy_forward(void* x, int x_dtype, int64_t x_stride, const int64_t* target, void* loss, void* z_loss,
                                const int64_t* n_non_ignore, int64_t n_rows, int64_t n_cols, int64_t ignore_index,
                                float lse_square_scale, float label_smoothing, int reduction, float softcap,
                                int has_softcap, void* stream);
 
-/* coat/activation/liger/cross_entropy.py:302-325 cross_entropy_backward (element_mul_kernel, liger/utils.py):
+/* coat/activation/liger/cross_entropy.py:281-302 cross_entropy_backward (element_mul_kernel, liger/utils.py):
  * x *= *grad_output in place; grad_output is one element of g_dtype in device memory.  The kernel itself returns
  * without touching x when the factor is 1 (the reference compares on the host with torch.equal, a synchronisation). */
 int coat_cross_entropy_scale_grad(void* x, int x_dtype, int64_t x_stride, const void* grad_output, int g_dtype,

@@ -312,7 +312,7 @@ def fp8_rmsnorm_backward(q, s, g, w, rstd, QB, accumulate=torch.float64):
 
 # ----------------------------------------------------------------------------- LayerNorm
 def layernorm_forward_value(q, s, QB, eps, w=None, b=None, accumulate=torch.float32):
-    """rq/func_layernorm_noparam.py:86-104 / rq/func_layernorm_param.py:85-107: x = dequant; mean = sum(x)/N;
+    """rq/func_layernorm_noparam.py:86-113 / rq/func_layernorm_param.py:87-119: x = dequant; mean = sum(x)/N;
     var = sum((x-mean)^2)/N; rstd = 1/sqrt(var+eps); y = (x-mean)*rstd (* w + b), all fp32."""
     x = _dequant32(q, s, QB)
     N = x.shape[1]
@@ -327,7 +327,7 @@ def layernorm_forward_value(q, s, QB, eps, w=None, b=None, accumulate=torch.floa
 
 
 def fp8_layernorm_forward(q, s, QB, eps, w=None, b=None, accumulate=torch.float32):
-    """rq/func_layernorm_noparam.py:193-247 / rq/func_layernorm_param.py:258-306: the normalised tensor stays fp32
+    """rq/func_layernorm_noparam.py:188-245 / rq/func_layernorm_param.py:243-302: the normalised tensor stays fp32
     (:205), row scale (max|y|+1e-10)/fp8max stored bf16 (:106-112), max over rows, division+transpose of the fp32 y."""
     y, mean, rstd = layernorm_forward_value(q, s, QB, eps, w, b, accumulate)
     s_row = ((y.abs().amax(dim=1) + SCALE_MIN_THRES) / FP8_MAX_VALUE[q.dtype]).to(torch.bfloat16)
@@ -336,7 +336,7 @@ def fp8_layernorm_forward(q, s, QB, eps, w=None, b=None, accumulate=torch.float3
 
 
 def fp8_layernorm_backward(q, s, g, mean, rstd, QB, w=None, accumulate=torch.float64):
-    """rq/func_layernorm_noparam.py:164-190 / rq/func_layernorm_param.py:186-226, :229-255:
+    """rq/func_layernorm_noparam.py:160-185 / rq/func_layernorm_param.py:178-209, :214-240:
     wdy = w*dy (dy without parameters); c1 = sum(xhat*wdy)/N; c2 = sum(wdy)/N; dx = (wdy - (xhat*c1 + c2))*rstd -> bf16;
     dw = sum_rows(dy*xhat), db = sum_rows(dy) (the reference accumulates them under a lock in w's dtype; stated here is
     the float64 sum rounded once)."""
