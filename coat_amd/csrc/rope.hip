@@ -1,7 +1,7 @@
 // Rotary position embedding for the bf16 attention of the decoder layers, forward and backward in one pass each.
 //
 // The reference applies RoPE with separate torch kernels (transformers' apply_rotary_pos_emb as called from
-// coat/models/coat_llama.py:1029-1030; olmo's RotaryEmbedding from coat/models/coat_olmo.py:862-863): two multiplies, a
+// coat/models/coat_llama.py:1029-1030; olmo's RotaryEmbedding from coat/models/coat_olmo.py:860-861): two multiplies, a
 // negate, a concatenation and an add per tensor and direction, each a full pass over q and k.  Here one streaming
 // kernel reads x once and writes the rotated tensor once; the backward pass is the same kernel with the angle negated.
 //   x, y: bf16 [rows, heads, head_dim] (rows = batch * seq, contiguous), "half" layout: element d pairs with d + head_dim/2

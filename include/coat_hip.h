@@ -143,7 +143,7 @@ int coat_fp8_silu_mul_forward_bf16(const void* gate, const void* up, int fp8, vo
  * scales for the format fp8_out (the per-tensor division that follows is coat_fp8_division).
  * Row pitches in elements, 0 = contiguous: in_pitch / s_pitch for gate, up and their scales when they are the two column
  * halves of a fused projection's output (coat/models/coat_olmo.py:520-523 chunks and copies them), y_pitch (backward
- * only) for y_gate / y_up written side by side into one [M, 2N] tensor (coat_olmo.py:599 concatenates them). */
+ * only) for y_gate / y_up written side by side into one [M, 2N] tensor (coat_olmo.py:600 concatenates them). */
 int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, const void* up, const void* s_up, const void* silu,
                                const void* s_silu, int fp8_in, int s_dtype, const void* g, void* y_gate,
                                float* s_max_gate, void* y_up, float* s_max_up, int fp8_out, int64_t M, int64_t N,
@@ -203,7 +203,7 @@ int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_d
 
 /* Rotary position embedding of the bf16 attention (no single counterpart in the reference, which applies it with
  * several torch kernels: transformers' apply_rotary_pos_emb as called at coat/models/coat_llama.py:1029-1030, olmo's
- * RotaryEmbedding at coat/models/coat_olmo.py:862-863).  x, y bf16 [rows, heads, head_dim], rows = batch * seq;
+ * RotaryEmbedding at coat/models/coat_olmo.py:860-861).  x, y bf16 [rows, heads, head_dim], rows = batch * seq;
  * cos_tab / sin_tab fp32 [n_pos, head_dim / 2]; pos int64 [rows] or NULL (position = row % seq_len);
  * y1 = x1 cos - x2 sin, y2 = x2 cos + x1 sin on the (d, d + head_dim/2) pairs; inverse != 0 negates the angle, which
  * is the backward pass.  head_dim % 16 == 0.  x_pitch / y_pitch: row pitches in elements, 0 = contiguous; a multiple

@@ -84,7 +84,7 @@ def test_fp8_quantize_transpose_bit_exact(dev, dtype, fp8, QB, M, N):
         x[:32, :128] = special_x(dtype)
     (q, s), (qt, st) = rq.fp8_quantize_transpose(x.to(dev), QB, fp8)
     (wq, ws), (wqt, wst) = R.fp8_quantize_transpose(x, QB, fp8)
-    if QB == 128:  # the reference's own test calls it with fp32 scales (tests/test_fp8_quantize.py:70)
+    if QB == 128:  # the reference's own test calls it with fp32 scales (tests/test_fp8_quantize.py:57)
         (q32, s32), (qt32, st32) = rq.fp8_quantize_transpose(x.to(dev), QB, fp8, scale_dtype=torch.float32)
         (_, ws32), (_, wst32) = R.fp8_quantize_transpose(x, QB, fp8, scale_dtype=torch.float32)
         assert torch.equal(s32.cpu(), ws32) and torch.equal(st32.cpu(), wst32) and eq_bytes(q32, q) and eq_bytes(qt32, qt)
