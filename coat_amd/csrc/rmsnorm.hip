@@ -11,6 +11,8 @@
 // partial row; a second kernel sums the partials in block order.
 #include <math.h>
 
+#include <atomic>
+
 #include "coat_host.h"
 #include "norm_common.h"
 
@@ -178,18 +180,10 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
     return coat_launch_status();
 }
 
-extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
-                                         const void* dy2, const void* dy3, const void* w, int w_dtype, const float* rstd,
-                                         void* dx, void* dw, float* dw_partial, int n_partial, int64_t M, int64_t N,
-                                         int QB, void* stream) {
-    if (int e = rms_check(M, N, QB)) return e;
-    if (M * N == 0) return COAT_OK;
-    if (!x || !s_x || !dy || !w || !rstd || !dx || !dw || !dw_partial || n_partial <= 0) return COAT_EINVAL;
-    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(dy) || !coat_aligned16(dx) || !coat_aligned16(dw_partial) ||
-        !coat_aligned16(dy2) || !coat_aligned16(dy3))
-        return COAT_EALIGN;
-    if (dy3 && !dy2) return COAT_EINVAL;
-    hipStream_t st = (hipStream_t)stream;
+// Shared by the two backward entry points: dx kernel on min(n_partial, M) blocks, then the column sum of their partial rows.
+static int rms_backward_launch(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
+                               const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
+                               float* dw_partial, int64_t n_partial, int64_t M, int64_t N, int QB, hipStream_t st) {
     const int64_t grid = n_partial < M ? n_partial : M;
     RMS_DISPATCH(k_rmsnorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB)
     if (int e = coat_launch_status()) return e;
@@ -200,4 +194,66 @@ extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x
         default: hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
     }
     return coat_launch_status();
+}
+
+static int rms_backward_check(const void* x, const void* s_x, const void* dy, const void* dy2, const void* dy3, const void* w,
+                              const float* rstd, void* dx, void* dw) {
+    if (!x || !s_x || !dy || !w || !rstd || !dx || !dw) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(dy) || !coat_aligned16(dx) || !coat_aligned16(dy2) ||
+        !coat_aligned16(dy3))
+        return COAT_EALIGN;
+    if (dy3 && !dy2) return COAT_EINVAL;
+    return COAT_OK;
+}
+
+extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
+                                         const void* dy2, const void* dy3, const void* w, int w_dtype, const float* rstd,
+                                         void* dx, void* dw, float* dw_partial, int n_partial, int64_t M, int64_t N,
+                                         int QB, void* stream) {
+    if (int e = rms_check(M, N, QB)) return e;
+    if (M * N == 0) return COAT_OK;
+    if (!dw_partial || n_partial <= 0) return COAT_EINVAL;
+    if (int e = rms_backward_check(x, s_x, dy, dy2, dy3, w, rstd, dx, dw)) return e;
+    if (!coat_aligned16(dw_partial)) return COAT_EALIGN;
+    return rms_backward_launch(x, fp8, s_x, s_dtype, dy, dy2, dy3, w, w_dtype, rstd, dx, dw, dw_partial, n_partial, M, N, QB,
+                               (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------------------------------------ no allocation
+// The weight-gradient partial rows of the entry point below live in this array instead of a caller-provided workspace:
+// 16 MiB per GPU, held from the moment the library is loaded until the process ends.  In host code `dw_scratch` is only a
+// handle for hipGetSymbolAddress; the device address is looked up once per device (each GPU has its own copy of the array at
+// its own address) and only that pointer is ever passed to a kernel.
+constexpr int64_t kDwScratchFloats = (int64_t)COAT_RMSNORM_STATIC_PARTIALS * COAT_RMSNORM_STATIC_FULL_N;
+static __device__ __align__(256) float dw_scratch[kDwScratchFloats];
+static std::atomic<float*> dw_scratch_ptr[kCoatMaxDevices];
+
+static int dw_scratch_address(float** out) {
+    const int dev = coat_device_index();
+    if (dev < 0) return COAT_EINVAL;
+    float* p = dw_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        // the current device is `dev`: the address returned is that device's copy.  Two threads racing here store the same value.
+        hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(dw_scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return COAT_EINVAL;
+        dw_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return COAT_OK;
+}
+
+extern "C" int coat_fp8_rmsnorm_backward_static(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
+                                                const void* dy2, const void* dy3, const void* w, int w_dtype,
+                                                const float* rstd, void* dx, void* dw, int64_t M, int64_t N, int QB,
+                                                void* stream) {
+    if (int e = rms_check(M, N, QB)) return e;  // N > 16384 is beyond what the scratch rows (and the kernels) hold
+    if (M * N == 0) return COAT_OK;
+    if (int e = rms_backward_check(x, s_x, dy, dy2, dy3, w, rstd, dx, dw)) return e;
+    float* partial = nullptr;
+    if (int e = dw_scratch_address(&partial)) return e;
+    // every block writes its whole partial row and the column sum reads only the rows of this launch's blocks, so
+    // nothing has to be cleared between calls
+    return rms_backward_launch(x, fp8, s_x, s_dtype, dy, dy2, dy3, w, w_dtype, rstd, dx, dw, partial,
+                               coat_rmsnorm_static_partials(N), M, N, QB, (hipStream_t)stream);
 }

@@ -3,7 +3,9 @@
  * Every entry point
  *   - takes raw device pointers, sizes, small enums and the HIP stream to launch on
  *     (`stream` is a hipStream_t passed as void*; NULL is the default stream);
- *   - allocates nothing, frees nothing, keeps no global state, never synchronises the host;
+ *   - allocates nothing, frees nothing and never synchronises the host; the only state kept between calls is per-device
+ *     and idempotent (atomic flags "this kernel's LDS limit has been raised", the cached CU count, the address of the
+ *     static scratch array of coat_fp8_rmsnorm_backward_static), so entry points may be called from several host threads;
  *   - returns COAT_OK (0), a negative COAT_E* code for a rejected argument, or the positive
  *     hipError_t of a failed launch.
  * Tensors are row-major and contiguous.  "pg" = per-group scales, one per 1 x QB group along the
@@ -184,6 +186,22 @@ int coat_fp8_product_division(const void* a, const void* s_a, int sa_dtype, cons
 int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
                               const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
                               float* dw_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream);
+/* No counterpart in the reference.  For callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): coat_fp8_rmsnorm_backward without the workspace argument.  The partial rows live in a
+ * device array inside the library, COAT_RMSNORM_STATIC_PARTIALS x COAT_RMSNORM_STATIC_FULL_N floats (16 MiB per GPU, held
+ * until the process ends); the call allocates and frees nothing.  It uses coat_rmsnorm_static_partials(N) partial rows
+ * (512 up to N = 8192, 256 beyond), so dx and dw equal those of coat_fp8_rmsnorm_backward called with that n_partial.
+ * N > 16384 is rejected with COAT_ESHAPE, as everywhere.  All calls on one GPU share the array: calls that overlap on one
+ * GPU (two streams, two threads) race on it; calls on one stream are ordered and need no clearing in between. */
+#define COAT_RMSNORM_STATIC_PARTIALS 512
+#define COAT_RMSNORM_STATIC_FULL_N 8192
+static inline int coat_rmsnorm_static_partials(int64_t N) {
+    const int64_t rows = N > 0 ? ((int64_t)COAT_RMSNORM_STATIC_PARTIALS * COAT_RMSNORM_STATIC_FULL_N) / N : 0;
+    return (int)(rows < COAT_RMSNORM_STATIC_PARTIALS ? rows : COAT_RMSNORM_STATIC_PARTIALS);
+}
+int coat_fp8_rmsnorm_backward_static(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
+                                     const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
+                                     int64_t M, int64_t N, int QB, void* stream);
 
 /* rq/func_layernorm_noparam.py:188 fp8_layernorm_noparam_forward (kernel :53-115) and rq/func_layernorm_param.py:243
  * fp8_layernorm_param_forward (kernel :52-119): y fp32 [M,N] = (x - mean) * rstd (* w + b); mean, rstd [M] fp32;
