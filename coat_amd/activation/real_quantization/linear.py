@@ -37,7 +37,9 @@ def fp8matmul(a, b, output_quantize, scale_a, scale_b, QB, bias=None, stochastic
         if s.numel() != 1:
             raise ValueError("fp8matmul takes per-tensor (single element) scales")
     scale_a = scale_a if scale_a.is_cuda else scale_a.to(a.device)
-    scale_b = scale_b.to(device=a.device, dtype=scale_a.dtype)
+    scale_b = scale_b if scale_b.is_cuda else scale_b.to(a.device)
+    # each scale is read in its own dtype and the two are multiplied in fp32 (reference linear.py:123-125): an fp32
+    # weight scale next to a bf16 activation scale is used with all its bits
     if bias is not None:
         bias = _hip.dense(bias)
     if output_quantize:
@@ -49,7 +51,7 @@ def fp8matmul(a, b, output_quantize, scale_a, scale_b, QB, bias=None, stochastic
         scale_c, kind = None, 0
     _hip.check(_hip.lib().coat_fp8_gemm(
         _hip.ptr(a), _hip.fp8(a.dtype), _hip.ptr(bn), _hip.fp8(bn.dtype), _hip.ptr(c), _hip.ptr(scale_c), kind,
-        _hip.ptr(scale_a), _hip.ptr(scale_b), _hip.dt(scale_a), _hip.ptr(bias), _hip.dt(bias) if bias is not None else 0,
+        _hip.ptr(scale_a), _hip.dt(scale_a), _hip.ptr(scale_b), _hip.dt(scale_b), _hip.ptr(bias), _hip.dt(bias) if bias is not None else 0,
         M, N, K, QB if output_quantize else 0, _hip.stream(a.device)), "fp8matmul")
     if batch is not None:
         c = c.reshape(batch, -1, N)

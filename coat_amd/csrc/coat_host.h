@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/coat_hip.h"
 
 // Status of the launch just issued: COAT_OK or the (positive) hipError_t.
@@ -21,14 +23,16 @@ static inline int coat_device_index() {
     return dev;
 }
 // Raises a kernel's dynamic-LDS limit once per device (the attribute is per device, the kernels are templates: each
-// instantiation passes its own flag array).
-template <typename K> static inline int coat_allow_lds(K kernel, int bytes, bool* done_per_device) {
+// instantiation passes its own flag array).  The flags are atomics: host threads may enter an entry point together, and the
+// worst that two of them can do is set the same attribute twice.
+typedef std::atomic<bool> coat_device_flags[kCoatMaxDevices];
+template <typename K> static inline int coat_allow_lds(K kernel, int bytes, std::atomic<bool>* done_per_device) {
     const int dev = coat_device_index();
     if (dev < 0) return COAT_EINVAL;
-    if (!done_per_device[dev]) {
+    if (!done_per_device[dev].load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         if (e != hipSuccess) return (int)e;
-        done_per_device[dev] = true;
+        done_per_device[dev].store(true, std::memory_order_release);
     }
     return COAT_OK;
 }

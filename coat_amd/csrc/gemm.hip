@@ -42,7 +42,7 @@ struct GemmArgs {
     const void* sa;     // per-tensor scales, one element each
     const void* sb;
     const void* bias;   // [N] or nullptr
-    int s_dt, bias_dt;
+    int sa_dt, sb_dt, bias_dt;
     int M, N, K;
     int tiles_m, tiles_n;
 };
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
-    const float scale = load_rt_f32(G.sa, 0, G.s_dt) * load_rt_f32(G.sb, 0, G.s_dt);
+    const float scale = load_rt_f32(G.sa, 0, G.sa_dt) * load_rt_f32(G.sb, 0, G.sb_dt);
     if (EPI != kEpiBf16) enable_fp8_saturation();
     const int half = lane >> 5;
     constexpr bool vec16 = VEC16;  // rows of C start 16-byte aligned (N % 8 == 0): 16-byte stores
@@ -392,8 +392,8 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
 using namespace coat;
 
 extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
-                             const void* scale_a, const void* scale_b, int s_dtype, const void* bias, int bias_dtype,
-                             int64_t M, int64_t N, int64_t K, int QB, void* stream) {
+                             const void* scale_a, int sa_dtype, const void* scale_b, int sb_dtype, const void* bias,
+                             int bias_dtype, int64_t M, int64_t N, int64_t K, int QB, void* stream) {
     if (M < 0 || N < 0 || K < 0) return COAT_EINVAL;
     if (M * N == 0) return COAT_OK;
     if (!a || !b || !c || !scale_a || !scale_b) return COAT_EINVAL;
@@ -404,30 +404,31 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     if ((fmt_a != COAT_E4M3 && fmt_a != COAT_E5M2) || (fmt_b != COAT_E4M3 && fmt_b != COAT_E5M2)) return COAT_EINVAL;
     if (out_kind < 0 || out_kind > 2) return COAT_EINVAL;
     if (out_kind != 0 && (QB != 16 || N % 16 != 0 || !c_scale)) return COAT_ESHAPE;
-    if (s_dtype < 0 || s_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return COAT_EDTYPE;
+    if (sa_dtype < 0 || sa_dtype > 2 || sb_dtype < 0 || sb_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return COAT_EDTYPE;
     GemmArgs G;
     G.A = (const uint8_t*)a; G.B = (const uint8_t*)b; G.C = c; G.Cs = c_scale;
-    G.sa = scale_a; G.sb = scale_b; G.bias = bias; G.s_dt = s_dtype; G.bias_dt = bias_dtype;
+    G.sa = scale_a; G.sb = scale_b; G.bias = bias; G.sa_dt = sa_dtype; G.sb_dt = sb_dtype; G.bias_dt = bias_dtype;
     G.M = (int)M; G.N = (int)N; G.K = (int)K;
     G.tiles_m = (int)((M + BM - 1) / BM);
     G.tiles_n = (int)((N + BN - 1) / BN);
     const int ntiles = G.tiles_m * G.tiles_n;
     // persistent grid: one block per CU (the block's LDS ring takes a whole CU's LDS); CU count cached per device
-    static int n_cu_dev[kCoatMaxDevices] = {};
+    static std::atomic<int> n_cu_dev[kCoatMaxDevices];
     const int dev = coat_device_index();
     if (dev < 0) return COAT_EINVAL;
-    if (n_cu_dev[dev] == 0) {
+    int n_cu = n_cu_dev[dev].load(std::memory_order_relaxed);
+    if (n_cu == 0) {
         int v = 0;
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 8) return COAT_EINVAL;
-        n_cu_dev[dev] = v & ~7;
+        n_cu = v & ~7;
+        n_cu_dev[dev].store(n_cu, std::memory_order_relaxed);
     }
-    const int n_cu = n_cu_dev[dev];
     const int grid = min(((ntiles + 7) / 8) * 8, n_cu);
     const size_t lds_bytes = kLdsBytes;
     hipStream_t st = (hipStream_t)stream;
 #define GEMM_LAUNCH_V(FA, FB, EP, V16)                                                                                  \
     {                                                                                                              \
-        static bool lds_ok[kCoatMaxDevices] = {};                                                                  \
+        static coat_device_flags lds_ok;                                                                         \
         if (int e = coat_allow_lds(k_fp8_gemm<FA, FB, EP, V16>, (int)lds_bytes, lds_ok)) return e;                 \
         hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, V16>), dim3(grid), dim3(512), lds_bytes, st, G); \
         return coat_launch_status();                                                                               \

@@ -983,7 +983,7 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
     DISPATCH_XDT(x_dtype, DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                 \
         constexpr int kLds = TMV * (TNV + 1) * 4;                                                                    \
         if (kLds > 65536) {                                                                                          \
-            static bool lds_ok[kCoatMaxDevices] = {};                                                                \
+            static coat_device_flags lds_ok;                                                                       \
             if (int e = coat_allow_lds(k_quantize_transpose<XDT, SDT, KIND, QBV, TMV, TNV>, kLds, lds_ok)) return e; \
         }                                                                                                            \
         hipLaunchKernelGGL((k_quantize_transpose<XDT, SDT, KIND, QBV, TMV, TNV>), dim3((unsigned)blocks), dim3(256), \

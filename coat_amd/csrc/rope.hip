@@ -5,7 +5,8 @@
 // negate, a concatenation and an add per tensor and direction, each a full pass over q and k.  Here one streaming
 // kernel reads x once and writes the rotated tensor once; the backward pass is the same kernel with the angle negated.
 //   x, y: bf16 [rows, heads, head_dim] (rows = batch * seq, contiguous), "half" layout: element d pairs with d + head_dim/2
-//   cos_tab, sin_tab: fp32 [n_pos, head_dim/2];  position of a row = pos[row] if pos is given, else row % seq_len
+//   cos_tab, sin_tab: fp32 [n_pos, head_dim/2];  position of a row = pos[row] if pos is given, else row % seq_len;
+//   a position outside the tables (only possible with pos) gets its angle p * theta^(-2d/head_dim) computed in the kernel
 //   y1 = x1 cos - x2 sin,  y2 = x2 cos + x1 sin   (inverse: sin -> -sin), computed in fp32, rounded once to bf16.
 #include "coat_device.h"
 #include "coat_host.h"
@@ -14,8 +15,9 @@ namespace coat {
 
 __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab,
-                                                    const int64_t* __restrict__ pos, int64_t rows, int seq_len, int heads,
-                                                    int head_dim, float sign, int64_t x_pitch, int64_t y_pitch) {
+                                                    int64_t n_pos, float theta, const int64_t* __restrict__ pos,
+                                                    int64_t rows, int seq_len, int heads, int head_dim, float sign,
+                                                    int64_t x_pitch, int64_t y_pitch) {
     const int half = head_dim >> 1;
     const int cpr = half >> 3;                      // 16-byte chunks per half row
     const int64_t total = rows * heads * cpr;       // one job = 8 pairs
@@ -27,11 +29,23 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
         const int head = (int)(rh - row * heads);
         const uint16_t* src = x + row * x_pitch + head * head_dim + c * 8;
         const uint4 a = *(const uint4*)src, b = *(const uint4*)(src + half);
-        const float4* ct = (const float4*)(cos_tab + p * half + c * 8);
-        const float4* st = (const float4*)(sin_tab + p * half + c * 8);
-        const float4 c0 = ct[0], c1 = ct[1], s0 = st[0], s1 = st[1];
-        const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-        const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        float cs[8], sn[8];
+        if (p >= 0 && p < n_pos) {
+            const float4* ct = (const float4*)(cos_tab + p * half + c * 8);
+            const float4* st = (const float4*)(sin_tab + p * half + c * 8);
+            const float4 c0 = ct[0], c1 = ct[1], s0 = st[0], s1 = st[1];
+            cs[0] = c0.x; cs[1] = c0.y; cs[2] = c0.z; cs[3] = c0.w; cs[4] = c1.x; cs[5] = c1.y; cs[6] = c1.z; cs[7] = c1.w;
+            sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+        } else {
+            // off the tables: the table's own formula, angle = float(p) * (1 / theta^(2d / head_dim)), never an out-of-bounds read
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float inv_freq = 1.0f / powf(theta, (float)(2 * (c * 8 + k)) / (float)head_dim);
+                const float ang = (float)p * inv_freq;
+                cs[k] = cosf(ang);
+                sn[k] = sinf(ang);
+            }
+        }
         const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
         uint32_t o1[4], o2[4];
 #pragma unroll
@@ -51,10 +65,11 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
 
 using namespace coat;
 
-extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, const int64_t* pos,
-                              int64_t rows, int seq_len, int heads, int head_dim, int inverse, int64_t x_pitch,
-                              int64_t y_pitch, void* stream) {
-    if (rows < 0 || heads <= 0 || head_dim <= 0 || seq_len <= 0) return COAT_EINVAL;
+extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, int64_t n_pos, float theta,
+                              const int64_t* pos, int64_t rows, int seq_len, int heads, int head_dim, int inverse,
+                              int64_t x_pitch, int64_t y_pitch, void* stream) {
+    if (rows < 0 || heads <= 0 || head_dim <= 0 || seq_len <= 0 || n_pos <= 0 || !(theta > 0.0f)) return COAT_EINVAL;
+    if (!pos && seq_len > n_pos) return COAT_ESHAPE;  // positions 0 .. seq_len-1 must all be in the tables
     if (head_dim % 16 != 0) return COAT_ESHAPE;  // 8 pairs per lane
     // row pitches in elements (0 = contiguous): x or y may be a column slice of a wider tensor (a fused q/k/v projection)
     const int64_t width = (int64_t)heads * head_dim;
@@ -68,6 +83,6 @@ extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, cons
     int64_t blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;
     hipLaunchKernelGGL(k_rope_bf16, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
-                       (uint16_t*)y, cos_tab, sin_tab, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f, x_pitch, y_pitch);
+                       (uint16_t*)y, cos_tab, sin_tab, n_pos, theta, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f, x_pitch, y_pitch);
     return coat_launch_status();
 }

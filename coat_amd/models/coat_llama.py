@@ -372,27 +372,29 @@ class _FusedRoPE(torch.autograd.Function):
     (``coat_rope_bf16``; the backward pass is the rotation by the negated angle)."""
 
     @staticmethod
-    def forward(ctx, x, cos_tab, sin_tab, pos, heads, head_dim):
+    def forward(ctx, x, cos_tab, sin_tab, pos, heads, head_dim, theta):
         from .. import _hip
         B, S, _ = x.shape
         x = _hip.dense(x)
         y = torch.empty_like(x)
-        _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(x), _hip.ptr(y), _hip.ptr(cos_tab), _hip.ptr(sin_tab), _hip.ptr(pos),
-                                             B * S, S, heads, head_dim, 0, 0, 0, _hip.stream(x.device)), "rope forward")
+        _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(x), _hip.ptr(y), _hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0],
+                                             theta, _hip.ptr(pos), B * S, S, heads, head_dim, 0, 0, 0,
+                                             _hip.stream(x.device)), "rope forward")
         ctx.save_for_backward(cos_tab, sin_tab, pos)
-        ctx.dims = (B, S, heads, head_dim)
+        ctx.dims = (B, S, heads, head_dim, theta)
         return y.view(B, S, heads, head_dim).transpose(1, 2)
 
     @staticmethod
     def backward(ctx, g):
         from .. import _hip
         cos_tab, sin_tab, pos = ctx.saved_tensors
-        B, S, heads, head_dim = ctx.dims
+        B, S, heads, head_dim, theta = ctx.dims
         g = _hip.dense(g.transpose(1, 2).to(torch.bfloat16))  # physically [B, S, heads, head_dim]
         dx = torch.empty_like(g)
-        _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(g), _hip.ptr(dx), _hip.ptr(cos_tab), _hip.ptr(sin_tab), _hip.ptr(pos),
-                                             B * S, S, heads, head_dim, 1, 0, 0, _hip.stream(g.device)), "rope backward")
-        return dx.view(B, S, heads * head_dim), None, None, None, None, None
+        _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(g), _hip.ptr(dx), _hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0],
+                                             theta, _hip.ptr(pos), B * S, S, heads, head_dim, 1, 0, 0,
+                                             _hip.stream(g.device)), "rope backward")
+        return dx.view(B, S, heads * head_dim), None, None, None, None, None, None
 
 
 class _FusedQKVRoPE(torch.autograd.Function):
@@ -402,7 +404,7 @@ class _FusedQKVRoPE(torch.autograd.Function):
     neither the ``.contiguous()`` copies of the slices nor the concatenation of the three gradients are needed."""
 
     @staticmethod
-    def forward(ctx, qkv, cos_tab, sin_tab, heads, kv_heads, head_dim):
+    def forward(ctx, qkv, cos_tab, sin_tab, heads, kv_heads, head_dim, theta):
         from .. import _hip
         B, S, W = qkv.shape
         Dq, Dkv = heads * head_dim, kv_heads * head_dim
@@ -412,12 +414,13 @@ class _FusedQKVRoPE(torch.autograd.Function):
         q = torch.empty((B, S, Dq), dtype=qkv.dtype, device=qkv.device)
         k = torch.empty((B, S, Dkv), dtype=qkv.dtype, device=qkv.device)
         lib, st = _hip.lib(), _hip.stream(qkv.device)
-        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, :Dq]), _hip.ptr(q), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
-                                      B * S, S, heads, head_dim, 0, W, 0, st), "rope forward (q of qkv)")
-        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, Dq:Dq + Dkv]), _hip.ptr(k), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
-                                      B * S, S, kv_heads, head_dim, 0, W, 0, st), "rope forward (k of qkv)")
+        tabs = (_hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0], theta, None)
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, :Dq]), _hip.ptr(q), *tabs, B * S, S, heads, head_dim, 0, W, 0, st),
+                   "rope forward (q of qkv)")
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, Dq:Dq + Dkv]), _hip.ptr(k), *tabs, B * S, S, kv_heads, head_dim, 0, W,
+                                      0, st), "rope forward (k of qkv)")
         ctx.save_for_backward(cos_tab, sin_tab)
-        ctx.dims = (B, S, heads, kv_heads, head_dim)
+        ctx.dims = (B, S, heads, kv_heads, head_dim, theta)
         v = qkv[..., Dq + Dkv:].view(B, S, kv_heads, head_dim).transpose(1, 2)
         return (q.view(B, S, heads, head_dim).transpose(1, 2), k.view(B, S, kv_heads, head_dim).transpose(1, 2), v)
 
@@ -425,7 +428,7 @@ class _FusedQKVRoPE(torch.autograd.Function):
     def backward(ctx, gq, gk, gv):
         from .. import _hip
         cos_tab, sin_tab = ctx.saved_tensors
-        B, S, heads, kv_heads, head_dim = ctx.dims
+        B, S, heads, kv_heads, head_dim, theta = ctx.dims
         Dq, Dkv = heads * head_dim, kv_heads * head_dim
         W = Dq + 2 * Dkv
         gq = _hip.dense(gq.transpose(1, 2).to(torch.bfloat16))  # physically [B, S, heads, head_dim]
@@ -433,19 +436,20 @@ class _FusedQKVRoPE(torch.autograd.Function):
         dqkv = torch.empty((B, S, W), dtype=torch.bfloat16, device=gq.device)
         flat = dqkv.view(B * S, W)
         lib, st = _hip.lib(), _hip.stream(gq.device)
-        _hip.check(lib.coat_rope_bf16(_hip.ptr(gq), _hip.ptr(flat[:, :Dq]), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
-                                      B * S, S, heads, head_dim, 1, 0, W, st), "rope backward (q of qkv)")
-        _hip.check(lib.coat_rope_bf16(_hip.ptr(gk), _hip.ptr(flat[:, Dq:Dq + Dkv]), _hip.ptr(cos_tab), _hip.ptr(sin_tab), None,
-                                      B * S, S, kv_heads, head_dim, 1, 0, W, st), "rope backward (k of qkv)")
+        tabs = (_hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0], theta, None)
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(gq), _hip.ptr(flat[:, :Dq]), *tabs, B * S, S, heads, head_dim, 1, 0, W, st),
+                   "rope backward (q of qkv)")
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(gk), _hip.ptr(flat[:, Dq:Dq + Dkv]), *tabs, B * S, S, kv_heads, head_dim, 1, 0,
+                                      W, st), "rope backward (k of qkv)")
         dqkv[..., Dq + Dkv:].copy_(gv.transpose(1, 2).reshape(B, S, Dkv))
-        return dqkv, None, None, None, None, None
+        return dqkv, None, None, None, None, None, None
 
 
 def fused_qkv_rotary(qkv, heads, kv_heads, head_dim, theta):
     """RoPE on the q and k parts of a fused projection output qkv [B, S, (heads + 2 kv_heads) * head_dim] (bf16, GPU);
     returns (q [B, heads, S, hd], k [B, kv_heads, S, hd], v [B, kv_heads, S, hd])."""
     cos_tab, sin_tab = rotary_tables(qkv.shape[1], head_dim, theta, qkv.device)
-    return _FusedQKVRoPE.apply(qkv, cos_tab, sin_tab, heads, kv_heads, head_dim)
+    return _FusedQKVRoPE.apply(qkv, cos_tab, sin_tab, heads, kv_heads, head_dim, float(theta))
 
 
 def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=None):
@@ -457,8 +461,9 @@ def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=Non
     else:
         n_pos = max(int(max_positions or 0), S)
         cos_tab, sin_tab = rotary_tables(n_pos, head_dim, theta, x.device)
-        pos = position_ids.expand(B, S).reshape(-1).to(torch.int64).clamp(0, n_pos - 1).contiguous()
-    return _FusedRoPE.apply(x, cos_tab, sin_tab, pos, heads, head_dim)
+        # positions beyond the table are not clamped: the kernel computes their angles itself (no read outside the table)
+        pos = position_ids.expand(B, S).reshape(-1).to(torch.int64).contiguous()
+    return _FusedRoPE.apply(x, cos_tab, sin_tab, pos, heads, head_dim, float(theta))
 
 
 class LlamaSdpaAttentionWithoutLinear(nn.Module):

@@ -124,7 +124,10 @@ class CoatAdamW(Optimizer):
 
         state = defaultdict(dict)
         for k, v in state_dict["state"].items():
-            state[id_map[k]] = place(id_map[k], v) if k in id_map else v
+            if k in id_map:
+                state[id_map[k]] = place(id_map[k], v)
+            else:  # a key outside the parameter mapping is kept as it is (torch.optim.Optimizer.load_state_dict does the same)
+                state[k] = v
         for g, s in zip(groups, saved_groups):
             s["params"] = g["params"]
         self.__setstate__({"state": state, "param_groups": saved_groups})

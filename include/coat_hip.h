@@ -222,13 +222,15 @@ int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_d
 /* Rotary position embedding of the bf16 attention (no single counterpart in the reference, which applies it with
  * several torch kernels: transformers' apply_rotary_pos_emb as called at coat/models/coat_llama.py:1029-1030, olmo's
  * RotaryEmbedding at coat/models/coat_olmo.py:860-861).  x, y bf16 [rows, heads, head_dim], rows = batch * seq;
- * cos_tab / sin_tab fp32 [n_pos, head_dim / 2]; pos int64 [rows] or NULL (position = row % seq_len);
+ * cos_tab / sin_tab fp32 [n_pos, head_dim / 2] holding cos / sin of p * theta^(-2d / head_dim); pos int64 [rows] or NULL
+ * (position = row % seq_len, seq_len <= n_pos); a pos[row] outside [0, n_pos) is never used as a table index: the kernel
+ * computes that row's angles from theta itself;
  * y1 = x1 cos - x2 sin, y2 = x2 cos + x1 sin on the (d, d + head_dim/2) pairs; inverse != 0 negates the angle, which
  * is the backward pass.  head_dim % 16 == 0.  x_pitch / y_pitch: row pitches in elements, 0 = contiguous; a multiple
  * of 8 (16-byte rows), for x or y that is a column slice of a fused q/k/v tensor (coat/models/coat_olmo.py:1003-1006). */
-int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, const int64_t* pos,
-                   int64_t rows, int seq_len, int heads, int head_dim, int inverse, int64_t x_pitch, int64_t y_pitch,
-                   void* stream);
+int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, int64_t n_pos, float theta,
+                   const int64_t* pos, int64_t rows, int seq_len, int heads, int head_dim, int inverse, int64_t x_pitch,
+                   int64_t y_pitch, void* stream);
 
 /* ---- GEMM -------------------------------------------------------------------------------------------
  * rq/linear.py:172 fp8matmul (kernel :61-169): C[M,N] = (A[M,K] . B[N,K]^T) * (float(*scale_a) * float(*scale_b))
@@ -236,10 +238,12 @@ int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* si
  * the .t() view of such a matrix, linear.py:253-302); fmt_a / fmt_b are coat_fp8 values and may differ.
  * out_kind 0: C is bf16 [M,N] (:166-169).  out_kind 1 / 2: C is e4m3 / e5m2 [M,N], quantized per 1 x QB group along
  * N with scale (amax + 1e-10) / fp8max, and c_scale is bf16 [M, N/QB] (:139-164); QB must be 16.
- * scale_a / scale_b: one element each of s_dtype in device memory.  K % 16 == 0. */
+ * scale_a / scale_b: one element each in device memory, of sa_dtype / sb_dtype (each is loaded in its own dtype and the
+ * two are multiplied in fp32, :123-125: an fp32 weight scale next to a bf16 activation scale keeps all its bits).
+ * K % 16 == 0. */
 int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
-                  const void* scale_a, const void* scale_b, int s_dtype, const void* bias, int bias_dtype, int64_t M,
-                  int64_t N, int64_t K, int QB, void* stream);
+                  const void* scale_a, int sa_dtype, const void* scale_b, int sb_dtype, const void* bias, int bias_dtype,
+                  int64_t M, int64_t N, int64_t K, int QB, void* stream);
 
 /* ---- optimizer -------------------------------------------------------------------------------- */
 

@@ -1,9 +1,10 @@
 """GPU parity: fused SiLU / GELU / mul / add / RMSNorm kernels against the CPU oracle.
 
 mul and add contain no transcendental function: codes, scales and bf16 values must be bit-exact.
-SiLU / GELU / RMSNorm differ from the oracle only through exp / erf / the order of a long sum (a few fp32 ulp
-before quantization), so the bar is: bf16 values equal or one bf16 ulp apart on < 1e-3 of the elements, per-tensor
-scale identical, FP8 codes different on < 1e-3 of the elements and by one code step at most.
+SiLU / GELU / RMSNorm / LayerNorm differ from the oracle only through exp / erf / the order of a long sum (a few fp32 ulp
+before quantization).  Measured on an MI355X (printed with ``pytest -rP``): FP8 codes differ on 0 .. 2.9e-6 of the elements
+(by one code step), bf16 values on 5e-6 .. 1e-5 (by one ulp; two on 1 of 6.3e6 norm gradients), per-tensor scales never.
+Bars: codes 1e-5, bf16 values 3e-5, per-tensor scale identical.
 Shape: batch 4 x seq 256 x channels 2048, QB 16 (tests/test_fp8_activations.py:218-226 of the reference)."""
 import pytest
 import torch
@@ -32,10 +33,16 @@ def b(t):
     return t.cpu().view(torch.uint8)
 
 
-def codes_close(got, want, max_frac=1e-3):
+def _caller():
+    import inspect
+    return inspect.stack()[2].function
+
+
+def codes_close(got, want, max_frac=1e-5):
     g, w = b(got).int().flatten(), b(want).int().flatten()
     neq = g != w
     frac = neq.float().mean().item()
+    print(f"[measured] {_caller()}: {frac:.3e} of {g.numel()} codes differ (bar {max_frac:.0e})")
     assert frac <= max_frac, f"{frac} of the codes differ"
     if neq.any():
         assert ((g[neq] & 0x7F) - (w[neq] & 0x7F)).abs().max().item() <= 1
@@ -43,12 +50,14 @@ def codes_close(got, want, max_frac=1e-3):
     return frac
 
 
-def bf16_close(got, want, max_frac=1e-3, max_ulp=1):
+def bf16_close(got, want, max_frac=3e-5, max_ulp=1):
     g, w = got.cpu().view(torch.int16).int().flatten(), want.view(torch.int16).int().flatten()
     neq = g != w
-    assert neq.float().mean().item() <= max_frac
-    if neq.any():
-        assert (g[neq] - w[neq]).abs().max().item() <= max_ulp  # neighbouring bf16 values (same sign)
+    frac = neq.float().mean().item()
+    ulp = (g[neq] - w[neq]).abs().max().item() if neq.any() else 0
+    print(f"[measured] {_caller()}: {frac:.3e} of {g.numel()} bf16 values differ, {ulp} ulp at most (bar {max_frac:.0e}, {max_ulp} ulp)")
+    assert frac <= max_frac
+    assert ulp <= max_ulp  # neighbouring bf16 values (same sign)
 
 
 def test_mul_forward_backward_bit_exact(dev):
@@ -129,12 +138,12 @@ def test_rmsnorm_forward_backward(dev, N):
     wq, wspt, wqt, wrstd = R.fp8_rmsnorm_forward(q, s, w, QB, 1e-5, accumulate=torch.float64)
     assert torch.allclose(rstd.cpu(), wrstd, rtol=1e-6, atol=0)
     assert spt.item() == wspt.item()
-    codes_close(qy, wq, 2e-3)
+    codes_close(qy, wq)
     assert torch.equal(b(qyt), b(qy).t())
     dx, dw = rq.fp8_rmsnorm_backward(q.to(dev), s.to(dev), g.to(dev), w.to(dev), rstd, QB, nw)
     wdx, wdw = R.fp8_rmsnorm_backward(q, s, g, w, wrstd, QB)
     # dx = (w*dy - xhat*c1)*rstd cancels; the fp32 summation order of c1 shows up as a few bf16 ulp on rare elements
-    bf16_close(dx, wdx, 5e-3, max_ulp=4)
+    bf16_close(dx, wdx, 3e-5, max_ulp=2)
     assert dw.dtype == w.dtype and torch.allclose(dw.cpu().float(), wdw.float(), rtol=1e-2, atol=1e-3)  # bf16 output
     # deterministic: the same call again gives the same bits (the reference's lock-ordered dw does not)
     dx2, dw2 = rq.fp8_rmsnorm_backward(q.to(dev), s.to(dev), g.to(dev), w.to(dev), rstd, QB, nw)
@@ -157,7 +166,7 @@ def test_layernorm_forward_backward(dev, N, affine):
     assert torch.allclose(mean.cpu(), wmean, rtol=1e-5, atol=1e-7)
     assert torch.allclose(rstd.cpu(), wrstd, rtol=2e-6, atol=0)
     assert spt.item() == wspt.item()
-    codes_close(qy, wq, 2e-3)
+    codes_close(qy, wq)
     assert torch.equal(b(qyt), b(qy).t())
     if affine:
         dx, dw, db = rq.fp8_layernorm_param_backward(q.to(dev), s.to(dev), g.to(dev), QB, w.to(dev), bb.to(dev), mean, rstd, nw)
@@ -173,7 +182,7 @@ def test_layernorm_forward_backward(dev, N, affine):
     # fp32 summation order of c1 / c2 decides its bits, so those elements are held to that absolute bound instead
     big = wdx.float().abs().max()
     small = (wdx.float().abs() < big * 2.0 ** -12) & (dx.cpu().float().abs() < big * 2.0 ** -12)
-    bf16_close(torch.where(small.to(dev), torch.zeros_like(dx), dx), torch.where(small, torch.zeros_like(wdx), wdx), 5e-3, max_ulp=4)
+    bf16_close(torch.where(small.to(dev), torch.zeros_like(dx), dx), torch.where(small, torch.zeros_like(wdx), wdx), 3e-5, max_ulp=2)
     # batched input keeps its leading dimensions
     q3, s3 = q.reshape(4, M // 4, N).to(dev), s.reshape(4, M // 4, N // QB).to(dev)
     if not affine:

@@ -1,14 +1,14 @@
 """GPU: CoatLlamaDecoderLayer forward + backward.
 
 Forward parity is against the CPU oracle chained into the same layer (same FP8 quantization points, float64 GEMM
-accumulation, fp32 attention): relative Frobenius error <= 8 % on what the layer adds to its input and <= 5 % on its
-dequantized FP8 copy.  The bound is not tighter because the chain re-quantizes five times: the bf16 attention on the
-GPU differs from the fp32 attention of the oracle by ~0.5 %, which moves ~8 % of the following e4m3 roundings by a
-whole code step (6 %); every single kernel of the chain is compared bit for bit (or to its stated tolerance) against
-the oracle on identical inputs in the other GPU test files.  Backward has no FP8 oracle chain; it is compared with the same layer
-differentiated in fp32 torch, where the stated bar is the FP8 quantization noise itself: relative Frobenius error
-<= 12 % on the input gradient and on every weight gradient (e4m3 operands carry 2^-4, e5m2 gradients 2^-3 relative
-rounding noise per element and two to three quantized GEMMs are chained)."""
+accumulation, fp32 attention): relative Frobenius error on what the layer adds to its input (measured 0.062, bar 0.08)
+and on its dequantized FP8 copy (measured 0.013, bar 0.035).  The bound is not tighter because the chain re-quantizes five
+times: the bf16 attention on the GPU differs from the fp32 attention of the oracle by ~0.5 %, which moves ~8 % of the
+following e4m3 roundings by a whole code step (6 %).  The modules' forward and backward are compared operation by operation,
+on identical inputs, in tests/test_gpu_layer_chain.py; here the whole layer is compared with the same layer differentiated
+in fp32 torch, where the bar is the FP8 quantization noise of the precision flow itself: measured 0.075 .. 0.108 on the
+weight gradients (bar 0.14), 0.082 on the forward (bar 0.12), 0.013 on the input gradient (bar 0.03; the residual path
+carries most of it in bf16).  Measured values are printed (``pytest -rP``)."""
 import pytest
 import torch
 import torch.nn.functional as F
@@ -55,6 +55,11 @@ def reference_layer(layer, x, dtype=torch.float32):
 
 def rel(a, b):
     return ((a.float().cpu() - b.float().cpu()).norm() / b.float().cpu().norm()).item()
+
+
+def within(what, value, bar):
+    print(f"[measured] {what}: {value:.4f} (bar {bar})")
+    assert value < bar, (what, value, bar)
 
 
 def oracle_layer_forward(layer, x):
@@ -125,18 +130,18 @@ def test_decoder_layer_forward_backward(dev, memory_efficient):
     yr.backward(gy.float())
     # forward parity against the chained CPU oracle (what the layer adds to its input; the residual path is exact)
     oh, oq, osc = oracle_layer_forward(layer, x)
-    assert rel(y.detach().cpu() - x.cpu(), oh - x.cpu()) < 0.08
+    within("forward vs chained oracle", rel(y.detach().cpu() - x.cpu(), oh - x.cpu()), 0.08)
     from oracle import activation_ref as R
     deq_gpu = R.fp8_dequantize(qh.detach().cpu().reshape(-1, H), sh.detach().cpu().reshape(-1, H // 16), 16)
     deq_cpu = R.fp8_dequantize(oq.reshape(-1, H), osc.reshape(-1, H // 16), 16)
-    assert rel(deq_gpu, deq_cpu) < 0.05
-    assert rel(deq_gpu, h.detach().reshape(-1, H)) < 0.04  # the FP8 copy of the output is the output, to e4m3 accuracy
+    within("FP8 copy vs chained oracle", rel(deq_gpu, deq_cpu), 0.035)
+    within("FP8 copy vs output", rel(deq_gpu, h.detach().reshape(-1, H)), 0.03)  # the FP8 copy of the output is the output, to e4m3 accuracy
     # against the fp32 layer: FP8 quantization noise
-    assert rel(y.detach() - x, yr.detach() - x.float()) < 0.12
-    assert rel(xin.grad, xr.grad) < 0.12
+    within("forward vs fp32 layer", rel(y.detach() - x, yr.detach() - x.float()), 0.12)
+    within("input gradient vs fp32 layer", rel(xin.grad, xr.grad), 0.03)
     for n, p in layer.named_parameters():
         assert p.grad is not None, n
-        assert rel(p.grad, W[n].grad) < 0.12, (n, rel(p.grad, W[n].grad))
+        within(n + " gradient vs fp32 layer", rel(p.grad, W[n].grad), 0.14)
 
     # second micro-batch reuses the cached weight scales / FP8 weights and gives the same result for the same input
     FP8Manager.is_first_microbatch = False
@@ -154,9 +159,11 @@ def test_decoder_layer_forward_backward(dev, memory_efficient):
     assert qe is None and rel(he, yr.detach()) < 0.02
 
 
-@pytest.mark.parametrize("with_ids", [False, True])
-def test_fused_rope_matches_formula(dev, with_ids):
-    """coat_rope_bf16 forward / backward against q*cos + rotate_half(q)*sin and its autograd in fp32 (one bf16 rounding)."""
+@pytest.mark.parametrize("with_ids,max_positions", [(False, 256), (True, 256), (True, 100)])
+def test_fused_rope_matches_formula(dev, with_ids, max_positions):
+    """coat_rope_bf16 forward / backward against q*cos + rotate_half(q)*sin and its autograd in fp32 (one bf16 rounding).
+    With max_positions = 100 the positions 100..112 of the second sequence lie beyond the cos / sin tables: the kernel
+    computes their angles itself instead of reading past the tables (or clamping the position)."""
     from coat_amd.models.coat_llama import apply_rotary_pos_emb, fused_rotary, rotary_cos_sin
     B, S, nh, hd = 2, 96, 4, 64
     g = torch.Generator().manual_seed(3)
@@ -164,7 +171,7 @@ def test_fused_rope_matches_formula(dev, with_ids):
     gy = torch.randn(B, nh, S, hd, generator=g).bfloat16()
     pos = (torch.arange(S).unsqueeze(0).expand(B, -1) + torch.tensor([[0], [17]])) if with_ids else None
     xd = x.to(dev).requires_grad_(True)
-    y = fused_rotary(xd, nh, hd, 10000.0, None if pos is None else pos.to(dev), 256)
+    y = fused_rotary(xd, nh, hd, 10000.0, None if pos is None else pos.to(dev), max_positions)
     assert y.shape == (B, nh, S, hd)
     y.backward(gy.to(dev))
     xr = x.float().requires_grad_(True)

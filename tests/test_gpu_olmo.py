@@ -46,6 +46,11 @@ def rel(a, b):
     return ((a.float().cpu() - b.float().cpu()).norm() / b.float().cpu().norm()).item()
 
 
+def within(what, value, bar):
+    print(f"[measured] {what}: {value:.4f} (bar {bar})")
+    assert value < bar, (what, value, bar)
+
+
 def oracle_block_forward(blk, x):
     """coat_olmo.py:160-207, :310-345, :480-555 restated with oracle/activation_ref.py on the CPU."""
     from oracle import activation_ref as R
@@ -102,16 +107,16 @@ def test_olmo_block_forward_backward(dev, memory_efficient):
     xr, yr, W = reference_block(blk, x)
     yr.backward(gy.float())
     oh, oq, osc = oracle_block_forward(blk, x)
-    assert rel(y.detach().cpu() - x.cpu(), oh - x.cpu()) < 0.05
+    within("forward vs chained oracle", rel(y.detach().cpu() - x.cpu(), oh - x.cpu()), 0.05)
     deq_gpu = R.fp8_dequantize(qh.detach().cpu().reshape(-1, D), sh.detach().cpu().reshape(-1, D // 16), 16)
     deq_cpu = R.fp8_dequantize(oq.reshape(-1, D), osc.reshape(-1, D // 16), 16)
-    assert rel(deq_gpu, deq_cpu) < 0.05
-    assert rel(deq_gpu, h.detach().reshape(-1, D)) < 0.04
-    assert rel(y.detach() - x, yr.detach() - x.float()) < 0.12
-    assert rel(xin.grad, xr.grad) < 0.12
+    within("FP8 copy vs chained oracle", rel(deq_gpu, deq_cpu), 0.035)
+    within("FP8 copy vs output", rel(deq_gpu, h.detach().reshape(-1, D)), 0.03)
+    within("forward vs fp32 layer", rel(y.detach() - x, yr.detach() - x.float()), 0.12)
+    within("input gradient vs fp32 layer", rel(xin.grad, xr.grad), 0.03)
     for n, p in blk.named_parameters():
         assert p.grad is not None, n
-        assert rel(p.grad, W[n].grad) < 0.12, (n, rel(p.grad, W[n].grad))
+        within(n + " gradient vs fp32 layer", rel(p.grad, W[n].grad), 0.12)
 
     # second micro-batch with cached weight scales / FP8 weights: identical result
     FP8Manager.is_first_microbatch = False

@@ -80,13 +80,13 @@ def test_argument_validation_of_the_remaining_entry_points_without_gpu():
     assert L.coat_fp8_rmsnorm_forward(p, 0, p, 1, p, 1, None, p, p, p, 4, 32768, 16, 1e-5, None) == ESHAPE   # row too long
     assert L.coat_fp8_rmsnorm_forward(p, 0, p, 1, p, 1, None, None, p, p, 4, 64, 16, 1e-5, None) == EINVAL
     # GEMM
-    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 0, p, p, 1, None, 0, 64, 64, 24, 16, None) == ESHAPE    # K % 16
-    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 1, p, p, 1, None, 0, 64, 64, 64, 16, None) == ESHAPE    # quantized output without scales
-    assert L.coat_fp8_gemm(p, 3, p, 0, p, None, 0, p, p, 1, None, 0, 64, 64, 64, 16, None) == EINVAL    # unknown operand format
-    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 0, p, p, 1, None, 0, 0, 64, 64, 16, None) == 0          # empty
+    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 0, p, 1, p, 1, None, 0, 64, 64, 24, 16, None) == ESHAPE    # K % 16
+    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 1, p, 1, p, 1, None, 0, 64, 64, 64, 16, None) == ESHAPE    # quantized output without scales
+    assert L.coat_fp8_gemm(p, 3, p, 0, p, None, 0, p, 1, p, 1, None, 0, 64, 64, 64, 16, None) == EINVAL    # unknown operand format
+    assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 0, p, 1, p, 1, None, 0, 0, 64, 64, 16, None) == 0          # empty
     # RoPE, cross-entropy, probe
-    assert L.coat_rope_bf16(p, p, p, p, None, 8, 8, 2, 24, 0, 0, 0, None) == ESHAPE                      # head_dim % 16
-    assert L.coat_rope_bf16(p, p, p, p, None, 8, 8, 2, 32, 0, 48, 0, None) == ESHAPE                     # pitch < heads * head_dim
+    assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 24, 0, 0, 0, None) == ESHAPE                      # head_dim % 16
+    assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 48, 0, None) == ESHAPE                     # pitch < heads * head_dim
     assert L.coat_cross_entropy_forward(p, 0, 8, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # stride < columns
     assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # mean without a count
     assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, p, 4, 16, -100, 0.0, 0.0, 7, 0.0, 0, None) == EINVAL
