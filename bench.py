@@ -1,15 +1,19 @@
 """Benchmark of the FP8 hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload adamw|quantize|quantize_transpose]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|adamw|quantize|quantize_transpose|gemm_fwd|...]
 
-Default workload = the headline configuration: one CoatAdamW step (Dynamic Range Expansion on) on an fp32 master
-weight [11008, 4096], grads N(0, 1e-3), lr 3e-4, betas (0.9, 0.95), wd 0.1, eps 1e-8, starting at step 10 from a
-moment state produced by nine untimed steps.  A "step" is one pass of the fused kernel over the whole tensor.
-Prints ONE JSON line.  `value` is algorithmic GB/s: every distinct input read once + every output written once
-(in-place tensors count read + write) divided by the wall-clock per step with inputs resident in HBM.
-`roofline.achieved` uses the kernel's average launch duration: HIP events on the launch stream around the K
-back-to-back launches of the timed region, divided by K (per-launch event pairs of a second pass give the spread).
-`cpu_baseline` times the plain-C oracle (one thread) on a bounded sample of the same workload.
+Prints ONE JSON line.  The default run (--workload all) times the headline configuration as `value` and adds an `extra`
+record for every other leg of the metric (quantize, quantize + transpose, the three GEMMs of the 7B MLP linear, the
+SiLU*mul and RMSNorm chains, the 7B and 13B decoder layers), each with its own roofline and CPU baseline.
+
+Headline = one CoatAdamW.step() (Dynamic Range Expansion on) on an fp32 master weight [11008, 4096], grads N(0, 1e-3),
+lr 3e-4, betas (0.9, 0.95), wd 0.1, eps 1e-8, starting at step 10 from a moment state produced by nine untimed steps.
+A "step" is one pass of the fused kernel over the whole tensor.  `value` is algorithmic GB/s: every distinct input read
+once + every output written once (in-place tensors count read + write) divided by the wall-clock per step with inputs
+resident in HBM.  `roofline.achieved` uses the kernel's average launch duration: HIP events on the launch stream around
+the K back-to-back launches of the timed region, divided by K (per-launch event pairs of a second pass give the spread).
+`cpu_baseline` times the CPU oracle (the plain-C AdamW port on every host core; the torch restatements for the other
+legs) on a bounded sample of the same workload.
 """
 import argparse
 import json
@@ -59,10 +63,39 @@ def make_adamw_workload(dev, shape, torch, expand=True):
     for _ in range(9):  # steps 1..9: builds a realistic moment state (k, c per group), untimed
         step()
     if expand:
-        return step, adamw_bytes(numel), {"workload": "CoatAdamW.step fp32 [11008,4096], DRE on, step 10+, qgroup 128",
+        return step, adamw_bytes(numel), {"workload": "qoptim_cuda.fp8_adamw_expand_step (the call CoatAdamW.step makes) fp32 [11008,4096], DRE on, step 10+, qgroup 128",
                                           "numel": numel, "kernel": "k_fp8_adamw_expand"}
-    return step, numel * 16 + ng * 16, {"workload": "CoatAdamW.step fp32 [11008,4096], DRE off, step 10+, qgroup 128",
+    return step, numel * 16 + ng * 16, {"workload": "qoptim_cuda.fp8_adamw_step fp32 [11008,4096], DRE off, step 10+, qgroup 128",
                                         "numel": numel, "kernel": "k_fp8_adamw_plain"}
+
+
+def make_adamw_class_workload(dev, shape, torch):
+    """The same step through the optimizer class: CoatAdamW.step() on one fp32 parameter [11008, 4096] (the host loop of
+    coat/optimizer/fp8_adamw.py:264-515 is then inside the timed region; it ends in the same kernel launch)."""
+    from coat_amd.optimizer.fp8_adamw import CoatAdamW
+    from coat_amd.utils._fp8_quantization_config import QuantizationConfig
+
+    numel = shape[0] * shape[1]
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    p = torch.nn.Parameter((torch.randn(shape, generator=gen) * 0.02).to(dev))
+    grads = []
+    for seed in range(1, 5):  # a few distinct gradient tensors, cycled
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        grads.append((torch.randn(shape, generator=g) * 1e-3).to(dev))
+    opt = CoatAdamW([p], lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1, qargs=QuantizationConfig())
+    assert opt.use_expansion, "the headline configuration runs with Dynamic Range Expansion"
+    state = {"i": 0}
+
+    def step():
+        state["i"] += 1
+        p.grad = grads[state["i"] % len(grads)]
+        opt.step()
+
+    for _ in range(9):  # steps 1..9: builds a realistic moment state (k, c per group), untimed
+        step()
+    return step, adamw_bytes(numel), {"workload": "CoatAdamW.step() on one fp32 parameter [11008,4096], DRE on, step 10+, "
+                                                  "qgroup 128 (optimizer class host loop + k_fp8_adamw_expand)",
+                                      "numel": numel, "kernel": "k_fp8_adamw_expand"}
 
 
 def make_quantize_workload(dev, torch, transpose, shape=(4096, 4096)):
@@ -420,48 +453,81 @@ def make_layer_workload(dev, torch, size, cache_weights=False):
         "tokens": B * S, "gemm_flops": gemm_flops}
 
 
+def host_threads():
+    """CPU threads this process may use: the affinity mask, capped at the 16 cores a one-GPU box grants."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    return max(1, min(n, 16))
+
+
+def _median(ts):
+    ts = sorted(ts)
+    return ts[len(ts) // 2]
+
+
 def cpu_baseline_adamw(torch):
-    """The plain-C oracle (one thread) on a bounded sample: same hyper-parameters, step 10 state built by the
-    oracle itself, sample sized for roughly 10-20 s."""
+    """The plain-C oracle on every host core: one thread per core, each stepping its own 4096-group slab of the tensor
+    (groups are independent, so this is how a CPU run of the whole tensor would be split), same hyper-parameters, moment
+    state built by three oracle steps, about 10 s of wall clock."""
+    import threading
+
     from oracle import adamw_ref as A
 
     hp = (0.9, 0.95, 3e-4, 0.1, 1e-8)
-    n = 128 * 4096  # 0.5 M elements of the [11008, 4096] tensor
-    gen = torch.Generator().manual_seed(0)
-    p = torch.randn(n, generator=gen) * 0.02
-    st = A.fresh_state(p, True)
+    n = 128 * 4096  # elements per thread
+    T = host_threads()
     keys = ("exp_avg", "scale_exp_avg", "expand_exp_avg", "sqrt_minmax_exp_avg", "exp_avg_sq", "scale_exp_avg_sq",
             "expand_exp_avg_sq", "sqrt_minmax_exp_avg_sq")
-    grads = [torch.randn(n, generator=gen) * 1e-3 for _ in range(4)]
-    step = 0
-    for _ in range(3):
-        step += 1
-        A.adamw_expand_step(p, grads[step % 4], *[st[k] for k in keys], *hp, step, 128, 16)
+    A.lib()
+    slabs = []
+    for t in range(T):
+        gen = torch.Generator().manual_seed(t)
+        p = torch.randn(n, generator=gen) * 0.02
+        st = A.fresh_state(p, True)
+        grads = [torch.randn(n, generator=gen) * 1e-3 for _ in range(4)]
+        for step in (1, 2, 3):
+            A.adamw_expand_step(p, grads[step % 4], *[st[k] for k in keys], *hp, step, 128, 16)
+        slabs.append((p, st, grads))
+    reps = [0] * T
+    t_end = time.perf_counter() + 10.0
+
+    def work(t):
+        p, st, grads = slabs[t]
+        step = 3
+        while time.perf_counter() < t_end:
+            step += 1
+            A.adamw_expand_step(p, grads[step % 4], *[st[k] for k in keys], *hp, step, 128, 16)  # ctypes drops the GIL
+            reps[t] += 1
+
     t0 = time.perf_counter()
-    reps = 0
-    while time.perf_counter() - t0 < 10.0:
-        step += 1
-        A.adamw_expand_step(p, grads[step % 4], *[st[k] for k in keys], *hp, step, 128, 16)
-        reps += 1
-    dt = (time.perf_counter() - t0) / reps
-    return {"value": round(adamw_bytes(n) / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} steps over the first {n} elements (4096 groups) of the tensor, oracle/adamw_ref.c, 1 thread"}
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(T)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    dt = time.perf_counter() - t0
+    return {"value": round(adamw_bytes(n) * sum(reps) / dt / 1e9, 4), "unit": "GB/s", "cores": T, "kind": "port",
+            "sample": f"oracle/adamw_ref.c, {T} threads, each stepping its own slab of {n} elements (4096 groups) of the "
+                      f"tensor, {sum(reps)} slab steps in {dt:.1f} s"}
 
 
 # HBM / fabric bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled by what the same
-# counters read for a 256 MiB copy); the runs are recorded under profiles/.  They cannot be taken inside this process.
+# counters read for a 256 MiB copy).  The counters cannot be read inside this process: the figures come from the separate
+# profiling runs recorded under profiles/, not from this run.
 MEASURED_TRAFFIC = {
-    "adamw": 759.1e6,               # profiles/k_fp8_adamw_expand__adamw_11008x4096.txt
-    "quantize": 52.5e6,             # profiles/k_quantize_pg__quantize_4096x4096_bf16.txt
-    "quantize_transpose": 73.6e6,   # profiles/k_quantize_transpose__quantize_transpose_4096x4096_bf16.txt
-    "gemm_fwd": 743.0e6,             # profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt
-    "gemm_dgrad": 608.4e6,
-    "cross_entropy": 2099.7e6,      # profiles/k_cross_entropy__llama2_vocab32000_8192tok_fp32.txt
+    "adamw": (759.1e6, "profiles/k_fp8_adamw_expand__adamw_11008x4096.txt"),
+    "quantize": (52.5e6, "profiles/k_quantize_pg__quantize_4096x4096_bf16.txt"),
+    "quantize_transpose": (73.6e6, "profiles/k_quantize_transpose__quantize_transpose_4096x4096_bf16.txt"),
+    "gemm_fwd": (743.0e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
+    "gemm_dgrad": (608.4e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
+    "cross_entropy": (2099.7e6, "profiles/k_cross_entropy__llama2_vocab32000_8192tok_fp32.txt"),
 }
 
 
 def cpu_baseline_quantize(torch, transpose, nbytes):
-    """The torch-CPU oracle on the whole [4096,4096] input (same seeded data), all host threads, median of 5 runs."""
+    """The torch-CPU oracle on the whole [4096,4096] input (same seeded data), all host threads, 3 warm-ups, median of 10."""
     from oracle import activation_ref as R
 
     gen = torch.Generator(device="cpu").manual_seed(0)
@@ -469,15 +535,127 @@ def cpu_baseline_quantize(torch, transpose, nbytes):
     x[torch.rand(4096, 4096, generator=gen) < 0.001] *= 100
     x = x.bfloat16()
     fn = R.fp8_quantize_transpose if transpose else R.fp8_quantize
-    fn(x, 16, "E4M3")
+    for _ in range(3):
+        fn(x, 16, "E4M3")
     ts = []
-    for _ in range(5):
+    for _ in range(10):
         t0 = time.perf_counter()
         fn(x, 16, "E4M3")
         ts.append(time.perf_counter() - t0)
-    ts.sort()
-    return {"value": round(nbytes / ts[2] / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"the whole bf16 [4096,4096] input, oracle/activation_ref.py ({fn.__name__}), median of 5 runs"}
+    return {"value": round(nbytes / _median(ts) / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"the whole bf16 [4096,4096] input, oracle/activation_ref.py ({fn.__name__}), median of 10 runs"}
+
+
+def cpu_baseline_gemm(torch, which):
+    """The oracle's GEMM (fp32 matmul of the decoded FP8 operands, times the two scales, rounded to bf16) on a 1024-row slab of
+    the left operand, all host threads, median of 3."""
+    from oracle import activation_ref as R
+
+    T, K, N = 8192, 4096, 11008
+    M_, N_, K_ = {"fwd": (T, N, K), "dgrad": (T, K, N), "wgrad": (N, K, T)}[which]
+    rows = 1024
+    gen = torch.Generator().manual_seed(0)
+    a = torch.randn(rows, K_, generator=gen).to(torch.float8_e4m3fn)
+    b = torch.randn(N_, K_, generator=gen).to(torch.float8_e4m3fn)
+    one = torch.tensor(0.01, dtype=torch.bfloat16)
+    R.fp8matmul(a, b.t(), False, one, one, 16)
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        R.fp8matmul(a, b.t(), False, one, one, 16)
+        ts.append(time.perf_counter() - t0)
+    return {"value": round(2 * rows * N_ * K_ / _median(ts) / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"oracle/activation_ref.py fp8matmul on {rows} of the {M_} rows of the left operand, median of 3 runs"}
+
+
+def cpu_baseline_silu_mul(torch, nbytes_full):
+    """The oracle's chain (quantize x 2, SiLU, mul, mul backward, SiLU backward, all with their per-tensor divisions) on a
+    256-row slab of the [8192, 11008] inputs, all host threads, median of 3."""
+    from oracle import activation_ref as R
+
+    rows, M, N, QB = 256, 8192, 11008, 16
+    gen = torch.Generator().manual_seed(0)
+    gate, up = torch.randn(rows, N, generator=gen).bfloat16(), torch.randn(rows, N, generator=gen).bfloat16()
+    g = (torch.randn(rows, N, generator=gen) * 1e-2).bfloat16()
+
+    def chain():
+        qg, sg = R.fp8_quantize(gate, QB, "E4M3")
+        qu, su = R.fp8_quantize(up, QB, "E4M3")
+        qs, ss = R.fp8_silu_forward(qg, sg, QB)
+        R.fp8_mul_forward(qs, ss, qu, su, QB)
+        g1, _ = R.fp8_mul_backward(qs, ss, qu, su, g, QB, "E5M2", True)
+        R.fp8_silu_backward(qg, sg, g1, QB, "E5M2", True)
+
+    chain()
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        chain()
+        ts.append(time.perf_counter() - t0)
+    return {"value": round(nbytes_full * rows / M / _median(ts) / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"oracle/activation_ref.py chain on {rows} of the {M} rows, median of 3 runs"}
+
+
+def cpu_baseline_rmsnorm(torch, nbytes_full):
+    from oracle import activation_ref as R
+
+    rows, M, N, QB = 1024, 8192, 4096, 16
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(rows, N, generator=gen).bfloat16()
+    w = torch.ones(N, dtype=torch.bfloat16)
+    g = (torch.randn(rows, N, generator=gen) * 1e-2).bfloat16()
+    q, s = R.fp8_quantize(x, QB, "E4M3")
+
+    def chain():
+        _, _, _, rstd = R.fp8_rmsnorm_forward(q, s, w, QB, 1e-5)
+        R.fp8_rmsnorm_backward(q, s, g, w, rstd, QB, accumulate=torch.float32)
+
+    chain()
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        chain()
+        ts.append(time.perf_counter() - t0)
+    return {"value": round(nbytes_full * rows / M / _median(ts) / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"oracle/activation_ref.py forward + backward on {rows} of the {M} rows, median of 3 runs"}
+
+
+def cpu_baseline_layer(torch, size):
+    """The same decoder layer in fp32 torch on the host (F.rms_norm / F.linear / SDPA / F.silu, forward + backward) on one
+    sequence of 256 tokens; ms scaled by tokens to the 4 x 2048 of the GPU run (attention, 5 % of the work, scales worse)."""
+    import torch.nn.functional as F
+
+    H, heads, I = (4096, 32, 11008) if size == "7b" else (5120, 40, 13824)
+    S, hd = 256, H // heads
+    gen = torch.Generator().manual_seed(0)
+    W = {n: (torch.randn(shape, generator=gen) * 0.02).requires_grad_(True) for n, shape in
+         (("q", (H, H)), ("k", (H, H)), ("v", (H, H)), ("o", (H, H)), ("gate", (I, H)), ("up", (I, H)), ("down", (H, I)))}
+    n1, n2 = torch.ones(H, requires_grad=True), torch.ones(H, requires_grad=True)
+    x = torch.randn(1, S, H, generator=gen)
+    gy = torch.randn(1, S, H, generator=gen) * 1e-2
+
+    def step():
+        for t in list(W.values()) + [n1, n2]:
+            t.grad = None
+        xin = x.clone().requires_grad_(True)
+        h = F.rms_norm(xin, (H,), n1, 1e-5)
+        q, k, v = (F.linear(h, W[n]).view(1, S, heads, hd).transpose(1, 2) for n in ("q", "k", "v"))
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(1, S, H)
+        x1 = xin + F.linear(a, W["o"])
+        h2 = F.rms_norm(x1, (H,), n2, 1e-5)
+        y = x1 + F.linear(F.silu(F.linear(h2, W["gate"])) * F.linear(h2, W["up"]), W["down"])
+        y.backward(gy)
+
+    step()
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        step()
+        ts.append(time.perf_counter() - t0)
+    ms = _median(ts) * 1e3
+    return {"value": round(ms * 8192 / S, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"fp32 torch layer of the same shape (RoPE left out), forward + backward on 1 x {S} tokens: {ms:.1f} ms, "
+                      f"median of 3 runs, scaled by 8192 / {S} tokens"}
 
 
 def ramp_clocks(step, seconds, torch):
@@ -491,13 +669,17 @@ def ramp_clocks(step, seconds, torch):
         torch.cuda.synchronize()
 
 
-def bench_layer(args, dev, torch):
-    if args.workload == "linear":
+METRIC = "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms"
+LAYER_WORKLOADS = ("layer_7b", "layer_13b", "linear", "olmo_block")
+
+
+def measure_layer(name, args, dev, torch, cpu):
+    if name == "linear":
         step_fp8, step_bf16, gemm_flops, cfg = make_linear_workload(dev, torch)
-    elif args.workload == "olmo_block":
+    elif name == "olmo_block":
         step_fp8, step_bf16, gemm_flops, cfg = make_olmo_workload(dev, torch)
     else:
-        step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, args.workload.split("_")[1], args.cache_weights)
+        step_fp8, step_bf16, gemm_flops, cfg = make_layer_workload(dev, torch, name.split("_")[1], args.cache_weights)
 
     def time_it(fn):
         ramp_clocks(fn, args.ramp_seconds, torch)
@@ -515,23 +697,117 @@ def bench_layer(args, dev, torch):
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e3 / args.steps
         ms = sorted(a.elapsed_time(b) for a, b in evs)
-        return wall, ms[len(ms) // 2]
+        return wall, ms[len(ms) // 2], ms[len(ms) // 5], ms[(4 * len(ms)) // 5]
 
-    wall8, med8 = time_it(step_fp8)
-    wall16, med16 = time_it(step_bf16)
-    out = {
-        "metric": "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms",
-        "value": round(wall8, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(wall8, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp8", "data": "synthetic", "config": cfg,
-        "layer": {"fp8_ms_median": round(med8, 4), "bf16_ms_median": round(med16, 4), "bf16_ms_per_step": round(wall16, 4),
+    wall8, med8, p20, p80 = time_it(step_fp8)
+    wall16, med16, _, _ = time_it(step_bf16)
+    rec = {
+        "value": round(wall8, 4), "unit": "ms", "ms_per_step": round(wall8, 4), "higher_is_better": False,
+        "dtype": "fp8", "config": cfg,
+        "layer": {"fp8_ms_median": round(med8, 4), "fp8_ms_p20": round(p20, 4), "fp8_ms_p80": round(p80, 4),
+                  "bf16_ms_median": round(med16, 4), "bf16_ms_per_step": round(wall16, 4),
                   "speedup_vs_bf16": round(med16 / med8, 4),
                   "fp8_gemm_tflops_equiv": round(gemm_flops / (med8 * 1e-3) / 1e12, 1)},
         "roofline": {"bound": "mfma", "achieved": round(gemm_flops / (med8 * 1e-3) / 1e12, 2), "peak": 5000.0,
-                     "unit": "TFLOP/s", "frac": round(gemm_flops / (med8 * 1e-3) / 1e12 / 5000.0, 4), "traffic": None},
+                     "unit": "TFLOP/s", "frac": round(gemm_flops / (med8 * 1e-3) / 1e12 / 5000.0, 4), "traffic": None,
+                     "note": "GEMM flops of the step over the whole step's time (attention and the FP8 glue kernels included)"},
+        "cpu_baseline": cpu_baseline_layer(torch, name.split("_")[1]) if cpu and name.startswith("layer_") else None,
+    }
+    return rec
+
+
+def make_stream_workload(name, args, dev, torch):
+    if name in ("adamw", "adamw_plain"):
+        return make_adamw_workload(dev, (11008, 4096), torch, expand=name == "adamw")
+    if name == "adamw_class":
+        return make_adamw_class_workload(dev, (11008, 4096), torch)
+    if name.startswith("gemm"):
+        return make_gemm_workload(dev, torch, name.split("_")[1], args.grad_format)
+    if name == "cross_entropy":
+        return make_cross_entropy_workload(dev, torch)
+    if name.startswith("hbm_"):
+        return make_hbm_probe_workload(dev, torch, name.split("_")[1])
+    if name == "layernorm":
+        return make_layernorm_workload(dev, torch)
+    if name in ("division", "division_sr", "division_transpose"):
+        return make_division_workload(dev, torch, name == "division_sr", transpose=name == "division_transpose")
+    if name == "silu_mul":
+        return make_silu_mul_workload(dev, torch)
+    if name == "rmsnorm":
+        return make_rmsnorm_workload(dev, torch)
+    return make_quantize_workload(dev, torch, name == "quantize_transpose", tuple(args.shape))
+
+
+def measure_stream(name, args, dev, torch, cpu):
+    """One workload whose step is a short chain of launches: K steps between two synchronisations for `value`, HIP events
+    on the launch stream around the same K back-to-back launches for the average launch duration of the roofline."""
+    is_gemm = name.startswith("gemm")
+    step, nbytes, cfg = make_stream_workload(name, args, dev, torch)
+    ramp_clocks(step, args.ramp_seconds, torch)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    prepare = getattr(step, "prepare", None)
+    # (1) the timed region: exactly K steps between two synchronisations, nothing else in the loop
+    wall = region_ms = None
+    if not prepare:
+        ra, rb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        ra.record()
+        for _ in range(args.steps):
+            step()
+        rb.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        region_ms = ra.elapsed_time(rb)  # HIP events over the timed region: K launches back to back
+    # (2) the same K steps again with HIP events around every launch, on the stream the kernels are launched on (torch's
+    # current stream): median / p20 / p80 of the launch duration (event records inside loop (1) would add their gaps
+    # to the wall clock)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        if prepare:
+            prepare()
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    kern_ms = sorted(a.elapsed_time(b) for a, b in evs)
+    avg_ms = sum(kern_ms) / len(kern_ms) if prepare else region_ms / args.steps
+    ms_per_step = avg_ms if prepare else wall * 1e3 / args.steps
+    value = nbytes / (ms_per_step * 1e-3) / 1e9
+    achieved = nbytes / (avg_ms * 1e-3) / 1e9
+    unit, peak, bound = ("TFLOP/s", 5000.0, "mfma") if is_gemm else ("GB/s", HBM_PEAK_GBS, "hbm")
+    if is_gemm:  # nbytes holds FLOPs for the GEMM workloads; report TFLOP/s
+        value, achieved = value / 1e3, achieved / 1e3
+    traffic = MEASURED_TRAFFIC.get("adamw" if name == "adamw_class" else name) if args.shape == [4096, 4096] else None
+    rec = {
+        "value": round(value, 2), "unit": unit, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "dtype": "fp8" if is_gemm else ("f32" if name.startswith("adamw") else "bf16"), "config": cfg,
+        "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": traffic[0] if traffic else None,
+                     "traffic_source": (traffic[1] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in a separate run, not this run)") if traffic else None,
+                     ("algorithmic_flops_per_launch" if is_gemm else "algorithmic_bytes_per_launch"): nbytes, "kernel_ms_avg": round(avg_ms, 5),
+                     "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
+                     "kernel_ms_per_launch_events_avg": round(sum(kern_ms) / len(kern_ms), 5),
+                     "kernel_ms_p20": round(kern_ms[len(kern_ms) // 5], 5), "kernel_ms_p80": round(kern_ms[(4 * len(kern_ms)) // 5], 5)},
         "cpu_baseline": None,
     }
-    print(json.dumps(out))
+    if cpu:
+        if name in ("adamw", "adamw_class"):
+            rec["cpu_baseline"] = cpu_baseline_adamw(torch)
+        elif name in ("quantize", "quantize_transpose") and args.shape == [4096, 4096]:
+            rec["cpu_baseline"] = cpu_baseline_quantize(torch, name == "quantize_transpose", nbytes)
+        elif is_gemm:
+            rec["cpu_baseline"] = cpu_baseline_gemm(torch, name.split("_")[1])
+        elif name == "silu_mul":
+            rec["cpu_baseline"] = cpu_baseline_silu_mul(torch, nbytes)
+        elif name == "rmsnorm":
+            rec["cpu_baseline"] = cpu_baseline_rmsnorm(torch, nbytes)
+    return rec
+
+
+# the default run: the headline workload (BASELINE configuration 2) plus one record per remaining leg of the metric
+EXTRAS = ("quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "silu_mul", "rmsnorm", "layer_7b", "layer_13b")
 
 
 def main():
@@ -539,9 +815,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="adamw", choices=["adamw", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "linear",
-                             "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr", "division_transpose", "olmo_block",
-                             "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b"])
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "adamw", "adamw_class", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad",
+                             "gemm_wgrad", "linear", "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr",
+                             "division_transpose", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b"],
+                    help="all (default): the headline AdamW step as `value` plus an `extra` record for every other leg of the metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", type=int, nargs=2, default=[4096, 4096], metavar=("M", "N"),
                     help="input shape of the quantize / quantize_transpose workloads (default: the headline [4096, 4096])")
@@ -571,29 +849,8 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-
-    is_gemm = args.workload.startswith("gemm")
-    if args.workload.startswith("layer_") or args.workload in ("linear", "olmo_block"):
-        return bench_layer(args, dev, torch)
-    if args.workload in ("adamw", "adamw_plain"):
-        step, nbytes, cfg = make_adamw_workload(dev, (11008, 4096), torch, expand=args.workload == "adamw")
-    elif is_gemm:
-        step, nbytes, cfg = make_gemm_workload(dev, torch, args.workload.split("_")[1], args.grad_format)
-    elif args.workload == "cross_entropy":
-        step, nbytes, cfg = make_cross_entropy_workload(dev, torch)
-    elif args.workload.startswith("hbm_"):
-        step, nbytes, cfg = make_hbm_probe_workload(dev, torch, args.workload.split("_")[1])
-    elif args.workload == "layernorm":
-        step, nbytes, cfg = make_layernorm_workload(dev, torch)
-    elif args.workload in ("division", "division_sr", "division_transpose"):
-        step, nbytes, cfg = make_division_workload(dev, torch, args.workload == "division_sr",
-                                                   transpose=args.workload == "division_transpose")
-    elif args.workload == "silu_mul":
-        step, nbytes, cfg = make_silu_mul_workload(dev, torch)
-    elif args.workload == "rmsnorm":
-        step, nbytes, cfg = make_rmsnorm_workload(dev, torch)
-    else:
-        step, nbytes, cfg = make_quantize_workload(dev, torch, args.workload == "quantize_transpose", tuple(args.shape))
+    torch.set_num_threads(host_threads())  # the CPU baselines use every core this process may use
+    cpu = not args.no_cpu_baseline
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -601,63 +858,33 @@ def main():
         for _ in range(5):
             dst.copy_(src)  # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
-    ramp_clocks(step, args.ramp_seconds, torch)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    prepare = getattr(step, "prepare", None)
-    # (1) the timed region: exactly K steps between two synchronisations, nothing else in the loop
-    wall = region_ms = None
-    if not prepare:
-        ra, rb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        ra.record()
-        for _ in range(args.steps):
-            step()
-        rb.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        region_ms = ra.elapsed_time(rb)  # HIP events over the timed region: K launches back to back
-    # (2) the same K steps again with HIP events around every launch, on the stream the kernels are launched on (torch's
-    # current stream): the kernel's own duration for the roofline (event records inside loop (1) would add their gaps
-    # to the wall clock)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    for a, b in evs:
-        if prepare:
-            prepare()
-        a.record()
-        step()
-        b.record()
-    torch.cuda.synchronize()
-    kern_ms = sorted(a.elapsed_time(b) for a, b in evs)
-    # average launch duration: the event pair over the timed region divided by K; the per-launch pairs (which include
-    # the event records' own gaps) give the spread
-    avg_ms = sum(kern_ms) / len(kern_ms) if prepare else region_ms / args.steps
-    ms_per_step = avg_ms if prepare else wall * 1e3 / args.steps
-    value = nbytes / (ms_per_step * 1e-3) / 1e9
-    achieved = nbytes / (avg_ms * 1e-3) / 1e9
+        del src, dst
 
-    unit, peak, bound = ("TFLOP/s", 5000.0, "mfma") if is_gemm else ("GB/s", HBM_PEAK_GBS, "hbm")
-    if is_gemm:  # nbytes holds FLOPs for the GEMM workloads; report TFLOP/s
-        value, achieved = value / 1e3, achieved / 1e3
-    out = {
-        "metric": "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms",
-        "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp8" if is_gemm else "f32", "data": "synthetic", "config": cfg,
-        "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload) if args.shape == [4096, 4096] else None,
-                     ("algorithmic_flops_per_launch" if is_gemm else "algorithmic_bytes_per_launch"): nbytes, "kernel_ms_avg": round(avg_ms, 5),
-                     "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
-                     "kernel_ms_per_launch_events_avg": round(sum(kern_ms) / len(kern_ms), 5),
-                     "kernel_ms_p20": round(kern_ms[len(kern_ms) // 5], 5), "kernel_ms_p80": round(kern_ms[(4 * len(kern_ms)) // 5], 5)},
-    }
-    if args.workload == "adamw" and not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_adamw(torch)
-    elif args.workload in ("quantize", "quantize_transpose") and not args.no_cpu_baseline and args.shape == [4096, 4096]:
-        out["cpu_baseline"] = cpu_baseline_quantize(torch, args.workload == "quantize_transpose", nbytes)
-    else:
-        out["cpu_baseline"] = None
+    def measure(name):
+        fn = measure_layer if name in LAYER_WORKLOADS else measure_stream
+        rec = fn(name, args, dev, torch, cpu)
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        return rec
+
+    head = measure("adamw_class" if args.workload == "all" else args.workload)
+    out = {"metric": METRIC, "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": head["higher_is_better"],
+           "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic", "config": head["config"]}
+    if "layer" in head:
+        out["layer"] = head["layer"]
+    out["roofline"] = head["roofline"]
+    out["cpu_baseline"] = head["cpu_baseline"]
+    if args.workload == "all":
+        # the other legs of the metric, each timed exactly like a run with --workload <name>
+        out["extra"] = {}
+        for name in EXTRAS:
+            r = measure(name)
+            out["extra"][name] = {k: r[k] for k in ("value", "unit", "ms_per_step", "dtype", "roofline", "cpu_baseline") if k in r}
+            out["extra"][name]["workload"] = r["config"]["workload"]
+            if "layer" in r:
+                out["extra"][name]["layer"] = r["layer"]
     print(json.dumps(out))
 
 
