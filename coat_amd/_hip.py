@@ -12,6 +12,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcoat_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
+MAX_SLOTS, MAX_SLOT_STRIDE = 16, 32  # COAT_MAX_SLOTS, COAT_MAX_SLOT_STRIDE of include/coat_hip.h
+MAX_WORDS = MAX_SLOTS * MAX_SLOT_STRIDE
 E4M3, E5M2 = 0, 1
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}

@@ -3,7 +3,7 @@ Reference: coat/activation/real_quantization/_division.py:153-207."""
 import torch
 
 from ... import _hip
-from .common import FP8_MAX_VALUE, SCALE_MIN_THRES, as_fp8_dtype, flatten_2d, new_max, restore
+from .common import FP8_MAX_VALUE, SCALE_MIN_THRES, as_fp8_dtype, flatten_2d, new_max, read_max, restore
 
 # the seed the reference's kernels pass to tl.rand (reference :110; _division_transpose.py:117)
 STOCHASTIC_SEED = 0
@@ -13,31 +13,32 @@ def absmax_scale(x, fp8type):
     """(x.abs().max() + 1e-10) / fp8max in x's dtype (reference :178-179), one pass over x."""
     amax = new_max(x.device)
     _hip.check(_hip.lib().coat_absmax(_hip.ptr(x), _hip.dt(x), _hip.ptr(amax), x.numel(), _hip.stream(x.device)), "absmax")
-    return (amax.to(x.dtype) + SCALE_MIN_THRES) / FP8_MAX_VALUE[fp8type]
+    return (read_max(amax).to(x.dtype) + SCALE_MIN_THRES) / FP8_MAX_VALUE[fp8type]
 
 
 def _division(x, fp8type, s_y, want_q, want_qt, what, stochastic=False, max_as=None):
-    """q and / or q^T of x divided by a per-tensor scale.  ``max_as`` (a torch dtype): ``s_y`` is the fp32 device
-    scalar into which a producer kernel merged the maximum of its group scales; the division kernel rounds it to that
-    dtype itself and writes the rounded scale, which is returned (no separate conversion launch)."""
+    """q and / or q^T of x divided by a per-tensor scale.  ``max_as`` (a torch dtype): ``s_y`` is the fp32 buffer
+    (``new_max``) into which a producer kernel merged the maximum of its group scales; the division kernel rounds the
+    maximum to that dtype itself and writes the rounded scale, which is returned (no separate conversion launch)."""
     M, N = x.shape
     if s_y is None:
         s_y = absmax_scale(x, fp8type)
-    if s_y.numel() != 1:
+    if max_as is not None and (stochastic or M * N == 0):
+        s_y = read_max(s_y).to(max_as)  # the kernel that reads the slots itself is not used on this path
+        max_as = None
+    if max_as is None and s_y.numel() != 1:
         raise ValueError(f"{what}: the scale must be a single element, got shape {tuple(s_y.shape)}")
     s_dev = s_y if s_y.is_cuda else s_y.to(x.device)
     y = torch.empty_like(x, dtype=fp8type) if want_q else None
     y_t = torch.empty((N, M), dtype=fp8type, device=x.device) if want_qt else None
-    if max_as is not None and not stochastic and M * N > 0:
-        if s_dev.dtype != torch.float32:
+    if max_as is not None:
+        if s_dev.dtype != torch.float32 or s_dev.numel() != _hip.MAX_WORDS:
             raise ValueError(f"{what}: the running maximum must be fp32")
         s_out = torch.empty((), dtype=max_as, device=x.device)
         _hip.check(_hip.lib().coat_fp8_division_from_max(
             _hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.ptr(s_out), _hip.dt(s_out), _hip.ptr(y), _hip.ptr(y_t), M, N,
             _hip.fp8(fp8type), _hip.stream(x.device)), what)
         return y, s_out, y_t
-    if max_as is not None:
-        s_y = s_dev = s_dev.to(max_as)
     if stochastic:
         _hip.check(_hip.lib().coat_fp8_division_stochastic(
             _hip.ptr(x), _hip.dt(x), _hip.ptr(s_dev), _hip.dt(s_dev), _hip.ptr(y), _hip.ptr(y_t), M, N,

@@ -45,23 +45,32 @@ def no_stochastic(stochastic, why):
 
 
 _MAX_POOL = {}
-_MAX_POOL_SIZE = 1024
+_MAX_POOL_SIZE = 64
 
 
 def new_max(device):
-    """Zero-initialised fp32 device scalar for the order-independent atomic maximum of the group scales.
+    """Zero-initialised buffer for the order-independent device-wide maximum of the group scales: ``_hip.MAX_WORDS`` fp32
+    words, 16 slots one 128-byte line apart (include/coat_hip.h, COAT_MAX_WORDS); ``read_max`` gives the maximum.
 
-    Scalars are handed out from a zero-filled pool (one fill kernel per 1024 of them instead of one each; a slot is
-    never reused, and the pool lives as long as any of its slots).  Pools are kept per device and stream, so a slot is
-    always used on the stream that zeroed it."""
+    Buffers are handed out from a zero-filled pool (one fill kernel per 64 of them instead of one each; a buffer is
+    never reused, and the pool lives as long as any of its buffers).  Pools are kept per device and stream, so a buffer
+    is always used on the stream that zeroed it."""
+    from ... import _hip
     device = torch.device(device)
     if device.type != "cuda":
-        return torch.zeros((), dtype=torch.float32, device=device)
+        return torch.zeros(_hip.MAX_WORDS, dtype=torch.float32, device=device)
     key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
     pool = _MAX_POOL.get(key)
     if pool is None or pool[1] >= _MAX_POOL_SIZE:
-        pool = [torch.zeros(_MAX_POOL_SIZE, dtype=torch.float32, device=device), 0]
+        pool = [torch.zeros(_MAX_POOL_SIZE * _hip.MAX_WORDS, dtype=torch.float32, device=device), 0]
         _MAX_POOL[key] = pool
     i = pool[1]
     pool[1] = i + 1
-    return pool[0][i]
+    return pool[0][i * _hip.MAX_WORDS:(i + 1) * _hip.MAX_WORDS]
+
+
+def read_max(buf):
+    """The maximum held by a ``new_max`` buffer, as a 0-dim fp32 tensor (for host-side code; the division kernels read
+    the slots themselves)."""
+    from ... import _hip
+    return buf[::_hip.MAX_SLOT_STRIDE].max()

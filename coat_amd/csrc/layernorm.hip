@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void k_layernorm_fwd(const uint8_t* __restrict
         ((uint16_t*)s_row)[row] = (uint16_t)f2bf16(sr);
         mean_out[row] = mean;
         rstd_out[row] = rstd;
-        atomic_max_nonneg(s_max, sr);
+        atomic_max_nonneg(max_slot(s_max), sr);
     }
 }
 

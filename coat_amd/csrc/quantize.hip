@@ -160,12 +160,13 @@ __global__ __launch_bounds__(256) void k_absmax(const void* __restrict__ x, floa
 }
 
 // The per-tensor scale of a division kernel.  s_out == NULL: *s_ptr is the scale, an element of dtype SDT.  Otherwise
-// *s_ptr is the fp32 maximum of the group scales left by the producer kernel's atomics: it is rounded to SDT here (what
+// s_ptr holds the slots of the fp32 maximum of the group scales left by the producer kernel's atomics (max over the slots =
+// the maximum): it is rounded to SDT here (what
 // the reference's ``s.max()`` over the stored scales gives, rounding being monotone) and the first thread of the grid
 // stores the rounded value to s_out for the consumers, which saves a separate conversion launch per tensor.
 template <int SDT> __device__ __forceinline__ float load_scale_or_max(const void* s_ptr, void* s_out) {
     if (!s_out) return load_as_f32<SDT>(s_ptr, 0);
-    const float s = round_to<SDT>(((const float*)s_ptr)[0]);
+    const float s = round_to<SDT>(load_max((const float*)s_ptr));
     if (blockIdx.x == 0 && threadIdx.x == 0) store_from_f32<SDT>(s_out, 0, s);
     return s;
 }

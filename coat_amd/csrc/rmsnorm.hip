@@ -20,7 +20,7 @@ namespace coat {
 
 // Forward: y = bf16(x * rstd * w), rstd[row], row scale (max|y| + 1e-10)/fp8max (bf16), tensor max of the row scales.
 template <int KIND, int WDT, int ITERS>
-__global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+__global__ __launch_bounds__(256) void k_rmsnorm_fwd_block(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
                                                       const void* __restrict__ w, void* __restrict__ y,
                                                       void* __restrict__ s_row, float* __restrict__ rstd_out,
                                                       float* __restrict__ s_max, int N, int qb, float eps) {
@@ -60,13 +60,13 @@ __global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__
         const float sr = group_scale<KIND>(amax);
         ((uint16_t*)s_row)[row] = (uint16_t)f2bf16(sr);
         rstd_out[row] = rstd;
-        atomic_max_nonneg(s_max, sr);
+        atomic_max_nonneg(max_slot(s_max), sr);
     }
 }
 
 // Backward: dx = bf16((w*dy - xhat * mean(xhat*w*dy)) * rstd); per-block partial of dw = sum_rows dy * xhat.
 template <int KIND, int WDT, int ITERS>
-__global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+__global__ __launch_bounds__(256) void k_rmsnorm_bwd_block(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
                                                       const void* __restrict__ dy, const void* __restrict__ dy2,
                                                       const void* __restrict__ dy3, const void* __restrict__ w,
                                                       const float* __restrict__ rstd_in, void* __restrict__ dx,
@@ -135,6 +135,260 @@ __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------ one wave per row
+// Rows up to 8192 columns.  A wave owns whole rows: lane l holds the 16-element chunks c * 64 + l (c < CH), so every load
+// instruction of the wave covers 1 KiB of consecutive codes, all loads of a row are in flight before the first
+// conversion, the next row's codes are requested before the current row is reduced (forward), and nothing waits at a
+// block-wide barrier.  The weight stays in registers for all rows of the wave.
+// The row sums are formed exactly as the block-per-row kernels above form them (chunk c belongs to "wave" c & 3 of that
+// kernel: in-lane running sum over c, c + 4, ..., one butterfly per partial, the four partials added in index order),
+// so rstd, dx and every code derived from them are bit-identical between the two layouts.
+template <int CH> struct RowRaw {
+    uint4 codes[CH];
+    uint32_t sc[CH];
+};
+template <int CH>
+__device__ __forceinline__ void load_row(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt, int64_t row, int N,
+                                         int qb, int lane, RowRaw<CH>& r) {
+    const uint8_t* qr = q + row * N;
+    const int64_t srow = row * (N / qb);
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int col = (c * 64 + lane) * 16;
+        if (col < N) {
+            r.codes[c] = *(const uint4*)(qr + col);
+            const int64_t si = srow + col / qb;
+            r.sc[c] = s_dt == kF32 ? ((const uint32_t*)s)[si] : (uint32_t)((const uint16_t*)s)[si];
+        }
+    }
+}
+__device__ __forceinline__ float scale_from_raw(uint32_t u, int s_dt) {
+    if (s_dt == kBF16) return u2f(u << 16);
+    if (s_dt == kF32) return u2f(u);
+    return f16lo(u);
+}
+template <int KIND> __device__ __forceinline__ void decode16(const uint4& c, float sc, float* v) {
+    const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float f[4];
+        fp8x4_to_f32<KIND>(w[k], f);
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[4 * k + i] = f[i] * sc;
+    }
+}
+template <int WDT> __device__ __forceinline__ void unpack_w16(const uint4* p, float* o) {
+    const uint32_t u[8] = {p[0].x, p[0].y, p[0].z, p[0].w, p[1].x, p[1].y, p[1].z, p[1].w};
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        o[2 * k] = WDT == kBF16 ? bf16lo(u[k]) : f16lo(u[k]);
+        o[2 * k + 1] = WDT == kBF16 ? bf16hi(u[k]) : f16hi(u[k]);
+    }
+}
+// the four partial sums of a row, reduced and added in the block-per-row kernel's order
+__device__ __forceinline__ float row_sum4(float* part) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) part[k] = cluster_sum<64>(part[k]);
+    return ((part[0] + part[1]) + part[2]) + part[3];
+}
+
+template <int KIND, int WDT, int CH>
+__global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                      const void* __restrict__ w, void* __restrict__ y,
+                                                      void* __restrict__ s_row, float* __restrict__ rstd_out,
+                                                      float* __restrict__ s_max, int64_t M, int N, int qb, float eps) {
+    constexpr bool HOLD_W = WDT != kF32;  // 8 registers per chunk; an fp32 weight is re-read from the cache per row
+    const int lane = threadIdx.x & 63;
+    const int64_t nwaves = (int64_t)gridDim.x * 4;
+    int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    uint4 wreg[HOLD_W ? CH : 1][2];
+    if (HOLD_W) {
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * 16;
+            if (col < N) {
+                const uint4* wp = (const uint4*)((const uint16_t*)w + col);
+                wreg[c][0] = wp[0];
+                wreg[c][1] = wp[1];
+            }
+        }
+    }
+    RowRaw<CH> cur, nxt;
+    if (row < M) load_row<CH>(q, s, s_dt, row, N, qb, lane, cur);
+    float wave_max = 0.0f;
+    while (row < M) {
+        const int64_t nrow = row + nwaves;
+        if (nrow < M) load_row<CH>(q, s, s_dt, nrow, N, qb, lane, nxt);
+        float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            if ((c * 64 + lane) * 16 < N) {
+                float x[16];
+                decode16<KIND>(cur.codes[c], scale_from_raw(cur.sc[c], s_dt), x);
+#pragma unroll
+                for (int i = 0; i < 16; i++) part[c & 3] += x[i] * x[i];
+            }
+        }
+        const float var = row_sum4(part) / (float)N;
+        const float rstd = 1 / sqrtf(var + eps);
+        float amax = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * 16;
+            if (col < N) {
+                float x[16], wv[16], yv[16];
+                decode16<KIND>(cur.codes[c], scale_from_raw(cur.sc[c], s_dt), x);
+                if (HOLD_W) unpack_w16<WDT>(wreg[c], wv);
+                else load_w16<WDT>(w, col, wv);
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    yv[i] = (x[i] * rstd) * wv[i];
+                    amax = fmaxf(amax, fabsf(yv[i]));
+                }
+                if (y) store_bf16_16(y, row * N + col, yv);  // NULL: statistics only (the division recomputes y)
+            }
+        }
+        amax = cluster_max<64>(amax);
+        const float sr = group_scale<KIND>(amax);
+        wave_max = fmaxf(wave_max, sr);
+        if (lane == 0) {
+            ((uint16_t*)s_row)[row] = (uint16_t)f2bf16(sr);
+            rstd_out[row] = rstd;
+        }
+        cur = nxt;
+        row = nrow;
+    }
+    // one lazy atomic per block (waves without rows hold 0)
+    __shared__ float wmax[4];
+    if (lane == 0) wmax[threadIdx.x >> 6] = wave_max;
+    __syncthreads();
+    if (threadIdx.x == 0) atomic_max_nonneg(max_slot(s_max), fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3])));
+}
+
+// Backward, one wave per row.  A block's four waves keep fp32 weight-gradient sums for the rows they walked; at the end
+// they are added in wave order through LDS, 1024 columns at a time, into the block's partial row.
+template <int KIND, int WDT, int CH>
+__global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                      const void* __restrict__ dy, const void* __restrict__ dy2,
+                                                      const void* __restrict__ dy3, const void* __restrict__ w,
+                                                      const float* __restrict__ rstd_in, void* __restrict__ dx,
+                                                      float* __restrict__ dw_partial, int64_t M, int N, int qb) {
+    constexpr bool HOLD_W = WDT != kF32;
+    __shared__ float red[4][64 * 16];
+    const int lane = threadIdx.x & 63, wv_id = threadIdx.x >> 6;
+    const int64_t nwaves = (int64_t)gridDim.x * 4;
+    uint4 wreg[HOLD_W ? CH : 1][2];
+    if (HOLD_W) {
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * 16;
+            if (col < N) {
+                const uint4* wp = (const uint4*)((const uint16_t*)w + col);
+                wreg[c][0] = wp[0];
+                wreg[c][1] = wp[1];
+            }
+        }
+    }
+    float acc[CH][16];
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[c][i] = 0.0f;
+    for (int64_t row = (int64_t)blockIdx.x * 4 + wv_id; row < M; row += nwaves) {
+        const int64_t row_off = row * N;
+        RowRaw<CH> raw;
+        uint4 g[CH][2];  // the (summed) gradient as packed bf16: exact, it is a bf16 value
+        load_row<CH>(q, s, s_dt, row, N, qb, lane, raw);
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * 16;
+            if (col < N) {
+                const uint4* gp = (const uint4*)((const uint16_t*)dy + row_off + col);
+                g[c][0] = gp[0];
+                g[c][1] = gp[1];
+            }
+        }
+        const float rstd = rstd_in[row];
+        if (dy2) {
+            // further gradients of the same tensor, summed the way a chain of bf16 tensor additions would:
+            // (dy + dy2) rounded to bf16, then + dy3 rounded to bf16 (wave-uniform branches)
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                const int col = (c * 64 + lane) * 16;
+                if (col < N) {
+                    float a[16], b[16];
+                    load_bf16_16(dy2, row_off + col, b);
+                    unpack_w16<kBF16>(g[c], a);
+#pragma unroll
+                    for (int i = 0; i < 16; i++) a[i] = round_to<kBF16>(a[i] + b[i]);
+                    if (dy3) {
+                        load_bf16_16(dy3, row_off + col, b);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) a[i] = round_to<kBF16>(a[i] + b[i]);
+                    }
+                    uint32_t pk[8];
+#pragma unroll
+                    for (int k = 0; k < 8; k++) pk[k] = pack_bf16x2(a[2 * k], a[2 * k + 1]);
+                    g[c][0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                    g[c][1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+                }
+            }
+        }
+        float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * 16;
+            if (col < N) {
+                float xv[16], wvv[16], gv[16];
+                decode16<KIND>(raw.codes[c], scale_from_raw(raw.sc[c], s_dt), xv);
+                if (HOLD_W) unpack_w16<WDT>(wreg[c], wvv);
+                else load_w16<WDT>(w, col, wvv);
+                unpack_w16<kBF16>(g[c], gv);
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const float xhat = xv[i] * rstd;
+                    const float wdy = wvv[i] * gv[i];
+                    part[c & 3] += xhat * wdy;
+                    acc[c][i] += gv[i] * xhat;
+                }
+            }
+        }
+        const float c1 = row_sum4(part) / (float)N;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int col = (c * 64 + lane) * 16;
+            if (col < N) {
+                float xv[16], wvv[16], gv[16], o[16];
+                decode16<KIND>(raw.codes[c], scale_from_raw(raw.sc[c], s_dt), xv);
+                if (HOLD_W) unpack_w16<WDT>(wreg[c], wvv);
+                else load_w16<WDT>(w, col, wvv);
+                unpack_w16<kBF16>(g[c], gv);
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[i] = ((wvv[i] * gv[i]) - ((xv[i] * rstd) * c1)) * rstd;
+                store_bf16_16(dx, row_off + col, o);
+            }
+        }
+    }
+    // the block's partial row: waves added in index order, 1024 columns per round
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        float4* mine = (float4*)&red[wv_id][lane * 16];
+#pragma unroll
+        for (int k = 0; k < 4; k++) mine[k] = make_float4(acc[c][4 * k], acc[c][4 * k + 1], acc[c][4 * k + 2], acc[c][4 * k + 3]);
+        __syncthreads();
+        const int e = threadIdx.x * 4, col = c * 1024 + e;
+        if (col < N) {
+            const float4 a0 = *(const float4*)&red[0][e], a1 = *(const float4*)&red[1][e], a2 = *(const float4*)&red[2][e],
+                         a3 = *(const float4*)&red[3][e];
+            *(float4*)(dw_partial + (int64_t)blockIdx.x * N + col) =
+                make_float4(((a0.x + a1.x) + a2.x) + a3.x, ((a0.y + a1.y) + a2.y) + a3.y, ((a0.z + a1.z) + a2.z) + a3.z,
+                            ((a0.w + a1.w) + a2.w) + a3.w);
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace coat
 
 using namespace coat;
@@ -146,28 +400,13 @@ static int rms_check(int64_t M, int64_t N, int QB) {
     return COAT_OK;
 }
 
-#define RMS_DISPATCH(KERNEL, GRID, ...)                                                                                \
-    {                                                                                                                  \
-        const int iters = N <= 4096 ? 1 : (N <= 8192 ? 2 : 4);                                                         \
-        if (fp8 != COAT_E4M3 && fp8 != COAT_E5M2) return COAT_EINVAL;                                                  \
-        if (w_dtype != COAT_BF16 && w_dtype != COAT_F32 && w_dtype != COAT_F16) return COAT_EDTYPE;                    \
-        switch ((fp8 * 3 + w_dtype) * 3 + (iters == 1 ? 0 : (iters == 2 ? 1 : 2))) {                                   \
-            RMS_CASES(KERNEL, GRID, __VA_ARGS__)                                                                       \
-            default: return COAT_EINVAL;                                                                               \
-        }                                                                                                              \
-    }
-#define RMS_CASE(KERNEL, GRID, K, W, I, ...)                                                                           \
-    case ((K * 3 + W) * 3 + (I == 1 ? 0 : (I == 2 ? 1 : 2))):                                                          \
-        hipLaunchKernelGGL((KERNEL<K, W, I>), dim3((unsigned)(GRID)), dim3(256), 0, st, __VA_ARGS__);                  \
-        break;
-#define RMS_CASES(KERNEL, GRID, ...)                                                                                   \
-    RMS_CASE(KERNEL, GRID, 0, 0, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 0, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 0, 4, __VA_ARGS__) \
-    RMS_CASE(KERNEL, GRID, 0, 1, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 1, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 1, 4, __VA_ARGS__) \
-    RMS_CASE(KERNEL, GRID, 0, 2, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 2, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 0, 2, 4, __VA_ARGS__) \
-    RMS_CASE(KERNEL, GRID, 1, 0, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 0, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 0, 4, __VA_ARGS__) \
-    RMS_CASE(KERNEL, GRID, 1, 1, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 1, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 1, 4, __VA_ARGS__) \
-    RMS_CASE(KERNEL, GRID, 1, 2, 1, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 2, 2, __VA_ARGS__) RMS_CASE(KERNEL, GRID, 1, 2, 4, __VA_ARGS__)
-
+// Rows up to 8192 columns go to the wave-per-row kernels (CH = 4 or 8 chunks of 16 per lane), wider rows (up to 16384) to
+// the block-per-row kernels.  KW = fp8 kind * 3 + weight dtype.
+constexpr int kRmsFwdMaxBlocks = 1024;  // x 4 waves: about two rows per wave at 8192 rows, the second prefetched under the first
+#define RMS_KW_CASES(X) X(0, 0) X(0, 1) X(0, 2) X(1, 0) X(1, 1) X(1, 2)
+#define RMS_CHECK_ENUMS()                                                                                   \
+    if (fp8 != COAT_E4M3 && fp8 != COAT_E5M2) return COAT_EINVAL;                                           \
+    if (w_dtype != COAT_BF16 && w_dtype != COAT_F32 && w_dtype != COAT_F16) return COAT_EDTYPE;
 extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype,
                                         void* y, void* s_row, float* rstd, float* s_max, int64_t M, int64_t N, int QB,
                                         float eps, void* stream) {
@@ -176,7 +415,25 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
     if (!x || !s_x || !w || !s_row || !rstd || !s_max) return COAT_EINVAL;  // y may be NULL
     if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(y)) return COAT_EALIGN;
     hipStream_t st = (hipStream_t)stream;
-    RMS_DISPATCH(k_rmsnorm_fwd, M, (const uint8_t*)x, s_x, s_dtype, w, y, s_row, rstd, s_max, (int)N, QB, eps)
+    RMS_CHECK_ENUMS()
+    const int64_t wave_blocks = (M + 3) / 4 < kRmsFwdMaxBlocks ? (M + 3) / 4 : kRmsFwdMaxBlocks;
+#define RMS_FWD(K, W)                                                                                                  \
+    case K * 3 + W:                                                                                                    \
+        if (N <= 4096)                                                                                                 \
+            hipLaunchKernelGGL((k_rmsnorm_fwd<K, W, 4>), dim3((unsigned)wave_blocks), dim3(256), 0, st, (const uint8_t*)x, s_x, \
+                               s_dtype, w, y, s_row, rstd, s_max, M, (int)N, QB, eps);                                 \
+        else if (N <= 8192)                                                                                            \
+            hipLaunchKernelGGL((k_rmsnorm_fwd<K, W, 8>), dim3((unsigned)wave_blocks), dim3(256), 0, st, (const uint8_t*)x, s_x, \
+                               s_dtype, w, y, s_row, rstd, s_max, M, (int)N, QB, eps);                                 \
+        else                                                                                                           \
+            hipLaunchKernelGGL((k_rmsnorm_fwd_block<K, W, 4>), dim3((unsigned)M), dim3(256), 0, st, (const uint8_t*)x, s_x, \
+                               s_dtype, w, y, s_row, rstd, s_max, (int)N, QB, eps);                                    \
+        break;
+    switch (fp8 * 3 + w_dtype) {
+        RMS_KW_CASES(RMS_FWD)
+        default: return COAT_EINVAL;
+    }
+#undef RMS_FWD
     return coat_launch_status();
 }
 
@@ -184,8 +441,29 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
 static int rms_backward_launch(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
                                const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
                                float* dw_partial, int64_t n_partial, int64_t M, int64_t N, int QB, hipStream_t st) {
-    const int64_t grid = n_partial < M ? n_partial : M;
-    RMS_DISPATCH(k_rmsnorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB)
+    RMS_CHECK_ENUMS()
+    // one partial row per block: min(n_partial, M) blocks of the block-per-row kernel, min(n_partial, ceil(M / 4)) blocks
+    // of four row-owning waves otherwise
+    const int64_t rows_per_block = N <= 8192 ? 4 : 1;
+    const int64_t want = (M + rows_per_block - 1) / rows_per_block;
+    const int64_t grid = n_partial < want ? n_partial : want;
+#define RMS_BWD(K, W)                                                                                                  \
+    case K * 3 + W:                                                                                                    \
+        if (N <= 4096)                                                                                                 \
+            hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, 4>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, s_dtype, \
+                               dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB);                                  \
+        else if (N <= 8192)                                                                                            \
+            hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, 8>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, s_dtype, \
+                               dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB);                                  \
+        else                                                                                                           \
+            hipLaunchKernelGGL((k_rmsnorm_bwd_block<K, W, 4>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, \
+                               s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB);                         \
+        break;
+    switch (fp8 * 3 + w_dtype) {
+        RMS_KW_CASES(RMS_BWD)
+        default: return COAT_EINVAL;
+    }
+#undef RMS_BWD
     if (int e = coat_launch_status()) return e;
     const int cols_blocks = (int)((N + 15) / 16);
     switch (w_dtype) {

@@ -35,6 +35,16 @@ enum coat_status {
 enum coat_dtype { COAT_F32 = 0, COAT_BF16 = 1, COAT_F16 = 2 };
 enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.float8_e5m2 (rq/common.py:22-27) */
 
+/* The device-wide maximum that links a producer kernel to the per-tensor division after it ("s_max", "amax" below) is not
+ * one word but COAT_MAX_WORDS fp32 words: COAT_MAX_SLOTS slots, one 128-byte line apart (atomics on one line are carried
+ * out one at a time; spreading the blocks of a launch over 16 lines takes their serialisation out of the kernel's
+ * duration).  The caller zero-fills the buffer (or leaves a previous partial maximum in it); block b of a producer merges
+ * into word COAT_MAX_SLOT_STRIDE * (b % COAT_MAX_SLOTS); the maximum is the largest of those COAT_MAX_SLOTS words, which
+ * is what the consuming entry points (coat_fp8_division_from_max, coat_fp8_*_division) compute for themselves. */
+#define COAT_MAX_SLOTS 16
+#define COAT_MAX_SLOT_STRIDE 32
+#define COAT_MAX_WORDS (COAT_MAX_SLOTS * COAT_MAX_SLOT_STRIDE)
+
 const char* coat_version(void);
 const char* coat_status_string(int status);
 /* Memory-bandwidth probe for the benchmarks (no counterpart in the reference): kind 0 copies bytes from src to dst,
@@ -54,14 +64,14 @@ int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, void* s, vo
                                 int64_t M, int64_t N, int QB, int fp8, void* stream);
 
 /* rq/_quantize_pertensor.py:46-103 (+ the `s_y.max()` at :139): per-group scales and their maximum.
- * s_pg [M,N/QB] s_dtype (may be NULL when only the maximum is wanted); s_max: one fp32 in device
- * memory that must hold 0.0f (or a previous partial maximum) on entry and receives max(s32) by
- * atomic max; round it to s_dtype to obtain the reference's `s_y.max()`. */
+ * s_pg [M,N/QB] s_dtype (may be NULL when only the maximum is wanted); s_max: COAT_MAX_WORDS fp32 in device
+ * memory that must hold 0.0f (or a previous partial maximum) on entry and receive max(s32) by
+ * atomic max; the largest of the slots, rounded to s_dtype, is the reference's `s_y.max()`. */
 int coat_fp8_group_scales(const void* x, int x_dtype, void* s_pg, int s_dtype, float* s_max, int64_t M, int64_t N,
                           int QB, int fp8, void* stream);
 
 /* rq/_division.py:178-179: s = (x.abs().max() + 1e-10) / fp8max evaluated in x's dtype.
- * amax: one fp32 in device memory holding 0.0f on entry; receives max|x| by atomic max. */
+ * amax: COAT_MAX_WORDS fp32 in device memory holding 0.0f on entry; the slots receive max|x| by atomic max. */
 int coat_absmax(const void* x, int x_dtype, float* amax, int64_t numel, void* stream);
 
 /* rq/_division.py:153 fp8_division (kernel :45-126, non-stochastic) and
@@ -71,8 +81,8 @@ int coat_absmax(const void* x, int x_dtype, float* amax, int64_t numel, void* st
 int coat_fp8_division(const void* x, int x_dtype, const void* s, int s_dtype, void* q, void* qt, int64_t M,
                       int64_t N, int fp8, void* stream);
 
-/* The same division fed with the producer kernel's fp32 maximum of the group scales (the word that
- * coat_fp8_group_scales and the fused kernels merge their atomics into): the kernel rounds *s_max to s_dtype, divides by
+/* The same division fed with the producer kernel's fp32 maximum of the group scales (the COAT_MAX_WORDS buffer that
+ * coat_fp8_group_scales and the fused kernels merge their atomics into): the kernel rounds the maximum to s_dtype, divides by
  * that value and stores it to s_out (one element of s_dtype) for the consumers.  Replaces "convert the maximum to bf16 on
  * the host side, then divide" (the reference's s_y.max() at rq/_quantize_pertensor.py:139 and the like) by one launch. */
 int coat_fp8_division_from_max(const void* x, int x_dtype, const float* s_max, void* s_out, int s_dtype, void* q, void* qt,
@@ -96,8 +106,8 @@ int coat_fp8_dequantize(const void* q, int fp8, const void* s, int s_dtype, void
 /* ---- fused element-wise kernels -----------------------------------------------------------------
  * Inputs x* are per-group FP8 ([M,N] codes + [M,N/QB] scales of s_dtype); g is a bf16 gradient.
  * "value" outputs y are bf16 [M,N]; s_y (optional, may be NULL) receives the bf16 per-group scales
- * (amax_g + 1e-10) / fp8max(fp8_out) of the fp32 value; s_max (optional) is a zero-initialised fp32 device
- * scalar that receives their maximum (the per-tensor scale of the division that follows in the reference). */
+ * (amax_g + 1e-10) / fp8max(fp8_out) of the fp32 value; s_max (optional) is a zero-initialised buffer of COAT_MAX_WORDS
+ * fp32 that receives their maximum (the per-tensor scale of the division that follows in the reference). */
 
 /* rq/silu_fwd.py:152 fp8_silu_forward (kernel :47-149): y = per-group fp8(silu(x)), same fp8 type as x. */
 int coat_fp8_silu_forward(const void* x, int fp8, const void* s_x, int s_dtype, void* y, void* s_y, int64_t M,
@@ -160,7 +170,7 @@ int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x, int s_dtyp
 /* The per-tensor division + transpose that ends rq/func_rmsnorm.py:223 (its fp8_division_transpose call at :269),
  * fed with the norm's inputs: every tile of y = bf16(x * rstd * w) is recomputed in registers with the forward kernel's
  * expressions, so q / qt equal those of coat_fp8_division_from_max on the stored y, and y is never written or read.
- * s_max: the fp32 maximum left by coat_fp8_rmsnorm_forward; s_out: one bf16 element, the rounded scale.
+ * s_max: the COAT_MAX_WORDS buffer filled by coat_fp8_rmsnorm_forward; s_out: one bf16 element, the rounded scale.
  * M % 16 == 0, N % 16 == 0, QB % 16 == 0; q / qt in the format of x. */
 int coat_fp8_rmsnorm_division(const void* x, int fp8, const void* s_x, int s_dtype, const void* w, int w_dtype,
                               const float* rstd, const float* s_max, void* s_out, void* q, void* qt, int64_t M, int64_t N,

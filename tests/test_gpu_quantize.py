@@ -197,13 +197,16 @@ def test_default_division_scale_is_the_device_expression(dev, dtype):
 @pytest.mark.parametrize("sdtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("shape", [(64, 128), (7, 37)])
 def test_division_from_fp32_max_equals_division_by_rounded_scale(dev, sdtype, shape):
-    """coat_fp8_division_from_max rounds the fp32 maximum to the scale dtype, divides by that value and stores it."""
+    """coat_fp8_division_from_max takes the largest of the maximum's slots (COAT_MAX_WORDS fp32, one slot per 128-byte line),
+    rounds it to the scale dtype, divides by that value and stores it."""
     from coat_amd import _hip
     M, N = shape
     x = make_x(M, N, 11, torch.bfloat16).to(dev)
     for m in (0.0123456789, 3.1e-7, 1.0):
-        s_max = torch.tensor(m, dtype=torch.float32, device=dev)
-        want_s = s_max.to(sdtype)
+        s_max = torch.zeros(_hip.MAX_WORDS, dtype=torch.float32, device=dev)
+        s_max[::_hip.MAX_SLOT_STRIDE] = torch.linspace(0.1, 1.0, _hip.MAX_SLOTS, device=dev).roll(5) * m  # largest in slot 4
+        s_max[1::_hip.MAX_SLOT_STRIDE] = 7.0  # words between the slots are not part of the maximum
+        want_s = torch.tensor(m, dtype=torch.float32, device=dev).to(sdtype)
         tr = M % 16 == 0 and N % 16 == 0
         q, qt = torch.empty((M, N), dtype=torch.uint8, device=dev), torch.empty((N, M), dtype=torch.uint8, device=dev)
         wq, wqt = torch.empty_like(q), torch.empty_like(qt)
