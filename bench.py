@@ -669,6 +669,52 @@ def ramp_clocks(step, seconds, torch):
         torch.cuda.synchronize()
 
 
+def gemm_clock(dev, torch):
+    """The shader clock the FP8 GEMM really runs at.  Needs a probe build of the library:
+        COAT_HIPCC_FLAGS=-DCOAT_GEMM_PROBE COAT_LIB_OUT=/tmp/libcoat_probe.so python -m coat_amd.build
+        COAT_HIP_LIB=/tmp/libcoat_probe.so python bench.py --workload gemm_clock
+    Every block of k_fp8_gemm records its duration in shader clocks (s_memtime) and in ticks of the constant 100 MHz
+    counter (s_memrealtime); their ratio is the clock.  Operands N(0, 1) as in the gemm_* workloads, and all zeros."""
+    import ctypes
+
+    from coat_amd import _hip
+    from coat_amd.activation.real_quantization.linear import fp8matmul
+    L = _hip.lib()
+    if not hasattr(L, "coat_gemm_set_probe"):
+        print("bench.py: --workload gemm_clock needs a library built with -DCOAT_GEMM_PROBE (see the docstring)", file=sys.stderr)
+        sys.exit(4)
+    probe = torch.zeros(2 * 256, dtype=torch.int64, device=dev)
+    L.coat_gemm_set_probe.argtypes = [ctypes.c_void_p]
+    L.coat_gemm_set_probe.restype = None
+    L.coat_gemm_set_probe(ctypes.c_void_p(probe.data_ptr()))
+    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+    one = torch.tensor(0.01, dtype=torch.bfloat16, device=dev)
+    out = {}
+    for name, (M, N, K), fa, zero in (("fwd", (8192, 11008, 4096), E4, False), ("dgrad", (8192, 4096, 11008), E5, False),
+                                      ("wgrad", (11008, 4096, 8192), E5, False), ("dgrad_zero_operands", (8192, 4096, 11008), E5, True)):
+        a = (torch.zeros if zero else torch.randn)(M, K, device=dev).to(fa)
+        b = (torch.zeros if zero else torch.randn)(N, K, device=dev).to(E4)
+        step = lambda: fp8matmul(a, b.t(), False, one, one, 16)  # noqa: E731
+        ramp_clocks(step, 2.0, torch)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record()
+        for _ in range(50):
+            step()
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / 50
+        p = probe.cpu().view(-1, 2).double()
+        tiles = ((M + 255) // 256) * ((N + 255) // 256)
+        ideal = tiles * ((K + 127) // 128) * 2048 / 256  # MFMA clocks per CU if the matrix pipes never waited
+        mhz = p[:, 0] / p[:, 1] * 100.0
+        out[name] = {"us_per_launch": round(ms * 1e3, 1), "tflops": round(2 * M * N * K / ms / 1e9, 0),
+                     "shader_clock_mhz_mean": round(mhz.mean().item()), "shader_clock_mhz_min": round(mhz.min().item()),
+                     "shader_clock_mhz_max": round(mhz.max().item()), "block_shader_clocks_mean": round(p[:, 0].mean().item()),
+                     "mfma_clocks_ideal_per_cu": round(ideal), "mfma_busy_of_block_clocks": round(ideal / p[:, 0].mean().item(), 4),
+                     "peak_at_this_clock_tflops": round(256 * 8192 * mhz.mean().item() / 1e6, 0)}
+    print(json.dumps({"workload": "gemm_clock", "gemm": out}))
+
+
 METRIC = "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms"
 LAYER_WORKLOADS = ("layer_7b", "layer_13b", "linear", "olmo_block")
 
@@ -816,7 +862,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "adamw", "adamw_class", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad",
+                    choices=["all", "gemm_clock", "adamw", "adamw_class", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad",
                              "gemm_wgrad", "linear", "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr",
                              "division_transpose", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b"],
                     help="all (default): the headline AdamW step as `value` plus an `extra` record for every other leg of the metric")
@@ -851,6 +897,8 @@ def main():
     torch.cuda.set_device(dev)
     torch.set_num_threads(host_threads())  # the CPU baselines use every core this process may use
     cpu = not args.no_cpu_baseline
+    if args.workload == "gemm_clock":
+        return gemm_clock(dev, torch)
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)

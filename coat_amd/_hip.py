@@ -9,7 +9,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libcoat_hip.so")
+# COAT_HIP_LIB: another build of the same library (an experiment or probe build made with COAT_LIB_OUT=... python -m coat_amd.build)
+LIB_PATH = os.environ.get("COAT_HIP_LIB") or os.path.join(_HERE, "libcoat_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
 MAX_SLOTS, MAX_SLOT_STRIDE = 16, 32  # COAT_MAX_SLOTS, COAT_MAX_SLOT_STRIDE of include/coat_hip.h

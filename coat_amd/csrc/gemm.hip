@@ -45,6 +45,9 @@ struct GemmArgs {
     int sa_dt, sb_dt, bias_dt;
     int M, N, K;
     int tiles_m, tiles_n;
+#ifdef COAT_GEMM_PROBE
+    unsigned long long* probe;
+#endif
 };
 
 // A slab row is 128 bytes = eight 16-byte chunks (one full cache line per row and load instruction: fetching rows as
@@ -102,6 +105,10 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     const int band = min(max(ntiles - xcd * per_xcd, 0), per_xcd);
     const int my_ntiles = my < band ? (band - my + stride - 1) / stride : 0;
     if (my_ntiles == 0) return;
+#ifdef COAT_GEMM_PROBE
+    // experiment build only: shader-clock and constant-clock (100 MHz) counters around the whole block
+    const uint64_t probe_t0 = __builtin_amdgcn_s_memtime(), probe_r0 = __builtin_amdgcn_s_memrealtime();
+#endif
     constexpr int GROUP_M = 4;  // 4 x 8 tiles per XCD round; measured against 2, 8, 16: 0.3-0.7 % per GEMM, 0.6 % on the 7B layer
     auto tile_origin = [&](int it, int& m0, int& n0) {
         const int tile = xcd * per_xcd + my + it * stride;
@@ -385,11 +392,25 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     }  // tiles
     if (!role) __builtin_amdgcn_s_barrier();  // role 0 started a phase early: its last barrier pairs with role 1's
     COAT_WAIT_VMCNT(0);  // drain the trailing zero-fill slabs before the block may exit
+#ifdef COAT_GEMM_PROBE
+    if (tid == 0 && G.probe) {
+        G.probe[2 * blockIdx.x] = __builtin_amdgcn_s_memtime() - probe_t0;
+        G.probe[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - probe_r0;
+    }
+#endif
 }
 
 }  // namespace coat
 
 using namespace coat;
+
+#ifdef COAT_GEMM_PROBE
+// Probe build only (-DCOAT_GEMM_PROBE, never the shipped library): every block of k_fp8_gemm leaves its duration in shader
+// clocks (s_memtime) and in ticks of the constant 100 MHz counter (s_memrealtime) in a caller-provided buffer of
+// 2 x 256 uint64, which gives the shader clock the GEMM really runs at.  bench.py --workload gemm_clock reads it.
+static std::atomic<unsigned long long*> coat_gemm_probe_buffer{nullptr};
+extern "C" void coat_gemm_set_probe(unsigned long long* buf) { coat_gemm_probe_buffer.store(buf); }
+#endif
 
 extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
                              const void* scale_a, int sa_dtype, const void* scale_b, int sb_dtype, const void* bias,
@@ -411,6 +432,9 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     G.M = (int)M; G.N = (int)N; G.K = (int)K;
     G.tiles_m = (int)((M + BM - 1) / BM);
     G.tiles_n = (int)((N + BN - 1) / BN);
+#ifdef COAT_GEMM_PROBE
+    G.probe = coat_gemm_probe_buffer.load();
+#endif
     const int ntiles = G.tiles_m * G.tiles_n;
     // persistent grid: one block per CU (the block's LDS ring takes a whole CU's LDS); CU count cached per device
     static std::atomic<int> n_cu_dev[kCoatMaxDevices];

@@ -3,12 +3,13 @@
 // Reference: coat/activation/real_quantization/func_rmsnorm.py (_rms_norm_fwd_fused :54-111,
 // _rms_norm_bwd_dx_fused :121-196, _rms_norm_bwd_dwdb :200-220).
 //
-// One 256-thread block per row; a lane owns 16-element chunks `lane + 256*it` of the row (16 B of FP8 codes,
-// 2 x 16 B of bf16 per chunk), so a row of up to 16384 columns lives in registers for the two passes over it
-// (statistic, then normalise).  Row sums are reduced in a fixed order (in-lane, DPP butterfly per wave, then
-// the four wave partials in index order), so results are deterministic, unlike the reference's lock-ordered dw.
-// dw is a two-stage reduction: every block accumulates the rows it owns into fp32 registers and writes one
-// partial row; a second kernel sums the partials in block order.
+// Rows up to 8192 columns: one wave per row (k_rmsnorm_fwd / k_rmsnorm_bwd below).  Wider rows, up to 16384 columns: one
+// 256-thread block per row (k_rmsnorm_*_block); a lane owns 16-element chunks `lane + 256*it` of the row (16 B of FP8
+// codes, 2 x 16 B of bf16 per chunk), so the row lives in registers for the two passes over it (statistic, then
+// normalise).  Row sums are reduced in a fixed order (in-lane, DPP butterfly per wave, then the four wave partials in
+// index order) in both layouts, so results are deterministic and independent of the layout, unlike the reference's
+// lock-ordered dw.  dw is a two-stage reduction: every block accumulates the rows it owns into fp32 registers and writes
+// one partial row; a second kernel sums the partials in block order.
 #include <math.h>
 
 #include <atomic>
@@ -402,7 +403,12 @@ static int rms_check(int64_t M, int64_t N, int QB) {
 
 // Rows up to 8192 columns go to the wave-per-row kernels (CH = 4 or 8 chunks of 16 per lane), wider rows (up to 16384) to
 // the block-per-row kernels.  KW = fp8 kind * 3 + weight dtype.
-constexpr int kRmsFwdMaxBlocks = 1024;  // x 4 waves: about two rows per wave at 8192 rows, the second prefetched under the first
+#ifndef COAT_RMS_FWD_BLOCKS
+#define COAT_RMS_FWD_BLOCKS 768
+#endif
+// three resident blocks (12 waves) on each of 256 CUs: 13.2 us at [8192, 4096] against 15.2 / 15.0 / 15.8 us with 512 / 1024 /
+// 2048 blocks; a wave walks its rows with the next one prefetched under the current one
+constexpr int kRmsFwdMaxBlocks = COAT_RMS_FWD_BLOCKS;
 #define RMS_KW_CASES(X) X(0, 0) X(0, 1) X(0, 2) X(1, 0) X(1, 1) X(1, 2)
 #define RMS_CHECK_ENUMS()                                                                                   \
     if (fp8 != COAT_E4M3 && fp8 != COAT_E5M2) return COAT_EINVAL;                                           \
