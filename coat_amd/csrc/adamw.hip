@@ -79,6 +79,18 @@ __device__ __forceinline__ float reference_tree_min(const float (&a)[4][4]) {
     return min_skip_zero(t0, t1);
 }
 
+// Correctly rounded sqrtf for x = +0 or a normal x >= 2^-96 (also right for +inf and NaN): the hardware approximation is
+// within one ulp; the residuals of its two neighbours, each one exact FMA, tell which of the three is the rounded root.
+// (The same correction the compiler's sqrtf applies, without the rescaling that only denormal inputs need.)
+__device__ __forceinline__ float sqrt_cr_normal(float x) {
+    const float s = __builtin_amdgcn_sqrtf(x);
+    const float s_dn = u2f(f2u(s) - 1u), s_up = u2f(f2u(s) + 1u);
+    const float r_dn = fmaf(-s_dn, s, x), r_up = fmaf(-s_up, s, x);
+    float r = r_dn <= 0.0f ? s_dn : s;
+    r = r_up > 0.0f ? s_up : r;
+    return r;
+}
+
 template <int PDT> struct PVec { static constexpr int kBytes = (PDT == kF32) ? 16 : 8; };
 
 template <int PDT> __device__ __forceinline__ void load4(const void* base, int64_t e, int64_t numel, float* o) {
@@ -128,19 +140,18 @@ __device__ __forceinline__ void store_codes4(uint8_t* base, int64_t e, int64_t n
 
 // ------------------------------------------------------------------------------------------------
 // Plain (no expansion) step: every operation is the IEEE operation of the reference, bit-exact.
-template <int PDT>
-__global__ __launch_bounds__(256) void k_fp8_adamw_plain(void* __restrict__ params, const void* __restrict__ grads,
-                                                          uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
-                                                          uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
-                                                          AdamArgs A, int64_t numel, int64_t ngroups) {
-    enable_fp8_saturation();
-    const int lane = threadIdx.x & 63, lam = lane & 7;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+// FULL: all eight groups of the wave are complete (no element or group masking anywhere).
+template <int PDT, bool FULL>
+__device__ __forceinline__ void adamw_plain_wave(void* __restrict__ params, const void* __restrict__ grads,
+                                                 uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
+                                                 uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
+                                                 const AdamArgs& A, int64_t numel_in, int64_t ngroups, int64_t wave, int lane) {
+    const int lam = lane & 7;
     const int64_t gi = wave * 8 + (lane >> 3);
-    if (wave * 8 >= ngroups) return;  // whole wave out of range (wave-uniform)
-    const bool gvalid = gi < ngroups;
+    const bool gvalid = FULL || gi < ngroups;
     const int64_t gidx = gvalid ? gi : ngroups - 1;  // lanes of absent groups redo the last group, stores masked
     const int64_t e0 = gidx * kGroup + lam * 4;
+    const int64_t numel = FULL ? (int64_t)1 << 62 : numel_in;  // FULL: every bounds test folds away
     const int64_t lim = gvalid ? numel : 0;
 
     float p[4][4], g[4][4];
@@ -155,6 +166,7 @@ __global__ __launch_bounds__(256) void k_fp8_adamw_plain(void* __restrict__ para
     const float sm = scale_m[gidx], sv = scale_v[gidx];
     float m[4][4], v[4][4];
     float mx_m = 0.0f, mx_v = 0.0f;
+    uint32_t low_v = 0xFFFFFFFFu;  // smallest second moment other than +0, as bits - 1 (+0 wraps to the largest value)
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         float fm[4], fv[4];
@@ -162,19 +174,50 @@ __global__ __launch_bounds__(256) void k_fp8_adamw_plain(void* __restrict__ para
         fp8x4_to_f32<kE4M3>(cv[j], fv);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const bool ok = e0 + 32 * j + i < lim;
+            const bool ok = FULL || e0 + 32 * j + i < lim;
             float em = fm[i] * sm, ev = fv[i] * sv;
-            const float gr = g[j][i], pr = p[j][i];
+            const float gr = g[j][i];
             em = A.beta1 * em + A.one_minus_beta1 * gr;
             ev = A.beta2 * ev + (A.one_minus_beta2 * gr) * gr;
-            float denom = (sqrtf(ev) / A.correction2_sqrt + A.eps) * A.correction1;
-            float update = (em / denom) + (A.wd * pr);
-            p[j][i] = pr - (A.lr * update);
             m[j][i] = em;
             v[j][i] = ev;
+            low_v = min(low_v, f2u(ev) - 1u);
             mx_m = fmaxf(mx_m, ok ? fabsf(em) : 0.0f);
             mx_v = fmaxf(mx_v, ok ? fabsf(ev) : 0.0f);
         }
+    }
+    // sqrt(v) / c2: the correctly rounded square root from the hardware approximation and one correction step, and the
+    // quotient through the reciprocal of the (wave-uniform) divisor with one correction step, which is the IEEE quotient
+    // (div_by_scale; c2 = sqrt(1 - beta2^step) lies in (0, 1]).  Together they take a third of the instructions of the
+    // compiler's sqrtf and division.  Anything outside their domain (denormal, infinite or NaN second moments, a
+    // degenerate c2) takes the compiler's sequences, decided once per wave.
+    const float c2 = A.correction2_sqrt;
+    // every second moment is +0 or lies in [2^-96, inf): the domain of sqrt_cr_normal (negative values and NaNs have the
+    // sign bit or an all-ones exponent, which also puts them above the upper bound)
+    const bool plain_range = low_v >= f2u(0x1p-96f) - 1u && mx_v < INFINITY;
+    const bool fast = __all(plain_range) && c2 >= 0x1p-20f && c2 <= 1.0f;
+    if (fast) {
+        const float rc2 = 1.0f / c2;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float pr = p[j][i];
+                const float sq = sqrt_cr_normal(v[j][i]);
+                const float denom = (div_by_scale(sq, c2, rc2) + A.eps) * A.correction1;
+                const float update = (m[j][i] / denom) + (A.wd * pr);
+                p[j][i] = pr - (A.lr * update);
+            }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float pr = p[j][i];
+                const float denom = (sqrtf(v[j][i]) / c2 + A.eps) * A.correction1;
+                const float update = (m[j][i] / denom) + (A.wd * pr);
+                p[j][i] = pr - (A.lr * update);
+            }
     }
 #pragma unroll
     for (int j = 0; j < 4; j++) store4<PDT>(params, e0 + 32 * j, lim, p[j]);
@@ -210,6 +253,21 @@ __global__ __launch_bounds__(256) void k_fp8_adamw_plain(void* __restrict__ para
         scale_m[gi] = snew_m;
         scale_v[gi] = snew_v;
     }
+}
+
+template <int PDT>
+__global__ __launch_bounds__(256) void k_fp8_adamw_plain(void* __restrict__ params, const void* __restrict__ grads,
+                                                          uint8_t* __restrict__ exp_avg, float* __restrict__ scale_m,
+                                                          uint8_t* __restrict__ exp_avg_sq, float* __restrict__ scale_v,
+                                                          AdamArgs A, int64_t numel, int64_t ngroups) {
+    enable_fp8_saturation();
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (wave * 8 >= ngroups) return;  // whole wave out of range (wave-uniform)
+    if ((wave * 8 + 8) * kGroup <= numel)
+        adamw_plain_wave<PDT, true>(params, grads, exp_avg, scale_m, exp_avg_sq, scale_v, A, numel, ngroups, wave, lane);
+    else
+        adamw_plain_wave<PDT, false>(params, grads, exp_avg, scale_m, exp_avg_sq, scale_v, A, numel, ngroups, wave, lane);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -255,3 +255,33 @@ int64_t coat_oracle_count_recip_div_mismatch(const float *x, int64_t nx, const f
     }
     return bad;
 }
+
+/* Check of the device's square-root correction (sqrt_cr_normal in coat_amd/csrc/adamw.hip): starting from the correctly
+ * rounded root moved by -1, 0 and +1 ulp (the hardware approximation is within one ulp), the two-residual correction must
+ * return the correctly rounded root, for x = +0, x = +inf and normal x >= 2^-96 (smaller inputs are outside the domain
+ * of the device function and are skipped).  Returns the number of (x, start) pairs for which it does not. */
+int64_t coat_oracle_count_sqrt_correction_mismatch(const float *x, int64_t nx) {
+    int64_t bad = 0;
+    for (int64_t i = 0; i < nx; i++) {
+        const float xv = x[i], ref = sqrtf(xv);
+        if (!(xv == 0.0f || xv >= 0x1p-96f)) continue;
+        uint32_t rb;
+        memcpy(&rb, &ref, 4);
+        const int exact_only = xv == 0.0f || isinf(xv);  /* the hardware returns these two exactly */
+        for (int d = exact_only ? 0 : -1; d <= (exact_only ? 0 : 1); d++) {
+            uint32_t sb = rb + (uint32_t)d, dn = sb - 1u, up = sb + 1u;
+            float s, s_dn, s_up;
+            memcpy(&s, &sb, 4);
+            memcpy(&s_dn, &dn, 4);
+            memcpy(&s_up, &up, 4);
+            const float r_dn = fmaf(-s_dn, s, xv), r_up = fmaf(-s_up, s, xv);
+            float r = r_dn <= 0.0f ? s_dn : s;
+            r = r_up > 0.0f ? s_up : r;
+            uint32_t a;
+            memcpy(&a, &r, 4);
+            bad += a != rb;
+        }
+    }
+    return bad;
+}
+

@@ -45,6 +45,8 @@ def lib():
         L.coat_oracle_e4m3_decode.restype = f
         L.coat_oracle_count_recip_div_mismatch.argtypes = [vp, i64, vp, i64]
         L.coat_oracle_count_recip_div_mismatch.restype = i64
+        L.coat_oracle_count_sqrt_correction_mismatch.argtypes = [vp, i64]
+        L.coat_oracle_count_sqrt_correction_mismatch.restype = i64
         _lib = L
     return _lib
 

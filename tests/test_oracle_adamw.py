@@ -186,3 +186,26 @@ def test_bf16_params_round_once():
     _run_expand(pb, gr, st_b, 1, hp=hp)
     assert torch.equal(pb, pa.bfloat16())
     assert torch.equal(st_a["exp_avg"].view(torch.uint8), st_b["exp_avg"].view(torch.uint8))
+
+
+def test_device_division_and_sqrt_shortcuts_are_exact_on_the_cpu():
+    """The plain AdamW kernel replaces two of the compiler's IEEE sequences by shorter ones that must give the same bits:
+    sqrt(v) / c2 through the reciprocal of c2 and one FMA correction (the three-operation sequence of div_by_scale), and
+    sqrtf through the hardware approximation (within one ulp) and a two-residual correction.  Both are restated in
+    oracle/adamw_ref.c with IEEE arithmetic and compared with / and sqrtf: 0 mismatches over every c2 = sqrt(1 - beta2^step)
+    of 2000 steps x 2e5 square roots, and over 3e6 second moments x the three possible starting points."""
+    L = A.lib()
+    gen = torch.Generator().manual_seed(0)
+    # second moments as they occur (g^2 scale, spread over 40 binades) and their correctly rounded roots
+    v = (torch.rand(200_000, generator=gen) * 2 + 0.5) * torch.pow(2.0, torch.randint(-80, 20, (200_000,), generator=gen).float())
+    roots = v.sqrt().contiguous()
+    c2 = []
+    for beta2 in (0.95, 0.999):
+        for step in range(1, 1001):
+            c2.append(math.sqrt(1.0 - float(torch.tensor(beta2, dtype=torch.float32).double().pow(float(step)).float())))
+    c2 = torch.tensor(c2, dtype=torch.float32).contiguous()
+    assert (c2 > 0).all() and (c2 <= 1).all()
+    assert L.coat_oracle_count_recip_div_mismatch(roots.data_ptr(), roots.numel(), c2.data_ptr(), c2.numel()) == 0
+    x = torch.cat([v, torch.rand(800_000, generator=gen) * 1e-3, torch.rand(2_000_000, generator=gen).pow(8) * 1e-2,
+                   torch.tensor([0.0, 2.0 ** -96, 1.0, 4.0, 2.0 ** 60, float("inf")])]).float().contiguous()
+    assert L.coat_oracle_count_sqrt_correction_mismatch(x.data_ptr(), x.numel()) == 0
