@@ -11,7 +11,7 @@ def fp8_silu_forward(x, s_x, QB):
     x, s_x, batch = prep_pg(x, s_x)
     M, N = x.shape
     y = torch.empty_like(x)
-    s_y = torch.empty_like(s_x, dtype=torch.bfloat16)
+    s_y = torch.empty_like(s_x)  # in the dtype of the input scales, as the reference allocates it (:166-167)
     _hip.check(_hip.lib().coat_fp8_silu_forward(_hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(y),
                                                 _hip.ptr(s_y), M, N, QB, _hip.stream(x.device)), "fp8_silu_forward")
-    return restore(y, batch), restore(s_y.to(s_x.dtype), batch)
+    return restore(y, batch), restore(s_y, batch)

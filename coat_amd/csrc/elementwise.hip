@@ -33,6 +33,8 @@ struct EwArgs {
     int64_t nchunk;   // number of 16-element chunks
     int qb;           // group size (multiple of 16)
     int s_in_dtype;   // dtype of s1 / s2 (COAT_BF16 or COAT_F32 / COAT_F16)
+    int s_out_dtype;  // dtype of s_out: bf16 (0-initialised default below is overwritten) except for the SiLU forward,
+                      // whose scales take the dtype of the input scales (silu_fwd.py:166-167)
 };
 
 __device__ __forceinline__ float load_scale_rt(const void* p, int64_t i, int dt) {
@@ -153,7 +155,12 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
                                       div_by_scale(v[4 * k + 2], s, r), div_by_scale(v[4 * k + 3], s, r));
         if (ok) *(uint4*)((uint8_t*)A.q + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
     }
-    if (A.s_out && ok && (threadIdx.x % lpg) == 0) ((uint16_t*)A.s_out)[(c * 16) / A.qb] = (uint16_t)f2bf16(s);
+    if (A.s_out && ok && (threadIdx.x % lpg) == 0) {
+        const int64_t si = (c * 16) / A.qb;
+        if (A.s_out_dtype == kBF16) ((uint16_t*)A.s_out)[si] = (uint16_t)f2bf16(s);
+        else if (A.s_out_dtype == kF32) ((float*)A.s_out)[si] = s;
+        else ((uint16_t*)A.s_out)[si] = (uint16_t)f2f16(s);
+    }
     if (A.s_max) tensor_max = fmaxf(tensor_max, ok ? s : 0.0f);
     }
     if (A.s_max) block_atomic_max_nonneg(A.s_max, tensor_max, smem_max);
@@ -325,8 +332,9 @@ static int ew_common(EwArgs& A, int64_t M, int64_t N, int QB, int s_in_dtype) {
 
 extern "C" int coat_fp8_silu_forward(const void* x, int fp8, const void* s_x, int s_dtype, void* y, void* s_y,
                                      int64_t M, int64_t N, int QB, void* stream) {
-    EwArgs A = {x, s_x, nullptr, nullptr, nullptr, nullptr, nullptr, y, s_y, nullptr, 0, 0, 0};
+    EwArgs A = {x, s_x, nullptr, nullptr, nullptr, nullptr, nullptr, y, s_y, nullptr, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, s_dtype)) return e;
+    A.s_out_dtype = s_dtype;  // the output scales are stored in the dtype of the input scales
     if (M * N == 0) return COAT_OK;
     if (!x || !s_x || !y || !s_y) return COAT_EINVAL;
     return launch_ew<kSiluFwd>(A, fp8, fp8, (hipStream_t)stream);
@@ -334,7 +342,7 @@ extern "C" int coat_fp8_silu_forward(const void* x, int fp8, const void* s_x, in
 
 extern "C" int coat_fp8_silu_backward(const void* x, int fp8_in, const void* s_x, int s_dtype, const void* g, void* y,
                                       void* s_y, float* s_max, int fp8_out, int64_t M, int64_t N, int QB, void* stream) {
-    EwArgs A = {x, s_x, nullptr, nullptr, g, y, nullptr, nullptr, s_y, s_max, 0, 0, 0};
+    EwArgs A = {x, s_x, nullptr, nullptr, g, y, nullptr, nullptr, s_y, s_max, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, s_dtype)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x || !s_x || !g || !y) return COAT_EINVAL;
@@ -344,7 +352,7 @@ extern "C" int coat_fp8_silu_backward(const void* x, int fp8_in, const void* s_x
 extern "C" int coat_fp8_mul_forward(const void* x1, const void* s_x1, const void* x2, const void* s_x2, int fp8_in,
                                     int s_dtype, void* y, void* s_y, float* s_max, int64_t M, int64_t N, int QB,
                                     void* stream) {
-    EwArgs A = {x1, s_x1, x2, s_x2, nullptr, y, nullptr, nullptr, s_y, s_max, 0, 0, 0};
+    EwArgs A = {x1, s_x1, x2, s_x2, nullptr, y, nullptr, nullptr, s_y, s_max, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, s_dtype)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x1 || !s_x1 || !x2 || !s_x2 || !y) return COAT_EINVAL;
@@ -354,7 +362,7 @@ extern "C" int coat_fp8_mul_forward(const void* x1, const void* s_x1, const void
 extern "C" int coat_fp8_mul_backward(const void* x1, const void* s_x1, const void* x2, const void* s_x2, int fp8_in,
                                      int s_dtype, const void* g, void* y1, void* y2, void* s_y2, float* s_max,
                                      int fp8_out, int64_t M, int64_t N, int QB, void* stream) {
-    EwArgs A = {x1, s_x1, x2, s_x2, g, y2, y1, nullptr, s_y2, s_max, 0, 0, 0};
+    EwArgs A = {x1, s_x1, x2, s_x2, g, y2, y1, nullptr, s_y2, s_max, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, s_dtype)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x1 || !s_x1 || !x2 || !s_x2 || !g || !y1 || !y2) return COAT_EINVAL;
@@ -363,7 +371,7 @@ extern "C" int coat_fp8_mul_backward(const void* x1, const void* s_x1, const voi
 
 extern "C" int coat_fp8_gelu_forward(const void* x, int fp8, const void* s_x, int s_dtype, void* y, void* s_y,
                                      float* s_max, int64_t M, int64_t N, int QB, void* stream) {
-    EwArgs A = {x, s_x, nullptr, nullptr, nullptr, y, nullptr, nullptr, s_y, s_max, 0, 0, 0};
+    EwArgs A = {x, s_x, nullptr, nullptr, nullptr, y, nullptr, nullptr, s_y, s_max, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, s_dtype)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x || !s_x || !y) return COAT_EINVAL;
@@ -372,7 +380,7 @@ extern "C" int coat_fp8_gelu_forward(const void* x, int fp8, const void* s_x, in
 
 extern "C" int coat_fp8_gelu_backward(const void* x, int fp8_in, const void* s_x, int s_dtype, const void* g, void* y,
                                       void* s_y, float* s_max, int fp8_out, int64_t M, int64_t N, int QB, void* stream) {
-    EwArgs A = {x, s_x, nullptr, nullptr, g, y, nullptr, nullptr, s_y, s_max, 0, 0, 0};
+    EwArgs A = {x, s_x, nullptr, nullptr, g, y, nullptr, nullptr, s_y, s_max, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, s_dtype)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x || !s_x || !g || !y) return COAT_EINVAL;
@@ -381,7 +389,7 @@ extern "C" int coat_fp8_gelu_backward(const void* x, int fp8_in, const void* s_x
 
 extern "C" int coat_fp8_add_fwd(const void* x1, const void* x2, void* y, void* q, void* s_q, int fp8_out, int64_t M,
                                 int64_t N, int QB, void* stream) {
-    EwArgs A = {x1, nullptr, x2, nullptr, nullptr, y, nullptr, q, s_q, nullptr, 0, 0, 0};
+    EwArgs A = {x1, nullptr, x2, nullptr, nullptr, y, nullptr, q, s_q, nullptr, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, COAT_BF16)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x1 || !x2 || !y || !q || !s_q) return COAT_EINVAL;
@@ -390,7 +398,7 @@ extern "C" int coat_fp8_add_fwd(const void* x1, const void* x2, void* y, void* q
 
 extern "C" int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s_y, float* s_max, int fp8_out,
                                 int64_t M, int64_t N, int QB, void* stream) {
-    EwArgs A = {x1, nullptr, x2, nullptr, nullptr, y, nullptr, nullptr, s_y, s_max, 0, 0, 0};
+    EwArgs A = {x1, nullptr, x2, nullptr, nullptr, y, nullptr, nullptr, s_y, s_max, 0, 0, 0, kBF16};
     if (int e = ew_common(A, M, N, QB, COAT_BF16)) return e;
     if (M * N == 0) return COAT_OK;
     if (!x1 || !x2 || !y) return COAT_EINVAL;
@@ -444,7 +452,7 @@ extern "C" int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, c
                                          int64_t N, int QB, int64_t in_pitch, int64_t s_pitch, void* stream) {
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !q_silu || !s_silu || !s_max)) return COAT_EINVAL;  // y may be NULL
     SiluMulArgs A = {gate, s_gate, up, s_up, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr,
-                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
+                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0, kBF16};
     return silu_mul_launch(A, false, fp8, fp8, M, N, QB, s_dtype, in_pitch, s_pitch, 0, (hipStream_t)stream);
 }
 
@@ -456,7 +464,7 @@ extern "C" int coat_fp8_silu_mul_forward_bf16(const void* gate, const void* up, 
     if ((M > 0 && N > 0) && (!gate || !up || !q_gate || !s_gate || !q_up || !s_up || !q_silu || !s_silu || !s_max))
         return COAT_EINVAL;  // y may be NULL
     SiluMulArgs A = {gate, nullptr, up, nullptr, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr,
-                     q_gate, s_gate, q_up, s_up, 0, 0, 0};
+                     q_gate, s_gate, q_up, s_up, 0, 0, 0, kBF16};
     return silu_mul_launch(A, false, fp8, fp8, M, N, QB, COAT_BF16, 0, 0, 0, (hipStream_t)stream);
 }
 
@@ -468,6 +476,6 @@ extern "C" int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, 
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !silu || !s_silu || !g || !y_gate || !s_max_gate || !y_up || !s_max_up))
         return COAT_EINVAL;
     SiluMulArgs A = {gate, s_gate, up, s_up, silu, s_silu, g, nullptr, nullptr, y_gate, y_up, s_max_gate, s_max_up,
-                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
+                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0, kBF16};
     return silu_mul_launch(A, true, fp8_in, fp8_out, M, N, QB, s_dtype, in_pitch, s_pitch, y_pitch, (hipStream_t)stream);
 }

@@ -86,8 +86,9 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 // v_mfma_f32_32x32x64_f8f6f4, two waves per SIMD.
 // Persistent: the grid is one block per CU; a block walks its share of the output tiles and the LDS ring runs straight
 // across tile boundaries, so the first slabs of the next tile are already in flight while the epilogue stores drain.
-template <int FMT_A, int FMT_B, int EPI, bool VEC16>
+template <int FMT_A, int FMT_B, int EPI, bool VEC16, int QBE>
 __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
+    static_assert(QBE == 16 || (EPI != kEpiBf16 && (QBE == 32 || QBE == 64)), "group size of the quantizing epilogue");
     constexpr int NWN = 4, NW = 2 * NWN;      // waves along N, waves per block
     constexpr int TJ = BN / (NWN * 32);       // n-tiles per wave (2); m-tiles per wave is 4
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -273,6 +274,60 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     const uint32_t s_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * (G.N >> 4) + wn * (TJ * 2)) * 2;
     const int q_n_lim = G.N - n0 - wn * (TJ * 32);          // a 16-column group at offset c exists iff c < q_n_lim
     const bool pack_scales = (G.N & 63) == 0 && q_n_lim >= TJ * 32 && ((uintptr_t)G.Cs & 7) == 0;  // wave-uniform
+    if constexpr (EPI != kEpiBf16 && QBE > 16) {
+        // Groups of 32 or 64 columns (reference linear.py:139-164 is generic in the group size): a row's 32 columns of
+        // one accumulator tile sit in lanes l and l ^ 32, its 64 columns of the wave in the two tiles of those lanes, so
+        // the group maximum is an in-lane maximum plus one lane swap.  Both tiles of a row are scaled before the first
+        // code is formed (32 live values instead of 16; this path is off the shipped configurations, which use 16).
+        constexpr int KIND = EPI == kEpiQuantE4M3 ? kE4M3 : kE5M2;
+        const int sn = G.N / QBE;  // scales per row
+        uint8_t* const sw_tile = (uint8_t*)G.Cs + ((int64_t)m0 * sn + (n0 + wn * (TJ * 32)) / QBE) * 2;
+        const uint32_t sw_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * sn) * 2;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float v[TJ][16], am[TJ];
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                const int nb = n0 + wn * (TJ * 32) + j * 32 + 4 * half;
+                float a = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float t = acc[j][i][r] * scale;
+                    if (G.bias) {
+                        const int n = nb + 8 * (r >> 2) + (r & 3);
+                        if (n < G.N) t += load_rt_f32(G.bias, n, G.bias_dt);
+                    }
+                    v[j][r] = t;
+                    a = fmaxf(a, fabsf(t));
+                }
+                const auto sw2 = __builtin_amdgcn_permlane32_swap(f2u(a), f2u(a), false, false);
+                am[j] = fmaxf(u2f(sw2[0]), u2f(sw2[1]));
+            }
+            if (QBE == 64) am[0] = am[1] = fmaxf(am[0], am[1]);
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                const float s = group_scale<KIND>(am[j]);
+                const float r = 1.0f / s;
+                const bool inside = i * 32 < m_lim && j * 32 < q_n_lim;  // N % QBE == 0: a group is inside or outside as a whole
+#pragma unroll
+                for (int g2 = 0; g2 < 2; g2++) {
+                    const uint32_t w0 = cvt4_fp8<KIND>(div_by_scale(v[j][8 * g2], s, r), div_by_scale(v[j][8 * g2 + 1], s, r),
+                                                       div_by_scale(v[j][8 * g2 + 2], s, r), div_by_scale(v[j][8 * g2 + 3], s, r));
+                    const uint32_t w1 = cvt4_fp8<KIND>(div_by_scale(v[j][8 * g2 + 4], s, r), div_by_scale(v[j][8 * g2 + 5], s, r),
+                                                       div_by_scale(v[j][8 * g2 + 6], s, r), div_by_scale(v[j][8 * g2 + 7], s, r));
+                    const auto sw = __builtin_amdgcn_permlane32_swap(w0, w1, false, false);
+                    if (inside) {
+                        uint8_t* base = q_tile + ((int64_t)(i * 32) * G.N + j * 32 + 16 * g2);
+                        *(uint2*)(base + q_lane_off) = make_uint2(sw[0], sw[1]);
+                    }
+                }
+                if (inside && half == 0 && (QBE == 32 || j == 0)) {
+                    uint8_t* sbase = sw_tile + ((int64_t)(i * 32) * sn + (QBE == 32 ? j : 0)) * 2;
+                    *(uint16_t*)(sbase + sw_lane_off) = (uint16_t)f2bf16(s);
+                }
+            }
+        }
+    } else {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int m = m0 + wm * 128 + i * 32 + (lane & 31);
@@ -362,6 +417,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
             *(uint2*)(sbase + s_lane_off) = make_uint2(spack[0], spack[1]);
         }
     }
+    }  // group size 16 / bf16 output
     }  // epilogue of tile it - 1
     if (it == my_ntiles) break;
 #pragma unroll
@@ -424,7 +480,7 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     if (!coat_aligned16(a) || !coat_aligned16(b) || !coat_aligned16(c)) return COAT_EALIGN;
     if ((fmt_a != COAT_E4M3 && fmt_a != COAT_E5M2) || (fmt_b != COAT_E4M3 && fmt_b != COAT_E5M2)) return COAT_EINVAL;
     if (out_kind < 0 || out_kind > 2) return COAT_EINVAL;
-    if (out_kind != 0 && (QB != 16 || N % 16 != 0 || !c_scale)) return COAT_ESHAPE;
+    if (out_kind != 0 && ((QB != 16 && QB != 32 && QB != 64) || N % QB != 0 || !c_scale)) return COAT_ESHAPE;
     if (sa_dtype < 0 || sa_dtype > 2 || sb_dtype < 0 || sb_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return COAT_EDTYPE;
     GemmArgs G;
     G.A = (const uint8_t*)a; G.B = (const uint8_t*)b; G.C = c; G.Cs = c_scale;
@@ -450,18 +506,24 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     const int grid = min(((ntiles + 7) / 8) * 8, n_cu);
     const size_t lds_bytes = kLdsBytes;
     hipStream_t st = (hipStream_t)stream;
-#define GEMM_LAUNCH_V(FA, FB, EP, V16)                                                                                  \
+#define GEMM_LAUNCH_V(FA, FB, EP, V16, QE)                                                                         \
     {                                                                                                              \
-        static coat_device_flags lds_ok;                                                                         \
-        if (int e = coat_allow_lds(k_fp8_gemm<FA, FB, EP, V16>, (int)lds_bytes, lds_ok)) return e;                 \
-        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, V16>), dim3(grid), dim3(512), lds_bytes, st, G); \
+        static coat_device_flags lds_ok;                                                                           \
+        if (int e = coat_allow_lds(k_fp8_gemm<FA, FB, EP, V16, QE>, (int)lds_bytes, lds_ok)) return e;             \
+        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, V16, QE>), dim3(grid), dim3(512), lds_bytes, st, G);            \
         return coat_launch_status();                                                                               \
     }
-// the 16-byte-store epilogue only exists for the bf16 output
-#define GEMM_LAUNCH(FA, FB, EP)                                                  \
-    {                                                                            \
-        if (EP == kEpiBf16 && (N & 7) == 0) GEMM_LAUNCH_V(FA, FB, EP, true)      \
-        GEMM_LAUNCH_V(FA, FB, EP, false)                                         \
+// the 16-byte-store epilogue only exists for the bf16 output, group sizes other than 16 only for the quantized ones
+#define GEMM_LAUNCH(FA, FB, EP)                                                       \
+    {                                                                                 \
+        if constexpr (EP == kEpiBf16) {                                               \
+            if ((N & 7) == 0) GEMM_LAUNCH_V(FA, FB, EP, true, 16)                     \
+            GEMM_LAUNCH_V(FA, FB, EP, false, 16)                                      \
+        } else {                                                                      \
+            if (QB == 32) GEMM_LAUNCH_V(FA, FB, EP, false, 32)                        \
+            if (QB == 64) GEMM_LAUNCH_V(FA, FB, EP, false, 64)                        \
+            GEMM_LAUNCH_V(FA, FB, EP, false, 16)                                      \
+        }                                                                             \
     }
 #define GEMM_FMT(EP)                                                             \
     if (fmt_a == COAT_E4M3 && fmt_b == COAT_E4M3) GEMM_LAUNCH(0, 0, EP)          \

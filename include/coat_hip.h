@@ -109,7 +109,8 @@ int coat_fp8_dequantize(const void* q, int fp8, const void* s, int s_dtype, void
  * (amax_g + 1e-10) / fp8max(fp8_out) of the fp32 value; s_max (optional) is a zero-initialised buffer of COAT_MAX_WORDS
  * fp32 that receives their maximum (the per-tensor scale of the division that follows in the reference). */
 
-/* rq/silu_fwd.py:152 fp8_silu_forward (kernel :47-149): y = per-group fp8(silu(x)), same fp8 type as x. */
+/* rq/silu_fwd.py:152 fp8_silu_forward (kernel :47-149): y = per-group fp8(silu(x)), same fp8 type as x; s_y in s_dtype,
+ * the dtype of the input scales (:166-167), unlike the bf16 s_y of the other kernels of this block. */
 int coat_fp8_silu_forward(const void* x, int fp8, const void* s_x, int s_dtype, void* y, void* s_y, int64_t M,
                           int64_t N, int QB, void* stream);
 /* rq/silu_bwd.py:170 fp8_silu_backward (kernel :47-167): y = bf16((sig + x*sig*(1-sig)) * g). */
@@ -247,7 +248,7 @@ int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* si
  * (+ bias[N]), fp32 accumulation on FP8 MFMA.  A and B are row-major with K contiguous (the reference passes B as
  * the .t() view of such a matrix, linear.py:253-302); fmt_a / fmt_b are coat_fp8 values and may differ.
  * out_kind 0: C is bf16 [M,N] (:166-169).  out_kind 1 / 2: C is e4m3 / e5m2 [M,N], quantized per 1 x QB group along
- * N with scale (amax + 1e-10) / fp8max, and c_scale is bf16 [M, N/QB] (:139-164); QB must be 16.
+ * N with scale (amax + 1e-10) / fp8max, and c_scale is bf16 [M, N/QB] (:139-164); QB 16, 32 or 64, N % QB == 0.
  * scale_a / scale_b: one element each in device memory, of sa_dtype / sb_dtype (each is loaded in its own dtype and the
  * two are multiplied in fp32, :123-125: an fp32 weight scale next to a bf16 activation scale keeps all its bits).
  * K % 16 == 0. */

@@ -101,6 +101,13 @@ def test_silu_forward_backward(dev, fp8):
     assert y.dtype == q.dtype
     codes_close(y, wy)
     bf16_close(sy, wsy)
+    # fp32 input scales: the output scales are stored as fp32 too (reference silu_fwd.py:166-167), not rounded through bf16
+    q32, s32 = R.fp8_quantize(x, QB, fp8, scale_dtype=torch.float32)
+    y32, sy32 = rq.fp8_silu_forward(q32.to(dev), s32.to(dev), QB)
+    wy32, wsy32 = R.fp8_silu_forward(q32, s32, QB)
+    assert sy32.dtype == torch.float32 and wsy32.dtype == torch.float32
+    assert torch.allclose(sy32.cpu(), wsy32, rtol=1e-6, atol=0) and (sy32.cpu() != sy32.cpu().bfloat16().float()).any()
+    codes_close(y32, wy32)
     gy, gs = rq.fp8_silu_backward(q.to(dev), s.to(dev), g.to(dev), QB, "E5M2")
     wgy, wgs = R.fp8_silu_backward(q, s, g, QB, "E5M2")
     bf16_close(gy, wgy)

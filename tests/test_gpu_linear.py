@@ -85,30 +85,39 @@ def test_fp8matmul_bias_batched_and_rowmajor_b(dev):
     assert torch.equal(c2, c)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 512, 256), (384, 272, 128)])
-def test_fp8matmul_quantized_output(dev, M, N, K):
+@pytest.mark.parametrize("M,N,K,QB", [(256, 512, 256, 16), (384, 272, 128, 16), (256, 512, 256, 32), (300, 448, 144, 64),
+                                      (384, 288, 128, 32), (4352, 4160, 80, 64)])
+def test_fp8matmul_quantized_output(dev, M, N, K, QB):
+    """Quantizing epilogue, groups of 16 (every shipped configuration), 32 and 64 columns (the reference's epilogue is
+    generic in the group size, linear.py:139-164); ragged last tile row / column, bias in the last case."""
     lin = _lin()
     a, b = rand_fp8((M, K), 6, E4), rand_fp8((N, K), 7, E4)
     sa, sb = torch.tensor(0.02).bfloat16(), torch.tensor(0.02).bfloat16()
-    cq, cs = lin.fp8matmul(a.to(dev), b.to(dev).t(), True, sa.to(dev), sb.to(dev), 16)
-    wq, ws = R.fp8matmul(a, b.t(), True, sa, sb, 16, accumulate=torch.float64)
-    assert cq.dtype == E4 and cs.shape == (M, N // 16) and cs.dtype == torch.bfloat16
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(8)).bfloat16() if M > 4000 else None
+    cq, cs = lin.fp8matmul(a.to(dev), b.to(dev).t(), True, sa.to(dev), sb.to(dev), QB, None if bias is None else bias.to(dev))
+    wq, ws = R.fp8matmul(a, b.t(), True, sa, sb, QB, bias, accumulate=torch.float64)
+    assert cq.dtype == E4 and cs.shape == (M, N // QB) and cs.dtype == torch.bfloat16
     g, w = cq.cpu().view(torch.uint8).int(), wq.view(torch.uint8).int()
     neq = g != w
     print(f"[measured] quantizing epilogue {M}x{N}x{K}: {neq.float().mean().item():.3e} of the codes differ (bar 4e-3)")
     assert neq.float().mean().item() < 4e-3
     # where the codes differ, the dequantized values differ by one code step of that magnitude or by the accumulation bound
-    dg = R.fp8_dequantize(cq.cpu(), cs.cpu(), 16).double()
-    dw = R.fp8_dequantize(wq, ws, 16).double()
+    dg = R.fp8_dequantize(cq.cpu(), cs.cpu(), QB).double()
+    dw = R.fp8_dequantize(wq, ws, QB).double()
     mag = (a.double().abs() @ b.double().abs().t()) * (sa.double() * sb.double())
-    assert ((dg - dw).abs() <= dw.abs() * 2.0 ** -3 + mag * 2.0 ** -13 + 1e-12).all()
+    if bias is not None:
+        mag = mag + bias.double().abs()
+    step0 = ws.double().repeat_interleave(QB, dim=1) * 2.0 ** -9  # one step of the subnormal codes of the group
+    assert ((dg - dw).abs() <= dw.abs() * 2.0 ** -3 + step0 + mag * 2.0 ** -13 + 1e-12).all()
     sg, sw = cs.cpu().view(torch.int16).int(), ws.view(torch.int16).int()
     print(f"[measured] quantizing epilogue {M}x{N}x{K}: {(sg != sw).float().mean().item():.3e} of the scales differ (bar 5e-3)")
     assert ((sg - sw).abs() <= 1).all() and (sg != sw).float().mean().item() < 5e-3
     # the dequantized product is the product
-    deq = R.fp8_dequantize(cq.cpu(), cs.cpu(), 16).double()
+    deq = R.fp8_dequantize(cq.cpu(), cs.cpu(), QB).double()
     ref = (a.double() @ b.double().t()) * (sa.double() * sb.double())
-    gmax = ref.reshape(M, N // 16, 16).abs().amax(dim=2).repeat_interleave(16, dim=1)
+    if bias is not None:
+        ref = ref + bias.double()
+    gmax = ref.reshape(M, N // QB, QB).abs().amax(dim=2).repeat_interleave(QB, dim=1)
     assert ((deq - ref).abs() <= gmax * 2.0 ** -4 * 1.05 + 1e-9).all()
 
 
