@@ -78,6 +78,17 @@ __device__ __forceinline__ float load_rt_f32(const void* p, int64_t i, int dt) {
     if (dt == kF32) return ((const float*)p)[i];
     return f16lo(((const uint16_t*)p)[i]);
 }
+// The same in two steps, for code that wants several loads in flight before the first conversion (a conversion right
+// after its load makes the wave wait for that load before it can issue the next one).
+__device__ __forceinline__ uint32_t load_rt_raw(const void* p, int64_t i, int dt) {
+    if (dt == kF32) return ((const uint32_t*)p)[i];
+    return ((const uint16_t*)p)[i];
+}
+__device__ __forceinline__ float rt_raw_to_f32(uint32_t raw, int dt) {
+    if (dt == kBF16) return u2f(raw << 16);
+    if (dt == kF32) return u2f(raw);
+    return f16lo(raw);
+}
 // Round an fp32 value to dtype DT and back (what storing and re-loading would give).
 template <int DT> __device__ __forceinline__ float round_to(float v) {
     if (DT == kF32) return v;

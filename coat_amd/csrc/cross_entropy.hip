@@ -29,6 +29,20 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 template <int XDT> struct ElemSize { static constexpr int kBytes = XDT == kF32 ? 4 : 2; };
 
+// The VEC values of a whole chunk from its 16 bytes.
+template <int XDT, int VEC> __device__ __forceinline__ void unpack_chunk(const uint4& t, float* v) {
+    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+    if (XDT == kF32) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i % VEC] = u2f(w[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[(2 * i) % VEC] = XDT == kBF16 ? bf16lo(w[i]) : f16lo(w[i]);
+            v[(2 * i + 1) % VEC] = XDT == kBF16 ? bf16hi(w[i]) : f16hi(w[i]);
+        }
+    }
+}
 // Chunk j of a row = elements [j * VEC, j * VEC + VEC); elements at or beyond V read as `fill`.
 template <int XDT, int VEC> __device__ __forceinline__ void load_chunk(const void* row, int64_t j, int64_t V, float fill, float* v) {
     const int64_t e0 = j * VEC;
@@ -123,11 +137,24 @@ __global__ __launch_bounds__(kCeThreads) void k_cross_entropy(CeArgs a) {
     float v[ITERS > 0 ? ITERS : 1][VEC];
     float m = ninf, d = 0.0f, sx = 0.0f;
     if (ITERS > 0) {
+        // All 16-byte loads of the row first, unconditionally (a chunk that is not a whole chunk of the row re-reads the
+        // row's last whole chunk and is replaced below): under a condition, or with a conversion between them, the
+        // compiler makes the wave wait for each load before it issues the next.
+        uint4 raw[ITERS > 0 ? ITERS : 1];
+        const int64_t nfull = V / VEC;  // whole chunks
+        if (VEC > 1 && nfull > 0) {
+#pragma unroll
+            for (int it = 0; it < ITERS; it++) {
+                const int64_t j = min((int64_t)it * kCeThreads + tid, nfull - 1);
+                raw[it] = ld_stream16((const uint8_t*)xrow + j * 16);
+            }
+        }
 #pragma unroll
         for (int it = 0; it < ITERS; it++) {
             const int64_t j = (int64_t)it * kCeThreads + tid;
             if (j < nchunk) {
-                load_chunk<XDT, VEC>(xrow, j, V, ninf, v[it]);
+                if (VEC > 1 && j < nfull) unpack_chunk<XDT, VEC>(raw[it], v[it]);
+                else load_chunk<XDT, VEC>(xrow, j, V, ninf, v[it]);
 #pragma unroll
                 for (int k = 0; k < VEC; k++) {
                     const bool valid = j * VEC + k < V;

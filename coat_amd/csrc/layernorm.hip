@@ -235,19 +235,19 @@ extern "C" int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s
     LN_DISPATCH(k_layernorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, mean, rstd, dx, dw_partial, db_partial, M, (int)N, QB)
     if (int e = coat_launch_status()) return e;
     if (w_dtype < 0) return COAT_OK;
-    const int cols_blocks = (int)((N + 15) / 16);
+    const int cols_blocks = (int)((N + kColsumCols - 1) / kColsumCols);
     switch (w_dtype) {
         case COAT_F32:
-            hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N);
-            hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(256), 0, st, db_partial, db, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, dw_partial, dw, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, db_partial, db, (int)grid, (int)N);
             break;
         case COAT_BF16:
-            hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N);
-            hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(256), 0, st, db_partial, db, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, dw_partial, dw, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, db_partial, db, (int)grid, (int)N);
             break;
         default:
-            hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N);
-            hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(256), 0, st, db_partial, db, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, dw_partial, dw, (int)grid, (int)N);
+            hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, db_partial, db, (int)grid, (int)N);
             break;
     }
     return coat_launch_status();

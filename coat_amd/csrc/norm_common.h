@@ -77,23 +77,34 @@ __device__ __forceinline__ void store_bf16_16(void* p, int64_t off, const float*
     dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
 }
 
-// dw[col] = sum over blocks (in block order) of the partials, stored in the weight's dtype.
+// dw[col] = sum of the partial rows in a fixed order (deterministic), stored in the weight's dtype.
+// 32 columns per block: one 128-byte line of every partial row, so no line is fetched by two blocks (blocks sit on
+// different XCDs with an L2 each; 16-column blocks fetched every line twice).  The rows are split over 16 thread slices,
+// slice s taking rows 8 s .. 8 s + 7 of every 128, with 32 loads in flight per thread.
+constexpr int kColsumCols = 32, kColsumThreads = 512;
 template <int WDT>
-__global__ __launch_bounds__(256) void k_norm_colsum(const float* __restrict__ partial, void* __restrict__ dw, int nblocks,
-                                                     int N) {
-    // 16 columns per block (256 blocks for N = 4096, one per CU), the partial rows split over 16 thread slices in a fixed
-    // order (deterministic), 8 loads in flight per thread
-    __shared__ float red[16][16];
-    const int c = threadIdx.x & 15, slice = threadIdx.x >> 4;
-    const int col = blockIdx.x * 16 + c;
+__global__ __launch_bounds__(kColsumThreads) void k_norm_colsum(const float* __restrict__ partial, void* __restrict__ dw,
+                                                                 int nblocks, int N) {
+    __shared__ float red[16][kColsumCols];
+    const int c = threadIdx.x & (kColsumCols - 1), slice = threadIdx.x / kColsumCols;
+    const int col = blockIdx.x * kColsumCols + c;
     float acc[8];
 #pragma unroll
     for (int u = 0; u < 8; u++) acc[u] = 0.0f;
     if (col < N) {
-        for (int b0 = slice * 8; b0 < nblocks; b0 += 128) {
+        // four rounds of rows at a time: all 32 loads are issued before the first addition (rows past the end are read
+        // from the last row and add 0), the additions keep their order
+        for (int b0 = slice * 8; b0 < nblocks; b0 += 512) {
+            float v[4][8];
 #pragma unroll
-            for (int u = 0; u < 8; u++)
-                if (b0 + u < nblocks) acc[u] += partial[(int64_t)(b0 + u) * N + col];
+            for (int k = 0; k < 4; k++)
+#pragma unroll
+                for (int u = 0; u < 8; u++)
+                    v[k][u] = partial[(int64_t)min(b0 + 128 * k + u, nblocks - 1) * N + col];
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+#pragma unroll
+                for (int u = 0; u < 8; u++) acc[u] += (b0 + 128 * k + u < nblocks) ? v[k][u] : 0.0f;
         }
     }
     red[slice][c] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
@@ -105,6 +116,5 @@ __global__ __launch_bounds__(256) void k_norm_colsum(const float* __restrict__ p
         store_from_f32<WDT>(dw, col, s);
     }
 }
-
 
 }  // namespace coat

@@ -471,11 +471,11 @@ static int rms_backward_launch(const void* x, int fp8, const void* s_x, int s_dt
     }
 #undef RMS_BWD
     if (int e = coat_launch_status()) return e;
-    const int cols_blocks = (int)((N + 15) / 16);
+    const int cols_blocks = (int)((N + kColsumCols - 1) / kColsumCols);
     switch (w_dtype) {
-        case COAT_F32: hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
-        case COAT_BF16: hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
-        default: hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(256), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        case COAT_F32: hipLaunchKernelGGL((k_norm_colsum<kF32>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        case COAT_BF16: hipLaunchKernelGGL((k_norm_colsum<kBF16>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, dw_partial, dw, (int)grid, (int)N); break;
+        default: hipLaunchKernelGGL((k_norm_colsum<kF16>), dim3(cols_blocks), dim3(kColsumThreads), 0, st, dw_partial, dw, (int)grid, (int)N); break;
     }
     return coat_launch_status();
 }
