@@ -20,7 +20,9 @@
  *
  * Pins: tests/test_oracle_adamw.py (closed-form AdamW from tests/test_fp8_adamw_expand.py:111-131
  * and nvcc_qoptim.cu:39-58; the reference test's search definition of the exponent k, :146-148;
- * DRE invariants; k=1,c=1 reduces to the plain kernel; fresh state step 1 == torch.optim.AdamW).
+ * DRE invariants; k=1,c=1 reduces to the plain kernel; fresh state step 1 == torch.optim.AdamW; the plain
+ * step's parameters, codes and scales bit-identical over six steps to the same kernel written with whole-tensor
+ * torch operations and torch's own float -> e4m3 cast).
  *
  * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off -shared -fPIC).
  */

@@ -209,3 +209,53 @@ def test_device_division_and_sqrt_shortcuts_are_exact_on_the_cpu():
     x = torch.cat([v, torch.rand(800_000, generator=gen) * 1e-3, torch.rand(2_000_000, generator=gen).pow(8) * 1e-2,
                    torch.tensor([0.0, 2.0 ** -96, 1.0, 4.0, 2.0 ** 60, float("inf")])]).float().contiguous()
     assert L.coat_oracle_count_sqrt_correction_mismatch(x.data_ptr(), x.numel()) == 0
+
+
+def test_plain_step_trajectory_against_torch_tensor_restatement():
+    """The plain step of the C oracle against the reference kernel written a second time with whole-tensor torch operations
+    (fp8_adamw_cuda_kernel.cu:37-53, 107-124: dequantize, moments, bias corrections, parameter update, group maximum + 1e-20
+    in double, scale = max / 448, codes = e4m3(moment / scale) by torch's own cast).  Six steps from the fresh state on a
+    tensor with a ragged last group: parameters, both code tensors and both scale vectors must be bit-identical at every
+    step.  (torch's CPU kernels round every + - * / sqrt separately, like the oracle; a dropped term, a wrong bias
+    correction or a scale taken from the wrong group shows in the first step.)"""
+    n, G = 128 * 5 + 77, 128
+    ng = (n + G - 1) // G
+    gen = torch.Generator().manual_seed(11)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    b1, b2, lr, wd, eps = 0.9, 0.95, 3e-4, 0.1, 1e-8
+    f32 = lambda x: torch.tensor(x, dtype=torch.float32)
+    # oracle state
+    p = p0.clone()
+    st = A.fresh_state(p, False)
+    # restatement state (padded to whole groups; the padding holds zeros and never reaches a stored value)
+    pr = p0.clone()
+    m8 = torch.zeros(ng * G, dtype=torch.float8_e4m3fn)
+    v8 = torch.zeros(ng * G, dtype=torch.float8_e4m3fn)
+    sm, sv = st["scale_exp_avg"].clone(), st["scale_exp_avg_sq"].clone()
+    for step in range(1, 7):
+        gr = torch.randn(n, generator=gen) * (1e-3 * step)
+        A.adamw_step(p, gr, st["exp_avg"], st["scale_exp_avg"], st["exp_avg_sq"], st["scale_exp_avg_sq"], b1, b2, lr, wd, eps, step, G)
+        g = torch.zeros(ng * G)
+        g[:n] = gr
+        m = m8.float() * sm.repeat_interleave(G)
+        v = v8.float() * sv.repeat_interleave(G)
+        m = f32(b1) * m + (f32(1.0) - f32(b1)) * g
+        v = f32(b2) * v + ((f32(1.0) - f32(b2)) * g) * g
+        c1 = f32(1.0) - torch.pow(f32(b1), f32(float(step)))
+        c2 = torch.sqrt(f32(1.0) - torch.pow(f32(b2), f32(float(step))))
+        denom = (torch.sqrt(v[:n]) / c2 + f32(eps)) * c1
+        update = m[:n] / denom + f32(wd) * pr
+        pr = pr - f32(lr) * update
+        m[n:] = 0.0
+        v[n:] = 0.0
+        amax_m = m.abs().reshape(ng, G).amax(dim=1)
+        amax_v = v.abs().reshape(ng, G).amax(dim=1)
+        sm = ((amax_m.double() + 1e-20).float()) / f32(448.0)
+        sv = ((amax_v.double() + 1e-20).float()) / f32(448.0)
+        m8 = (m / sm.repeat_interleave(G)).to(torch.float8_e4m3fn)
+        v8 = (v / sv.repeat_interleave(G)).to(torch.float8_e4m3fn)
+        assert torch.equal(p.view(torch.int32), pr.view(torch.int32)), step
+        assert torch.equal(st["scale_exp_avg"].view(torch.int32), sm.view(torch.int32)), step
+        assert torch.equal(st["scale_exp_avg_sq"].view(torch.int32), sv.view(torch.int32)), step
+        assert torch.equal(st["exp_avg"].view(torch.uint8).flatten()[:n], m8.view(torch.uint8)[:n]), step
+        assert torch.equal(st["exp_avg_sq"].view(torch.uint8).flatten()[:n], v8.view(torch.uint8)[:n]), step
