@@ -269,13 +269,15 @@ __global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__
 
 // Backward, one wave per row.  A block's four waves keep fp32 weight-gradient sums for the rows they walked; at the end
 // they are added in wave order through LDS, 1024 columns at a time, into the block's partial row.
-template <int KIND, int WDT, int CH>
+// MULTI: up to two further gradients of the same tensor are added to dy (dy2, dy3).  A variant of its own, because the
+// extra loads in flight cost it the second resident block per CU, which the single-gradient kernel keeps.
+template <int KIND, int WDT, int CH, bool MULTI>
 __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
                                                       const void* __restrict__ dy, const void* __restrict__ dy2,
                                                       const void* __restrict__ dy3, const void* __restrict__ w,
                                                       const float* __restrict__ rstd_in, void* __restrict__ dx,
                                                       float* __restrict__ dw_partial, int64_t M, int N, int qb) {
-    constexpr bool HOLD_W = WDT != kF32;
+    constexpr bool HOLD_W = WDT != kF32 && !MULTI;  // MULTI spends those registers on gradient loads in flight
     __shared__ float red[4][64 * 16];
     const int lane = threadIdx.x & 63, wv_id = threadIdx.x >> 6;
     const int64_t nwaves = (int64_t)gridDim.x * 4;
@@ -311,28 +313,70 @@ __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__
             }
         }
         const float rstd = rstd_in[row];
-        if (dy2) {
+        if constexpr (MULTI) {
             // further gradients of the same tensor, summed the way a chain of bf16 tensor additions would:
-            // (dy + dy2) rounded to bf16, then + dy3 rounded to bf16 (wave-uniform branches)
+            // (dy + dy2) rounded to bf16, then + dy3 rounded to bf16.  Their loads are unconditional (a chunk past the
+            // row's end re-reads its last 16 columns and is dropped; without a third gradient the second is read again,
+            // from the cache) and issued ahead of the additions: loaded and converted chunk by chunk, every one of the
+            // up to 2 x CH loads was a round trip of its own.
+            const void* const d3 = dy3 ? dy3 : dy2;
+            auto add_to = [&](int c, const uint4* r2, const uint4* r3) {  // adds both (as loaded) to chunk c of g
+                float a[16], b[16];
+                unpack_w16<kBF16>(g[c], a);
+                unpack_w16<kBF16>(r2, b);
 #pragma unroll
-            for (int c = 0; c < CH; c++) {
-                const int col = (c * 64 + lane) * 16;
-                if (col < N) {
-                    float a[16], b[16];
-                    load_bf16_16(dy2, row_off + col, b);
-                    unpack_w16<kBF16>(g[c], a);
+                for (int i = 0; i < 16; i++) a[i] = round_to<kBF16>(a[i] + b[i]);
+                if (dy3) {  // wave-uniform
+                    unpack_w16<kBF16>(r3, b);
 #pragma unroll
                     for (int i = 0; i < 16; i++) a[i] = round_to<kBF16>(a[i] + b[i]);
-                    if (dy3) {
-                        load_bf16_16(dy3, row_off + col, b);
+                }
+                uint32_t pk[8];
 #pragma unroll
-                        for (int i = 0; i < 16; i++) a[i] = round_to<kBF16>(a[i] + b[i]);
+                for (int k = 0; k < 8; k++) pk[k] = pack_bf16x2(a[2 * k], a[2 * k + 1]);
+                g[c][0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                g[c][1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+            };
+            if constexpr (CH <= 4) {  // a whole row of one gradient at a time: two round trips instead of 2 x CH
+                uint4 r[CH][2];
+                auto load_all = [&](const void* src) {
+#pragma unroll
+                    for (int c = 0; c < CH; c++) {
+                        const int col = min((c * 64 + lane) * 16, N - 16);
+                        const uint4* p = (const uint4*)((const uint16_t*)src + row_off + col);
+                        r[c][0] = p[0]; r[c][1] = p[1];
                     }
-                    uint32_t pk[8];
+                };
+                auto add_all = [&]() {
 #pragma unroll
-                    for (int k = 0; k < 8; k++) pk[k] = pack_bf16x2(a[2 * k], a[2 * k + 1]);
-                    g[c][0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-                    g[c][1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+                    for (int c = 0; c < CH; c++) {
+                        if ((c * 64 + lane) * 16 < N) {
+                            float a[16], b[16];
+                            unpack_w16<kBF16>(g[c], a);
+                            unpack_w16<kBF16>(r[c], b);
+                            uint32_t pk[8];
+#pragma unroll
+                            for (int k = 0; k < 8; k++)
+                                pk[k] = pack_bf16x2(round_to<kBF16>(a[2 * k] + b[2 * k]), round_to<kBF16>(a[2 * k + 1] + b[2 * k + 1]));
+                            g[c][0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                            g[c][1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+                        }
+                    }
+                };
+                load_all(dy2);
+                add_all();
+                if (dy3) {  // wave-uniform
+                    load_all(dy3);
+                    add_all();
+                }
+            } else {  // eight chunks: one chunk's four loads at a time
+#pragma unroll
+                for (int c = 0; c < CH; c++) {
+                    const int col = (c * 64 + lane) * 16, lcol = min(col, N - 16);
+                    const uint4* p2 = (const uint4*)((const uint16_t*)dy2 + row_off + lcol);
+                    const uint4* p3 = (const uint4*)((const uint16_t*)d3 + row_off + lcol);
+                    const uint4 r2[2] = {p2[0], p2[1]}, r3[2] = {p3[0], p3[1]};
+                    if (col < N) add_to(c, r2, r3);
                 }
             }
         }
@@ -453,23 +497,28 @@ static int rms_backward_launch(const void* x, int fp8, const void* s_x, int s_dt
     const int64_t rows_per_block = N <= 8192 ? 4 : 1;
     const int64_t want = (M + rows_per_block - 1) / rows_per_block;
     const int64_t grid = n_partial < want ? n_partial : want;
+#define RMS_BWD_WAVE(K, W, CHV, MU)                                                                                    \
+    hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, CHV, MU>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, s_dtype, \
+                       dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB)
 #define RMS_BWD(K, W)                                                                                                  \
     case K * 3 + W:                                                                                                    \
-        if (N <= 4096)                                                                                                 \
-            hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, 4>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, s_dtype, \
-                               dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB);                                  \
-        else if (N <= 8192)                                                                                            \
-            hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, 8>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, s_dtype, \
-                               dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB);                                  \
-        else                                                                                                           \
+        if (N <= 4096) {                                                                                               \
+            if (dy2) RMS_BWD_WAVE(K, W, 4, true);                                                                      \
+            else RMS_BWD_WAVE(K, W, 4, false);                                                                         \
+        } else if (N <= 8192) {                                                                                        \
+            if (dy2) RMS_BWD_WAVE(K, W, 8, true);                                                                      \
+            else RMS_BWD_WAVE(K, W, 8, false);                                                                         \
+        } else {                                                                                                       \
             hipLaunchKernelGGL((k_rmsnorm_bwd_block<K, W, 4>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, \
                                s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB);                         \
+        }                                                                                                              \
         break;
     switch (fp8 * 3 + w_dtype) {
         RMS_KW_CASES(RMS_BWD)
         default: return COAT_EINVAL;
     }
 #undef RMS_BWD
+#undef RMS_BWD_WAVE
     if (int e = coat_launch_status()) return e;
     const int cols_blocks = (int)((N + kColsumCols - 1) / kColsumCols);
     switch (w_dtype) {
