@@ -523,6 +523,8 @@ MEASURED_TRAFFIC = {
     "gemm_fwd": (743.1e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
     "gemm_dgrad": (608.4e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
     "cross_entropy": (2099.7e6, "profiles/k_cross_entropy__llama2_vocab32000_8192tok_fp32.txt"),
+    "silu_mul": (2616.7e6, "profiles/k_silu_mul__silu_mul_8192x11008.txt (the five launches of forward + backward together; two passes over the tensors)"),
+    "rmsnorm": (332.4e6, "profiles/k_rmsnorm__rmsnorm_8192x4096.txt (the four kernels of forward + backward together)"),
 }
 
 
