@@ -26,6 +26,33 @@ def test_library_exports_every_declared_symbol():
     assert b"128 per-group" in L.coat_status_string(-4)
 
 
+def test_python_signatures_match_the_header():
+    """Every ctypes signature has as many arguments as the header's declaration, with pointers, 64-bit integers, ints
+    and floats in the same places (a mismatch would shift every later argument of a call)."""
+    from coat_amd import _hip
+
+    header = open(os.path.join(ROOT, "include", "coat_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", " ", header, flags=re.S)
+    kinds = {ctypes.c_void_p: "p", ctypes.c_int: "i", ctypes.c_int64: "l", ctypes.c_float: "f", ctypes.c_uint64: "l"}
+    for name, argtypes in _hip.SIGNATURES.items():
+        m = re.search(r"\bint\s+" + name + r"\s*\(([^)]*)\)\s*;", header)
+        assert m, f"{name} not declared as an int function"
+        want = ""
+        for par in m.group(1).split(","):
+            par = " ".join(par.split())
+            if "*" in par:
+                want += "p"
+            elif par.startswith(("int64_t", "uint64_t")):
+                want += "l"
+            elif par.startswith("float"):
+                want += "f"
+            else:
+                assert par.startswith("int "), (name, par)
+                want += "i"
+        have = "".join(kinds[t] for t in argtypes)
+        assert have == want, f"{name}: ctypes {have} vs header {want}"
+
+
 def test_argument_validation_without_gpu():
     """Rejected arguments return before any launch, so these run without a GPU."""
     from coat_amd import _hip
