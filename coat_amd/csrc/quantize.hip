@@ -641,8 +641,10 @@ __global__ __launch_bounds__(256) void k_quantize_transpose(const void* __restri
 // 128-byte lines / 16-byte scale pieces.  Phase 2 reads one dword = two neighbouring columns of one row, so a lane owns
 // a column pair over a 16-row chunk (two 16-byte stores into neighbouring q^T rows); chunks vary fastest over the
 // lanes, so 8 neighbouring lanes complete one 128-byte q^T line.
-template <int XDT, int SDT, int KIND, int QB>
-__global__ __launch_bounds__(256) void k_quantize_transpose16(const void* __restrict__ x, void* __restrict__ q,
+// NT threads per tile: 256 when the grid is about one round of resident blocks (17.6 against 19.5 us at [4096, 4096]),
+// 512 = twice the waves per CU for larger tensors (78.9 against 82.4 us at [8192, 11008]).
+template <int XDT, int SDT, int KIND, int QB, int NT>
+__global__ __launch_bounds__(NT) void k_quantize_transpose16(const void* __restrict__ x, void* __restrict__ q,
                                                                void* __restrict__ s_out, void* __restrict__ qt,
                                                                void* __restrict__ st_out, int64_t M, int64_t N) {
     static_assert(XDT != kF32, "16-bit inputs only");
@@ -659,18 +661,18 @@ __global__ __launch_bounds__(256) void k_quantize_transpose16(const void* __rest
     const int64_t m0 = tm * T, n0 = tn * T;
 
     // phase 1: 16 jobs of 8 elements per row, 8 jobs per thread; all loads first
-    constexpr int JPR = T / 8, NIT = T * JPR / 256;
+    constexpr int JPR = T / 8, NIT = T * JPR / NT;
     uint4 raw[NIT];
 #pragma unroll
     for (int it = 0; it < NIT; it++) {
-        const int job = threadIdx.x + it * 256;
+        const int job = threadIdx.x + it * NT;
         const int64_t m = m0 + job / JPR, n = n0 + (job % JPR) * 8;
         // (conditional on purpose: all eight loads issued back to back were measured 11 % slower, 19.7 against 17.7 us)
         raw[it] = (m < M && n < N) ? *(const uint4*)((const uint16_t*)x + m * N + n) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int it = 0; it < NIT; it++) {
-        const int job = threadIdx.x + it * 256;
+        const int job = threadIdx.x + it * NT;
         const int row = job / JPR, cv = job % JPR;
         const int64_t m = m0 + row, n = n0 + cv * 8;
         const bool ok = m < M && n < N;  // N % QB == 0: a group is inside or outside as a whole
@@ -693,7 +695,7 @@ __global__ __launch_bounds__(256) void k_quantize_transpose16(const void* __rest
     // phase 2: job = (column pair cp, 16-row chunk mc), mc fastest; groups of QB rows are QB/16 neighbouring lanes
     constexpr int MC = T / 16, LPG_T = QB / 16, JOBS2 = MC * (T / 2);
 #pragma unroll
-    for (int j0 = 0; j0 < JOBS2; j0 += 256) {
+    for (int j0 = 0; j0 < JOBS2; j0 += NT) {
         const int job = j0 + threadIdx.x;
         const int mc = job % MC, cp = job / MC;
         const int64_t m = m0 + mc * 16, n = n0 + 2 * cp;
@@ -1027,8 +1029,12 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
         if (blocks16 >= ((int64_t)1 << 31)) return COAT_ESHAPE;
 #define LAUNCH_QT16(XD, QBV)                                                                                          \
     DISPATCH_SDT(s_dtype, DISPATCH_KIND(fp8, {                                                                        \
-        hipLaunchKernelGGL((k_quantize_transpose16<XD, SDT, KIND, QBV>), dim3((unsigned)blocks16), dim3(256), 0, st, x, q, \
-                           s, qt, st_out, M, N);                                                                      \
+        if (blocks16 > 2048)                                                                                          \
+            hipLaunchKernelGGL((k_quantize_transpose16<XD, SDT, KIND, QBV, 512>), dim3((unsigned)blocks16), dim3(512), 0, st,  \
+                               x, q, s, qt, st_out, M, N);                                                            \
+        else                                                                                                          \
+            hipLaunchKernelGGL((k_quantize_transpose16<XD, SDT, KIND, QBV, 256>), dim3((unsigned)blocks16), dim3(256), 0, st,  \
+                               x, q, s, qt, st_out, M, N);                                                            \
         return coat_launch_status();                                                                                  \
     }))
 #define LAUNCH_QT16_QB(XD)                                  \
