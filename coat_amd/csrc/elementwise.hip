@@ -37,14 +37,10 @@ struct EwArgs {
                       // whose scales take the dtype of the input scales (silu_fwd.py:166-167)
 };
 
-__device__ __forceinline__ float load_scale_rt(const void* p, int64_t i, int dt) {
-    if (dt == kBF16) return u2f((uint32_t)((const uint16_t*)p)[i] << 16);
-    if (dt == kF32) return ((const float*)p)[i];
-    return f16lo(((const uint16_t*)p)[i]);
-}
-
-template <int KIND> __device__ __forceinline__ void load_fp8x16(const void* p, int64_t chunk, float scale, float* v) {
-    uint4 c = *(const uint4*)((const uint8_t*)p + chunk * 16);
+// Dequantizes 16 loaded codes.  The 16 bytes of codes and the raw scale word are loaded first (load_rt_raw) and
+// converted here, after every load of the iteration has been issued; a scale converted right where it is loaded costs
+// a run-time dtype branch and a wait for that one load before the next is issued.
+template <int KIND> __device__ __forceinline__ void dequant_chunk(uint4 c, float scale, float* v) {
     uint32_t w[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll
     for (int k = 0; k < 4; k++) {
@@ -54,6 +50,7 @@ template <int KIND> __device__ __forceinline__ void load_fp8x16(const void* p, i
         for (int i = 0; i < 4; i++) v[4 * k + i] = f[i] * scale;  // dequantize: float(q) * float(s)
     }
 }
+__device__ __forceinline__ uint4 load_codes16(const void* p, int64_t chunk) { return *(const uint4*)((const uint8_t*)p + chunk * 16); }
 __device__ __forceinline__ void load_bf16x16(const void* p, int64_t chunk, float* v) {
     const uint4* src = (const uint4*)((const uint16_t*)p + chunk * 16);
     uint4 a = src[0], b = src[1];
@@ -94,6 +91,7 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
     __shared__ float smem_max[4];
     enable_fp8_saturation();
     const int lpg = A.qb >> 4;  // lanes per group
+    const int gshift = 27 - __builtin_clz(A.qb);  // chunk index -> group index (qb is a power of two >= 16)
     float tensor_max = 0.0f;
     // grid-stride over 256-chunk slabs: the trip count is block-uniform, so the lanes of a group stay together
     for (int64_t base = (int64_t)blockIdx.x * 256; base < A.nchunk; base += (int64_t)gridDim.x * 256) {
@@ -106,11 +104,15 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
         load_bf16x16(A.x1, c, a);
         load_bf16x16(A.x2, c, b);
     } else {
-        const int64_t gidx = (c * 16) / A.qb;
-        load_fp8x16<KIND_IN>(A.x1, c, load_scale_rt(A.s1, gidx, A.s_in_dtype), a);
-        if (kTwoIn) load_fp8x16<KIND_IN>(A.x2, c, load_scale_rt(A.s2, gidx, A.s_in_dtype), b);
+        const int64_t gidx = c >> gshift;
+        const uint32_t rs1 = load_rt_raw(A.s1, gidx, A.s_in_dtype);
+        const uint32_t rs2 = kTwoIn ? load_rt_raw(A.s2, gidx, A.s_in_dtype) : 0u;
+        const uint4 c1 = load_codes16(A.x1, c);
+        const uint4 c2 = kTwoIn ? load_codes16(A.x2, c) : make_uint4(0, 0, 0, 0);
+        if (kHasG) load_bf16x16(A.g, c, g);
+        dequant_chunk<KIND_IN>(c1, rt_raw_to_f32(rs1, A.s_in_dtype), a);
+        if (kTwoIn) dequant_chunk<KIND_IN>(c2, rt_raw_to_f32(rs2, A.s_in_dtype), b);
     }
-    if (kHasG) load_bf16x16(A.g, c, g);
 
 #pragma unroll
     for (int i = 0; i < 16; i++) {
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(256) void k_elementwise(EwArgs A) {
         if (ok) *(uint4*)((uint8_t*)A.q + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
     }
     if (A.s_out && ok && (threadIdx.x % lpg) == 0) {
-        const int64_t si = (c * 16) / A.qb;
+        const int64_t si = c >> gshift;
         if (A.s_out_dtype == kBF16) ((uint16_t*)A.s_out)[si] = (uint16_t)f2bf16(s);
         else if (A.s_out_dtype == kF32) ((float*)A.s_out)[si] = s;
         else ((uint16_t*)A.s_out)[si] = (uint16_t)f2f16(s);
@@ -211,20 +213,21 @@ __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
     __shared__ float smem_max[4];
     enable_fp8_saturation();
     const int lpg = A.qb >> 4;
+    const int gshift = 27 - __builtin_clz(A.qb);  // chunk index -> group index (qb is a power of two >= 16)
     float tmax = 0.0f, tmax2 = 0.0f;
     for (int64_t base = (int64_t)blockIdx.x * 256; base < A.nchunk; base += (int64_t)gridDim.x * 256) {
         const int64_t chunk = base + threadIdx.x;
         const bool ok = chunk < A.nchunk;
         const int64_t c = ok ? chunk : 0;
-        const int64_t gidx = (c * 16) / A.qb;
+        const int64_t gidx = c >> gshift;
         int64_t cin = c, gin = gidx, cy = c;
         if (A.strided) {  // uniform
             const int64_t row = c / A.cpr, col = c - row * A.cpr;
             cin = row * A.in_cpr + col;
-            gin = row * A.in_spr + (col * 16) / A.qb;
+            gin = row * A.in_spr + (col >> gshift);
             cy = row * A.y_cpr + col;
         }
-        float a[16], b[16];
+        float a[16], b[16], sl[16], g[16];
         if (FROM16) {
             float raw[2][16];
             load_bf16x16(A.gate, c, raw[0]);
@@ -245,8 +248,17 @@ __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
                 dequant_words<KIND_IN>(w, round_bf16(s), t ? b : a);  // as the saved activation is read back
             }
         } else {
-            load_fp8x16<KIND_IN>(A.gate, cin, load_scale_rt(A.s_gate, gin, A.s_dtype), a);
-            load_fp8x16<KIND_IN>(A.up, cin, load_scale_rt(A.s_up, gin, A.s_dtype), b);
+            // every load of the iteration is issued before the first conversion
+            const uint32_t rs_a = load_rt_raw(A.s_gate, gin, A.s_dtype), rs_b = load_rt_raw(A.s_up, gin, A.s_dtype);
+            const uint32_t rs_l = BWD ? load_rt_raw(A.s_silu, gidx, A.s_dtype) : 0u;
+            const uint4 ca = load_codes16(A.gate, cin), cb = load_codes16(A.up, cin);
+            if (BWD) {
+                const uint4 cl = load_codes16(A.silu, c);
+                load_bf16x16(A.g, c, g);
+                dequant_chunk<KIND_IN>(cl, rt_raw_to_f32(rs_l, A.s_dtype), sl);
+            }
+            dequant_chunk<KIND_IN>(ca, rt_raw_to_f32(rs_a, A.s_dtype), a);
+            dequant_chunk<KIND_IN>(cb, rt_raw_to_f32(rs_b, A.s_dtype), b);
         }
         if (!BWD) {
             float sv[16];
@@ -272,9 +284,7 @@ __global__ __launch_bounds__(256) void k_silu_mul(SiluMulArgs A) {
             const float s2 = group_scale<KIND_IN>(cluster_max_rt(amax16(v), lpg));
             tmax = fmaxf(tmax, ok ? s2 : 0.0f);
         } else {
-            float sl[16], g[16], v[16], v2[16];
-            load_fp8x16<KIND_IN>(A.silu, c, load_scale_rt(A.s_silu, gidx, A.s_dtype), sl);
-            load_bf16x16(A.g, c, g);
+            float v[16], v2[16];
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 v2[i] = g[i] * sl[i];                       // gradient of up
