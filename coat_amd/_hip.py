@@ -60,6 +60,7 @@ SIGNATURES = {
                                    _i64, _i64, _vp],
     "coat_rope_bf16": [_vp, _vp, _vp, _vp, _i64, _f, _vp, _i64, _i, _i, _i, _i, _i64, _i64, _vp],
     "coat_fp8_gemm": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _i, _vp],
+    "coat_fp8_gemm_grouped": [_i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _i, _vp],
     "coat_fp8_adamw_expand_step": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _i,
                                    _i64, _i64, _vp],
     "coat_fp8_adamw_step": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _i64, _i64, _vp],
@@ -117,6 +118,11 @@ def stream(device=None):
 
 def ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def ptr_array(tensors):
+    """Host array of device pointers (NULL for None), for entry points that take ``const void* const*``."""
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
 
 
 def dense(t):

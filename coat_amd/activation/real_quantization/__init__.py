@@ -20,5 +20,6 @@ from .mul_bwd import fp8_mul_backward
 from .mul_fwd import fp8_mul_forward
 from .silu_bwd import fp8_silu_backward
 from .silu_fwd import fp8_silu_forward
-from .linear import fp8_linear_backward, fp8_linear_forward
+from .linear import (fp8_linear_backward, fp8_linear_backward_grouped, fp8_linear_forward, fp8_linear_forward_grouped,
+                     fp8matmul_grouped)
 from .func_quantize import Coat_quantize_bgn, Coat_quantize_end

@@ -61,6 +61,71 @@ def fp8matmul(a, b, output_quantize, scale_a, scale_b, QB, bias=None, stochastic
     return (c, scale_c) if output_quantize else c
 
 
+_MAX_GROUP = 4  # problems per grouped launch (kMaxGroup of the kernel)
+
+
+def fp8matmul_grouped(a_list, b_list, output_quantize, scale_a_list, scale_b_list, QB):
+    """``[fp8matmul(a, b, output_quantize, sa, sb, QB) for ...]`` in one launch when every problem has the same shape
+    and formats (2-D ``a``, no bias): the q / k / v or gate / up projections of a layer and their backward products.
+    The results are bit-identical to the separate calls; on the persistent grid the problems' tiles form one sequence,
+    so a partial last round of tiles is paid once per group.  Anything else falls back to the separate calls."""
+    n = len(a_list)
+    assert n == len(b_list) == len(scale_a_list) == len(scale_b_list)
+    same = (1 < n <= _MAX_GROUP and all(a.dim() == 2 and a.is_contiguous() for a in a_list)
+            and len({(tuple(a.shape), a.dtype, tuple(b.shape), b.dtype, b.t().is_contiguous())
+                     for a, b in zip(a_list, b_list)}) == 1 and b_list[0].t().is_contiguous()
+            and len({s.dtype for s in scale_a_list}) == 1 and len({s.dtype for s in scale_b_list}) == 1
+            and all(s.numel() == 1 and s.is_cuda for s in (*scale_a_list, *scale_b_list)))
+    if not same:
+        return [fp8matmul(a, b, output_quantize, sa, sb, QB)
+                for a, b, sa, sb in zip(a_list, b_list, scale_a_list, scale_b_list)]
+    a_list = [_hip.dense(a) for a in a_list]
+    bn_list = [_hip.dense(b.t()) for b in b_list]
+    M, K = a_list[0].shape
+    N = bn_list[0].shape[0]
+    assert K == bn_list[0].shape[1], "Incompatible dimensions"
+    dev = a_list[0].device
+    if output_quantize:
+        c_list = [torch.empty((M, N), device=dev, dtype=a_list[0].dtype) for _ in range(n)]
+        cs_list = [torch.empty((M, N // QB), device=dev, dtype=torch.bfloat16) for _ in range(n)]
+        kind = _OUT_KIND[a_list[0].dtype]
+    else:
+        c_list = [torch.empty((M, N), device=dev, dtype=torch.bfloat16) for _ in range(n)]
+        cs_list, kind = None, 0
+    _hip.check(_hip.lib().coat_fp8_gemm_grouped(
+        n, _hip.ptr_array(a_list), _hip.fp8(a_list[0].dtype), _hip.ptr_array(bn_list), _hip.fp8(bn_list[0].dtype),
+        _hip.ptr_array(c_list), _hip.ptr_array(cs_list) if cs_list else None, kind,
+        _hip.ptr_array(scale_a_list), _hip.dt(scale_a_list[0]), _hip.ptr_array(scale_b_list), _hip.dt(scale_b_list[0]),
+        None, 0, M, N, K, QB if output_quantize else 0, _hip.stream(dev)), "fp8matmul_grouped")
+    return list(zip(c_list, cs_list)) if output_quantize else c_list
+
+
+def fp8_linear_forward_grouped(x, s, w_list, s_w_list, output_quantize, QB):
+    """``[fp8_linear_forward(x, s, w, s_w, output_quantize, QB) for ...]`` for projections of one input."""
+    assert s.numel() == 1, f"X uses per-tensor quantization in linear forward, but the scale shape is {s.shape}"
+    n = len(w_list)
+    x2 = x.reshape(-1, x.shape[-1]) if x.dim() == 3 else x
+    outs = fp8matmul_grouped([x2] * n, [w.t() for w in w_list], output_quantize, [s] * n, s_w_list, QB)
+    if x.dim() != 3:
+        return outs
+    lead = x.shape[:2]
+    if output_quantize:
+        return [(c.reshape(*lead, -1), cs.reshape(*lead, -1)) for c, cs in outs]
+    return [c.reshape(*lead, -1) for c in outs]
+
+
+def fp8_linear_backward_grouped(x_t, s, g_list, s_g_list, g_t_list, w_t_list, s_w_list, QB):
+    """``[fp8_linear_backward(x_t, s, g, s_g, g_t, w_t, s_w, QB) for ...]`` for projections of one input: the dgrads in
+    one launch and the wgrads in another.  Returns (list of dx, list of dW)."""
+    n = len(g_list)
+    assert s.numel() == 1 and all(t.numel() == 1 for t in (*s_g_list, *s_w_list)), "per-tensor scales in linear backward"
+    g2 = [g.reshape(-1, g.shape[-1]) if g.dim() == 3 else g for g in g_list]
+    dx = fp8matmul_grouped(g2, [w_t.t() for w_t in w_t_list], False, s_g_list, s_w_list, QB)
+    dx = [d.reshape(*g.shape[:2], -1) if g.dim() == 3 else d for d, g in zip(dx, g_list)]
+    dw = fp8matmul_grouped(g_t_list, [x_t.t()] * n, False, s_g_list, [s] * n, QB)
+    return dx, dw
+
+
 def fp8_linear_forward(x, s, w, s_w, output_quantize, QB, bias=None):
     """y = x @ w^T with w [N, K] (reference :253-258)."""
     assert s.numel() == 1, f"X uses per-tensor quantization in linear forward, but the scale shape is {s.shape}"

@@ -34,7 +34,11 @@ static_assert(BM == BN, "A and B slabs share one unit size");
 
 enum Epilogue { kEpiBf16 = 0, kEpiQuantE4M3 = 1, kEpiQuantE5M2 = 2 };
 
-struct GemmArgs {
+// One launch multiplies up to kMaxGroup independent problems of one shape (the q / k / v or gate / up projections of a
+// layer): their tiles form one sequence for the persistent grid, so a partial last round of tiles is paid once per
+// group instead of once per problem, and the LDS ring runs on from one problem into the next.
+constexpr int kMaxGroup = 4;
+struct GemmProblem {
     const uint8_t* A;   // [M, K]
     const uint8_t* B;   // [N, K]
     void* C;            // bf16 [M, N] or fp8 [M, N]
@@ -42,9 +46,16 @@ struct GemmArgs {
     const void* sa;     // per-tensor scales, one element each
     const void* sb;
     const void* bias;   // [N] or nullptr
+};
+// The shape and the first problem come first: a wave reads its kernel arguments from host-visible memory when it starts,
+// and the plain GEMM then touches two 64-byte lines of them as it would without the group (with the seven pointers laid
+// out as arrays of four the same kernel ran 1.3 % slower on config 3).
+struct GemmArgs {
     int sa_dt, sb_dt, bias_dt;
     int M, N, K;
     int tiles_m, tiles_n;
+    int nprob;                     // problems in this launch (1 .. kMaxGroup)
+    GemmProblem P[kMaxGroup];
 #ifdef COAT_GEMM_PROBE
     unsigned long long* probe;
 #endif
@@ -58,6 +69,7 @@ struct GemmArgs {
 __device__ __forceinline__ int swz_chunk(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) void* global_ptr_t;
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 // buffer_load_dwordx4 ... lds: every lane fetches 16 bytes at byte offset `voff` of the buffer and the wave's 1 KiB
@@ -77,6 +89,33 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
     return (v4i){(int)(uint32_t)a, (int)(uint32_t)(a >> 32) & 0xFFFF, (int)bytes, 0x00020000};
 }
 
+// v_writelane with a constant lane: lane LANE of `t` becomes the wave-uniform value v.
+template <int LANE> __device__ __forceinline__ void write_lane(uint32_t& t, uint32_t v) {
+    asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(t) : "s"(v), "n"(LANE));
+}
+template <int LANE> __device__ __forceinline__ void write_lane_ptr(uint32_t& t, const void* p) {
+    write_lane<LANE>(t, (uint32_t)(uintptr_t)p);
+    write_lane<LANE + 1>(t, (uint32_t)((uintptr_t)p >> 32));
+}
+// Problems P .. kMaxGroup - 1 into the table: lanes 14 P .. 14 P + 13 = the seven pointers, lane 14 kMaxGroup + P = the
+// product of the two scales.
+template <int P> __device__ __forceinline__ void fill_table(uint32_t& t, const GemmArgs& G) {
+    if constexpr (P < kMaxGroup) {
+        if (P < G.nprob) {  // (the arguments of unused problems are not even fetched: they are lines of host-visible memory)
+            write_lane_ptr<14 * P + 0>(t, G.P[P].A);
+            write_lane_ptr<14 * P + 2>(t, G.P[P].B);
+            write_lane_ptr<14 * P + 4>(t, G.P[P].C);
+            write_lane_ptr<14 * P + 6>(t, G.P[P].Cs);
+            write_lane_ptr<14 * P + 8>(t, G.P[P].sa);
+            write_lane_ptr<14 * P + 10>(t, G.P[P].sb);
+            write_lane_ptr<14 * P + 12>(t, G.P[P].bias);
+            const float sc = load_rt_f32(G.P[P].sa, 0, G.sa_dt) * load_rt_f32(G.P[P].sb, 0, G.sb_dt);
+            write_lane<14 * kMaxGroup + P>(t, __builtin_amdgcn_readfirstlane(f2u(sc)));
+            fill_table<P + 1>(t, G);
+        }
+    }
+}
+
 // s_waitcnt vmcnt(N) only (expcnt / lgkmcnt left at their maxima), gfx9 encoding.
 #define COAT_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (0x7 << 4) | (0xF << 8) | ((((N) >> 4) & 0x3) << 14))
 // lgkmcnt(0) only: all LDS reads issued so far have returned
@@ -86,7 +125,7 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, uint32_t bytes) {
 // v_mfma_f32_32x32x64_f8f6f4, two waves per SIMD.
 // Persistent: the grid is one block per CU; a block walks its share of the output tiles and the LDS ring runs straight
 // across tile boundaries, so the first slabs of the next tile are already in flight while the epilogue stores drain.
-template <int FMT_A, int FMT_B, int EPI, bool VEC16, int QBE>
+template <int FMT_A, int FMT_B, int EPI, bool VEC16, int QBE, bool GROUPED>
 __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     static_assert(QBE == 16 || (EPI != kEpiBf16 && (QBE == 32 || QBE == 64)), "group size of the quantizing epilogue");
     constexpr int NWN = 4, NW = 2 * NWN;      // waves along N, waves per block
@@ -100,7 +139,8 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     // XCD x owns the contiguous band [x * per_xcd, (x + 1) * per_xcd) of the tile order below, and its blocks take the
     // band's tiles in rounds of gridDim.x / 8: at any time one XCD works on neighbouring tiles, whose A / B slabs are
     // shared through that XCD's L2.  The tile order runs down panels of GROUP_M tile-rows.
-    const int ntiles = G.tiles_m * G.tiles_n;
+    const int ntiles1 = G.tiles_m * G.tiles_n;  // tiles of one problem; the problems' tiles follow one another
+    const int ntiles = GROUPED ? G.nprob * ntiles1 : ntiles1;
     const int per_xcd = (ntiles + 7) / 8;
     const int xcd = blockIdx.x & 7, my = blockIdx.x >> 3, stride = gridDim.x >> 3;
     const int band = min(max(ntiles - xcd * per_xcd, 0), per_xcd);
@@ -110,9 +150,31 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     // experiment build only: shader-clock and constant-clock (100 MHz) counters around the whole block
     const uint64_t probe_t0 = __builtin_amdgcn_s_memtime(), probe_r0 = __builtin_amdgcn_s_memrealtime();
 #endif
+    // Grouped launch: the problems' pointers and scales are kept across the lanes of one VGPR (lane 14 p + 2 f and the
+    // next: pointer f of problem p as two dwords; lane 56 + p: its combined scale) and fetched with v_readlane when a
+    // tile begins: scalar registers for four problems are not to be had, and reading the kernel arguments at that point
+    // would put a round trip to host-visible memory into the loading role's path once per tile.
+    uint32_t ptab = 0;
+    if (GROUPED) {
+        static_assert(sizeof(GemmProblem) == 56 && kMaxGroup * 14 + kMaxGroup <= 64, "table fits the lanes of one register");
+        // the kernel arguments arrive through scalar loads (one fetch per scalar cache, not one per wave)
+        fill_table<0>(ptab, G);
+    }
+    auto tab_ptr = [&](int prob, int field) -> const void* {
+        const uint32_t lo = __builtin_amdgcn_readlane(ptab, prob * 14 + 2 * field);
+        const uint32_t hi = __builtin_amdgcn_readlane(ptab, prob * 14 + 2 * field + 1);
+        // known to be global memory: a generic pointer would turn the epilogue's stores into flat stores, which count
+        // as LDS operations too, and the next tile's first wait for its fragment reads would then wait for them
+        return (const void*)(global_ptr_t)(((uint64_t)hi << 32) | lo);
+    };
     constexpr int GROUP_M = 4;  // 4 x 8 tiles per XCD round; measured against 2, 8, 16: 0.3-0.7 % per GEMM, 0.6 % on the 7B layer
-    auto tile_origin = [&](int it, int& m0, int& n0) {
-        const int tile = xcd * per_xcd + my + it * stride;
+    auto tile_origin = [&](int it, int& m0, int& n0, int& prob) {
+        int tile = xcd * per_xcd + my + it * stride;
+        prob = 0;
+        if (GROUPED) {
+            prob = __builtin_amdgcn_readfirstlane(tile / ntiles1);
+            tile -= prob * ntiles1;
+        }
         const int width = GROUP_M * G.tiles_n;
         const int group = tile / width;
         const int gsize = min(G.tiles_m - group * GROUP_M, GROUP_M);
@@ -136,7 +198,8 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     // Slots: B(j+1) replaces A(j-1) and A(j+2) replaces B(j-1), both last read in phase 2j-2; a wave waits for its own
     // loads at the end of its compute phase (a whole phase after issuing them), before the barrier that publishes them.
     const int role = wave >> 2;                     // 0: loads B slabs, 1: loads A slabs
-    const v4i rsrc = role ? make_rsrc(G.A, (uint32_t)(G.M * G.K)) : make_rsrc(G.B, (uint32_t)(G.N * G.K));
+    const uint32_t rsrc_bytes = role ? (uint32_t)(G.M * G.K) : (uint32_t)(G.N * G.K);
+    v4i rsrc = make_rsrc(role ? G.P[0].A : G.P[0].B, rsrc_bytes);  // of the problem whose slabs are being loaded
     const int R = role ? G.M : G.N;                 // rows of the matrix this wave loads
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
     const int nstep = (G.K + BK - 1) / BK;
@@ -154,8 +217,11 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     bool ledge = false;                             // its rows run past the end of the matrix (or there is no such tile)
     auto set_load_tile = [&](int it) {
         const bool live = it < my_ntiles;
-        int m0 = 0, n0 = 0;
-        if (live) tile_origin(it, m0, n0);
+        int m0 = 0, n0 = 0, prob = 0;
+        if (live) {
+            tile_origin(it, m0, n0, prob);
+            if (GROUPED) rsrc = make_rsrc(tab_ptr(prob, role ? 0 : 1), rsrc_bytes);
+        }
         lr0 = live ? (role ? m0 : n0) : R;
         ledge = lr0 + BM > R;
 #pragma unroll
@@ -250,7 +316,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
-    const float scale = load_rt_f32(G.sa, 0, G.sa_dt) * load_rt_f32(G.sb, 0, G.sb_dt);
+    const float scale0 = load_rt_f32(G.P[0].sa, 0, G.sa_dt) * load_rt_f32(G.P[0].sb, 0, G.sb_dt);
     if (EPI != kEpiBf16) enable_fp8_saturation();
     const int half = lane >> 5;
     constexpr bool vec16 = VEC16;  // rows of C start 16-byte aligned (N % 8 == 0): 16-byte stores
@@ -259,21 +325,31 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     // meanwhile); after the last tile it runs on its own.
     for (int it = 0; it <= my_ntiles; it++) {
     if (it > 0) {
-    int m0, n0;
-    tile_origin(it - 1, m0, n0);
+    int m0, n0, prob;
+    tile_origin(it - 1, m0, n0, prob);
+    float scale = scale0;
+    void* Cp = G.P[0].C;
+    void* Csp = G.P[0].Cs;
+    const void* biasp = G.P[0].bias;
+    if (GROUPED) {
+        scale = u2f(__builtin_amdgcn_readlane(ptab, kMaxGroup * 14 + prob));
+        Cp = (void*)tab_ptr(prob, 2);
+        Csp = (void*)tab_ptr(prob, 3);
+        biasp = tab_ptr(prob, 6);
+    }
 
     // ---- epilogue (stores are not waited for: they drain while the next tile is multiplied)
-    uint8_t* const c_tile = (uint8_t*)G.C + ((int64_t)m0 * G.N + n0) * 2;  // bf16 output: origin of this tile
+    uint8_t* const c_tile = (uint8_t*)Cp + ((int64_t)m0 * G.N + n0) * 2;  // bf16 output: origin of this tile
     const uint32_t c_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * G.N + wn * (TJ * 32) + 8 * half) * 2;
     const int m_lim = G.M - m0 - wm * 128 - (lane & 31);   // row i * 32 of this lane exists iff i * 32 < m_lim
     const int n_lim = G.N - n0 - wn * (TJ * 32) - 8 * half;  // column offset c of this lane exists iff c < n_lim
     // quantized output: fp8 codes [M, N] and bf16 scales [M, N / 16] (N % 16 == 0), same addressing scheme
-    uint8_t* const q_tile = (uint8_t*)G.C + ((int64_t)m0 * G.N + n0);
-    uint8_t* const s_tile = (uint8_t*)G.Cs + ((int64_t)m0 * (G.N >> 4) + (n0 >> 4)) * 2;
+    uint8_t* const q_tile = (uint8_t*)Cp + ((int64_t)m0 * G.N + n0);
+    uint8_t* const s_tile = (uint8_t*)Csp + ((int64_t)m0 * (G.N >> 4) + (n0 >> 4)) * 2;
     const uint32_t q_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * G.N + wn * (TJ * 32) + 8 * half);
     const uint32_t s_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * (G.N >> 4) + wn * (TJ * 2)) * 2;
     const int q_n_lim = G.N - n0 - wn * (TJ * 32);          // a 16-column group at offset c exists iff c < q_n_lim
-    const bool pack_scales = (G.N & 63) == 0 && q_n_lim >= TJ * 32 && ((uintptr_t)G.Cs & 7) == 0;  // wave-uniform
+    const bool pack_scales = (G.N & 63) == 0 && q_n_lim >= TJ * 32 && ((uintptr_t)Csp & 7) == 0;  // wave-uniform
     if constexpr (EPI != kEpiBf16 && QBE > 16) {
         // Groups of 32 or 64 columns (reference linear.py:139-164 is generic in the group size): a row's 32 columns of
         // one accumulator tile sit in lanes l and l ^ 32, its 64 columns of the wave in the two tiles of those lanes, so
@@ -281,7 +357,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
         // code is formed (32 live values instead of 16; this path is off the shipped configurations, which use 16).
         constexpr int KIND = EPI == kEpiQuantE4M3 ? kE4M3 : kE5M2;
         const int sn = G.N / QBE;  // scales per row
-        uint8_t* const sw_tile = (uint8_t*)G.Cs + ((int64_t)m0 * sn + (n0 + wn * (TJ * 32)) / QBE) * 2;
+        uint8_t* const sw_tile = (uint8_t*)Csp + ((int64_t)m0 * sn + (n0 + wn * (TJ * 32)) / QBE) * 2;
         const uint32_t sw_lane_off = (uint32_t)((wm * 128 + (lane & 31)) * sn) * 2;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -293,9 +369,9 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     float t = acc[j][i][r] * scale;
-                    if (G.bias) {
+                    if (biasp) {
                         const int n = nb + 8 * (r >> 2) + (r & 3);
-                        if (n < G.N) t += load_rt_f32(G.bias, n, G.bias_dt);
+                        if (n < G.N) t += load_rt_f32(biasp, n, G.bias_dt);
                     }
                     v[j][r] = t;
                     a = fmaxf(a, fabsf(t));
@@ -338,13 +414,13 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
             float v[16];
 #pragma unroll
             for (int r = 0; r < 16; r++) v[r] = acc[j][i][r] * scale;
-            if (G.bias) {
+            if (biasp) {
 #pragma unroll
                 for (int q = 0; q < 4; q++)
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int n = nb + 8 * q + e;
-                        if (n < G.N) v[4 * q + e] += load_rt_f32(G.bias, n, G.bias_dt);
+                        if (n < G.N) v[4 * q + e] += load_rt_f32(biasp, n, G.bias_dt);
                     }
             }
             __builtin_amdgcn_sched_barrier(0);  // one accumulator tile at a time: keeps the epilogue's live ranges short
@@ -370,11 +446,11 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                     for (int q = 0; q < 4; q++) {
                         const int n = nb + 8 * q;
                         if (n + 3 < G.N) {
-                            *(uint2*)((uint16_t*)G.C + (int64_t)m * G.N + n) =
+                            *(uint2*)((uint16_t*)Cp + (int64_t)m * G.N + n) =
                                 make_uint2(pack_bf16x2(v[4 * q], v[4 * q + 1]), pack_bf16x2(v[4 * q + 2], v[4 * q + 3]));
                         } else {
                             for (int e = 0; e < 4; e++)
-                                if (n + e < G.N) ((uint16_t*)G.C)[(int64_t)m * G.N + n + e] = (uint16_t)f2bf16(v[4 * q + e]);
+                                if (n + e < G.N) ((uint16_t*)Cp)[(int64_t)m * G.N + n + e] = (uint16_t)f2bf16(v[4 * q + e]);
                         }
                     }
                 }
@@ -468,30 +544,44 @@ static std::atomic<unsigned long long*> coat_gemm_probe_buffer{nullptr};
 extern "C" void coat_gemm_set_probe(unsigned long long* buf) { coat_gemm_probe_buffer.store(buf); }
 #endif
 
-extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
-                             const void* scale_a, int sa_dtype, const void* scale_b, int sb_dtype, const void* bias,
-                             int bias_dtype, int64_t M, int64_t N, int64_t K, int QB, void* stream) {
+// Validates and launches `count` problems of one shape (count = 1: the plain GEMM).
+static int gemm_launch(int count, const void* const* a, int fmt_a, const void* const* b, int fmt_b, void* const* c,
+                       void* const* c_scale, int out_kind, const void* const* scale_a, int sa_dtype,
+                       const void* const* scale_b, int sb_dtype, const void* const* bias, int bias_dtype, int64_t M,
+                       int64_t N, int64_t K, int QB, void* stream) {
+    if (count < 1 || count > kMaxGroup) return COAT_EINVAL;
     if (M < 0 || N < 0 || K < 0) return COAT_EINVAL;
     if (M * N == 0) return COAT_OK;
     if (!a || !b || !c || !scale_a || !scale_b) return COAT_EINVAL;
     if (M >= (1 << 30) || N >= (1 << 30) || K >= (1 << 30)) return COAT_ESHAPE;
     if (K % 16 != 0) return COAT_ESHAPE;
     if (M * K >= ((int64_t)1 << 31) - 64 || N * K >= ((int64_t)1 << 31) - 64) return COAT_ESHAPE;  // 32-bit buffer offsets
-    if (!coat_aligned16(a) || !coat_aligned16(b) || !coat_aligned16(c)) return COAT_EALIGN;
     if ((fmt_a != COAT_E4M3 && fmt_a != COAT_E5M2) || (fmt_b != COAT_E4M3 && fmt_b != COAT_E5M2)) return COAT_EINVAL;
     if (out_kind < 0 || out_kind > 2) return COAT_EINVAL;
     if (out_kind != 0 && ((QB != 16 && QB != 32 && QB != 64) || N % QB != 0 || !c_scale)) return COAT_ESHAPE;
-    if (sa_dtype < 0 || sa_dtype > 2 || sb_dtype < 0 || sb_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return COAT_EDTYPE;
-    GemmArgs G;
-    G.A = (const uint8_t*)a; G.B = (const uint8_t*)b; G.C = c; G.Cs = c_scale;
-    G.sa = scale_a; G.sb = scale_b; G.bias = bias; G.sa_dt = sa_dtype; G.sb_dt = sb_dtype; G.bias_dt = bias_dtype;
+    if (sa_dtype < 0 || sa_dtype > 2 || sb_dtype < 0 || sb_dtype > 2) return COAT_EDTYPE;
+    GemmArgs G = {};
+    G.nprob = count;
+    bool any_bias = false;
+    for (int p = 0; p < count; p++) {
+        if (!a[p] || !b[p] || !c[p] || !scale_a[p] || !scale_b[p]) return COAT_EINVAL;
+        if (out_kind != 0 && !c_scale[p]) return COAT_ESHAPE;
+        if (!coat_aligned16(a[p]) || !coat_aligned16(b[p]) || !coat_aligned16(c[p])) return COAT_EALIGN;
+        G.P[p].A = (const uint8_t*)a[p]; G.P[p].B = (const uint8_t*)b[p]; G.P[p].C = c[p];
+        G.P[p].Cs = out_kind != 0 ? c_scale[p] : nullptr;
+        G.P[p].sa = scale_a[p]; G.P[p].sb = scale_b[p];
+        G.P[p].bias = bias ? bias[p] : nullptr;
+        any_bias = any_bias || G.P[p].bias;
+    }
+    if (any_bias && (bias_dtype < 0 || bias_dtype > 2)) return COAT_EDTYPE;
+    G.sa_dt = sa_dtype; G.sb_dt = sb_dtype; G.bias_dt = bias_dtype;
     G.M = (int)M; G.N = (int)N; G.K = (int)K;
     G.tiles_m = (int)((M + BM - 1) / BM);
     G.tiles_n = (int)((N + BN - 1) / BN);
 #ifdef COAT_GEMM_PROBE
     G.probe = coat_gemm_probe_buffer.load();
 #endif
-    const int ntiles = G.tiles_m * G.tiles_n;
+    const int ntiles = G.nprob * G.tiles_m * G.tiles_n;
     // persistent grid: one block per CU (the block's LDS ring takes a whole CU's LDS); CU count cached per device
     static std::atomic<int> n_cu_dev[kCoatMaxDevices];
     const int dev = coat_device_index();
@@ -506,12 +596,17 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     const int grid = min(((ntiles + 7) / 8) * 8, n_cu);
     const size_t lds_bytes = kLdsBytes;
     hipStream_t st = (hipStream_t)stream;
-#define GEMM_LAUNCH_V(FA, FB, EP, V16, QE)                                                                         \
+#define GEMM_LAUNCH_G(FA, FB, EP, V16, QE, GR)                                                                     \
     {                                                                                                              \
         static coat_device_flags lds_ok;                                                                           \
-        if (int e = coat_allow_lds(k_fp8_gemm<FA, FB, EP, V16, QE>, (int)lds_bytes, lds_ok)) return e;             \
-        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, V16, QE>), dim3(grid), dim3(512), lds_bytes, st, G);            \
+        if (int e = coat_allow_lds(k_fp8_gemm<FA, FB, EP, V16, QE, GR>, (int)lds_bytes, lds_ok)) return e;         \
+        hipLaunchKernelGGL((k_fp8_gemm<FA, FB, EP, V16, QE, GR>), dim3(grid), dim3(512), lds_bytes, st, G);        \
         return coat_launch_status();                                                                               \
+    }
+#define GEMM_LAUNCH_V(FA, FB, EP, V16, QE)                      \
+    {                                                           \
+        if (G.nprob > 1) GEMM_LAUNCH_G(FA, FB, EP, V16, QE, true) \
+        GEMM_LAUNCH_G(FA, FB, EP, V16, QE, false)               \
     }
 // the 16-byte-store epilogue only exists for the bf16 output, group sizes other than 16 only for the quantized ones
 #define GEMM_LAUNCH(FA, FB, EP)                                                       \
@@ -534,4 +629,19 @@ extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b,
     if (out_kind == 1) { GEMM_FMT(kEpiQuantE4M3) }
     if (out_kind == 2) { GEMM_FMT(kEpiQuantE5M2) }
     return COAT_EINVAL;
+}
+
+extern "C" int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
+                             const void* scale_a, int sa_dtype, const void* scale_b, int sb_dtype, const void* bias,
+                             int bias_dtype, int64_t M, int64_t N, int64_t K, int QB, void* stream) {
+    return gemm_launch(1, &a, fmt_a, &b, fmt_b, &c, &c_scale, out_kind, &scale_a, sa_dtype, &scale_b, sb_dtype, &bias,
+                       bias_dtype, M, N, K, QB, stream);
+}
+
+extern "C" int coat_fp8_gemm_grouped(int count, const void* const* a, int fmt_a, const void* const* b, int fmt_b,
+                                     void* const* c, void* const* c_scale, int out_kind, const void* const* scale_a,
+                                     int sa_dtype, const void* const* scale_b, int sb_dtype, const void* const* bias,
+                                     int bias_dtype, int64_t M, int64_t N, int64_t K, int QB, void* stream) {
+    return gemm_launch(count, a, fmt_a, b, fmt_b, c, c_scale, out_kind, scale_a, sa_dtype, scale_b, sb_dtype, bias,
+                       bias_dtype, M, N, K, QB, stream);
 }

@@ -23,7 +23,8 @@ import torch.nn.functional as F
 
 from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt, fp8_division,
-                                            fp8_division_transpose, fp8_linear_backward, fp8_linear_forward,
+                                            fp8_division_transpose, fp8_linear_backward, fp8_linear_backward_grouped,
+                                            fp8_linear_forward, fp8_linear_forward_grouped,
                                             fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
                                             fp8_rmsnorm_backward, fp8_rmsnorm_forward, fp8_silu_mul_backward,
                                             fp8_silu_mul_forward, fp8_transpose)
@@ -151,10 +152,11 @@ class _CoatLlamaBeforeAttentionResidual(torch.autograd.Function):
         in_x = _as_e4m3_input(in_x, fwobits)
         ln_x, ln_s, ln_x_t, ln_utils = fp8_rmsnorm_forward(in_x, in_s, rmsnorm_weight, group_size, eps,
                                                            transpose_output_2d=True)
-        outs = []
-        for origin, cached, scale in ((w1_origin, w1, w1_s), (w2_origin, w2, w2_s), (w3_origin, w3, w3_s)):
-            w8 = _forward_weight(origin, cached, scale, qargs, fwobits)
-            outs.append(fp8_linear_forward(ln_x, ln_s, w8, scale, False, group_size))
+        # q / k / v projections in one launch (the reference's three fp8_linear_forward calls, :267-269)
+        w8s = [_forward_weight(origin, cached, scale, qargs, fwobits)
+               for origin, cached, scale in ((w1_origin, w1, w1_s), (w2_origin, w2, w2_s), (w3_origin, w3, w3_s))]
+        outs = fp8_linear_forward_grouped(ln_x, ln_s, w8s, [w1_s, w2_s, w3_s], False, group_size)
+        del w8s
         ctx.save_for_backward(in_x, in_s, ln_x_t, ln_s)
         if qargs.weight_memory_efficient:
             ctx.weight = w1_origin, w1_s, w2_origin, w2_s, w3_origin, w3_s
@@ -171,15 +173,18 @@ class _CoatLlamaBeforeAttentionResidual(torch.autograd.Function):
         group_size = ctx.group_size
         rms_weight, rstd, num_warps = ctx.ln_utils
         fwobits, layer_id, config, qargs = ctx.utils
-        dgrads, wgrads = [], []
-        for g, (w_saved, w_s) in zip((query_g, key_g, value_g), zip(ctx.weight[0::2], ctx.weight[1::2])):
+        g8s, gss, g8_ts, w_ts = [], [], [], []
+        for g, w_saved, w_s in zip((query_g, key_g, value_g), ctx.weight[0::2], ctx.weight[1::2]):
             # the gradients leaving RoPE / attention are bf16: per-tensor e5m2 in both layouts
             g8, gs, g8_t = fp8_quantize_pertensor_transpose(g, group_size, fwobits["babit"], transpose_output_2d=True,
                                                             stochastic=False)
-            w_t = _backward_weight_t(w_saved, w_s, qargs, fwobits)
-            dx, dw = fp8_linear_backward(ln_x_t, ln_s, g8, gs, g8_t, w_t, w_s, group_size)
-            dgrads.append(dx)
-            wgrads.append(dw)
+            g8s.append(g8)
+            gss.append(gs)
+            g8_ts.append(g8_t)
+            w_ts.append(_backward_weight_t(w_saved, w_s, qargs, fwobits))
+        # the three fp8_linear_backward calls of the reference (:318-326): dgrads in one launch, wgrads in another
+        dgrads, wgrads = fp8_linear_backward_grouped(ln_x_t, ln_s, g8s, gss, g8_ts, w_ts, list(ctx.weight[1::2]), group_size)
+        del g8s, g8_ts, w_ts
         # fc1_g = dgrads[0] + dgrads[1] + dgrads[2] (reference :328), summed inside the kernel with the same roundings
         in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, tuple(dgrads), rms_weight, rstd, group_size, num_warps)
         re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],
@@ -271,10 +276,10 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
         ln_x, ln_s, ln_x_t, ln_utils = fp8_rmsnorm_forward(in_x, in_s, rmsnorm_weight, group_size, eps,
                                                            transpose_output_2d=True)
         # gate / up projections write per-group FP8 straight from the GEMM epilogue
-        gate_x, gate_s = fp8_linear_forward(ln_x, ln_s, _forward_weight(w1_origin, w1, w1_s, qargs, fwobits), w1_s, True,
-                                            group_size)
-        up_x, up_s = fp8_linear_forward(ln_x, ln_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits), w2_s, True,
-                                        group_size)
+        # (the reference's two fp8_linear_forward calls, :647-648, in one launch)
+        (gate_x, gate_s), (up_x, up_s) = fp8_linear_forward_grouped(
+            ln_x, ln_s, [_forward_weight(w1_origin, w1, w1_s, qargs, fwobits), _forward_weight(w2_origin, w2, w2_s, qargs, fwobits)],
+            [w1_s, w2_s], True, group_size)
         # one kernel for fp8_silu_forward + fp8_mul_forward of the reference (:664-668), same tensors
         silu_x, silu_s, mul_x, mul_s, mul_x_t = fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, group_size,
                                                                       transpose_output_2d=True)
@@ -312,8 +317,9 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
         # gate / up projections
         w1_t = _backward_weight_t(w1_saved, w1_s, qargs, fwobits)
         w2_t = _backward_weight_t(w2_saved, w2_s, qargs, fwobits)
-        fc1_g, weight1_grad = fp8_linear_backward(ln_x_t, ln_s, silu_g, silu_gs, silu_g_t, w1_t, w1_s, group_size)
-        fc2_g, weight2_grad = fp8_linear_backward(ln_x_t, ln_s, mul_g2, mul_gs2, mul_g2_t, w2_t, w2_s, group_size)
+        # (the reference's two fp8_linear_backward calls, :735-740: dgrads in one launch, wgrads in another)
+        (fc1_g, fc2_g), (weight1_grad, weight2_grad) = fp8_linear_backward_grouped(
+            ln_x_t, ln_s, [silu_g, mul_g2], [silu_gs, mul_gs2], [silu_g_t, mul_g2_t], [w1_t, w2_t], [w1_s, w2_s], group_size)
         # fc_g = fc1_g + fc2_g (reference :742), summed inside the kernel
         in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, (fc1_g, fc2_g), rms_weight, rstd, group_size, num_warps)
         re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],

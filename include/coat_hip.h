@@ -256,6 +256,18 @@ int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, v
                   const void* scale_a, int sa_dtype, const void* scale_b, int sb_dtype, const void* bias, int bias_dtype,
                   int64_t M, int64_t N, int64_t K, int QB, void* stream);
 
+/* `count` (1 .. 4) such products of one shape and one pair of formats in one launch: problem i is
+ * (a[i], b[i], c[i], c_scale[i], scale_a[i], scale_b[i], bias[i]); the seven arrays are host arrays of `count` device
+ * pointers, read before the call returns (c_scale may be NULL for out_kind 0, bias may be NULL or hold NULLs).  Every
+ * result is bit-identical to coat_fp8_gemm on the same problem.  The reference calls fp8matmul once per projection
+ * (coat/models/coat_llama.py:267-269 q / k / v, :647-648 gate / up, and their backward :318-326, :735-740); on a persistent grid of
+ * 256 x 256 tiles the problems' tiles are taken as one sequence, so the partial last round of tiles is paid once per
+ * group. */
+int coat_fp8_gemm_grouped(int count, const void* const* a, int fmt_a, const void* const* b, int fmt_b, void* const* c,
+                          void* const* c_scale, int out_kind, const void* const* scale_a, int sa_dtype,
+                          const void* const* scale_b, int sb_dtype, const void* const* bias, int bias_dtype, int64_t M,
+                          int64_t N, int64_t K, int QB, void* stream);
+
 /* ---- optimizer -------------------------------------------------------------------------------- */
 
 /* qoptim_cuda.fp8_adamw_expand_step (coat/optimizer/kernels/bindings.cpp:7,

@@ -114,6 +114,26 @@ class Recorder:
         self.calls = []
         for name in RECORDED:
             monkeypatch.setattr(L, name, self._wrap(name, getattr(L, name)))
+        # the modules launch the projections of one input together; each such call is logged as the per-projection calls
+        # of the reference that it stands for, so the checks below read like the reference's call sequence
+        monkeypatch.setattr(L, "fp8_linear_forward_grouped", self._wrap_forward_grouped(L.fp8_linear_forward_grouped))
+        monkeypatch.setattr(L, "fp8_linear_backward_grouped", self._wrap_backward_grouped(L.fp8_linear_backward_grouped))
+
+    def _wrap_forward_grouped(self, fn):
+        def wrapper(x, s, w_list, s_w_list, output_quantize, QB):
+            outs = fn(x, s, w_list, s_w_list, output_quantize, QB)
+            for w, s_w, out in zip(w_list, s_w_list, outs):
+                self.calls.append(("fp8_linear_forward", (x, s, w, s_w, output_quantize, QB), {}, out))
+            return outs
+        return wrapper
+
+    def _wrap_backward_grouped(self, fn):
+        def wrapper(x_t, s, g_list, s_g_list, g_t_list, w_t_list, s_w_list, QB):
+            dxs, dws = fn(x_t, s, g_list, s_g_list, g_t_list, w_t_list, s_w_list, QB)
+            for g, s_g, g_t, w_t, s_w, dx, dw in zip(g_list, s_g_list, g_t_list, w_t_list, s_w_list, dxs, dws):
+                self.calls.append(("fp8_linear_backward", (x_t, s, g, s_g, g_t, w_t, s_w, QB), {}, (dx, dw)))
+            return dxs, dws
+        return wrapper
 
     def _wrap(self, name, fn):
         def wrapper(*args, **kwargs):

@@ -176,3 +176,83 @@ def test_fp8matmul_scales_in_different_dtypes(dev):
     cq, cs = lin.fp8matmul(a.to(dev), b.to(dev).t(), True, sb.to(dev), sa.to(dev), 16)
     wq, ws = R._quantize_pg(acc * (sb * sa.float()), 16, E4)
     assert torch.equal(cq.cpu().view(torch.uint8), wq.view(torch.uint8)) and torch.equal(cs.cpu(), ws)
+
+
+@pytest.mark.parametrize("count,M,N,K,fa,fb,quant", [
+    (3, 512, 512, 256, E4, E4, False),      # q / k / v forward: 12 tiles, problems change inside a block's walk
+    (2, 300, 272, 144, E5, E4, False),      # ragged tiles, partial last K-step, e5m2 gradients
+    (2, 768, 512, 384, E4, E4, True),       # gate / up forward through the quantizing epilogue
+    (4, 2304, 2048, 128, E5, E4, False),    # 4 x 72 tiles: more tiles than CUs, every XCD band spans problems
+])
+def test_grouped_gemm_equals_separate_launches(dev, count, M, N, K, fa, fb, quant):
+    """coat_fp8_gemm_grouped through the C ABI: every problem's output is bit-identical to coat_fp8_gemm on it."""
+    import ctypes
+    from coat_amd import _hip
+    lib = _hip.lib()
+    a = [rand_fp8((M, K), 100 + i, fa).to(dev) for i in range(count)]
+    b = [rand_fp8((N, K), 200 + i, fb).to(dev) for i in range(count)]
+    sa = [torch.tensor(0.02 + 0.003 * i).bfloat16().to(dev) for i in range(count)]
+    sb = [torch.tensor(0.013 - 0.002 * i).float().to(dev) for i in range(count)]
+    kind = {E4: 1, E5: 2}[fa] if quant else 0
+    odt = fa if quant else torch.bfloat16
+    want = [torch.empty((M, N), dtype=odt, device=dev) for _ in range(count)]
+    got = [torch.zeros((M, N), dtype=torch.uint8, device=dev).view(odt) if quant else torch.zeros((M, N), dtype=odt, device=dev)
+           for _ in range(count)]
+    want_s = [torch.empty((M, N // 16), dtype=torch.bfloat16, device=dev) for _ in range(count)] if quant else None
+    got_s = [torch.zeros((M, N // 16), dtype=torch.bfloat16, device=dev) for _ in range(count)] if quant else None
+    st = _hip.stream(dev)
+    for i in range(count):
+        _hip.check(lib.coat_fp8_gemm(_hip.ptr(a[i]), _hip.fp8(fa), _hip.ptr(b[i]), _hip.fp8(fb), _hip.ptr(want[i]),
+                                     _hip.ptr(want_s[i]) if quant else None, kind, _hip.ptr(sa[i]), _hip.dt(sa[i]),
+                                     _hip.ptr(sb[i]), _hip.dt(sb[i]), None, 0, M, N, K, 16 if quant else 0, st), "gemm")
+    _hip.check(lib.coat_fp8_gemm_grouped(count, _hip.ptr_array(a), _hip.fp8(fa), _hip.ptr_array(b), _hip.fp8(fb),
+                                         _hip.ptr_array(got), _hip.ptr_array(got_s) if quant else None, kind,
+                                         _hip.ptr_array(sa), _hip.dt(sa[0]), _hip.ptr_array(sb), _hip.dt(sb[0]), None, 0,
+                                         M, N, K, 16 if quant else 0, st), "gemm_grouped")
+    for i in range(count):
+        assert torch.equal(got[i].view(torch.uint8), want[i].view(torch.uint8)), i
+        if quant:
+            assert torch.equal(got_s[i].view(torch.int16), want_s[i].view(torch.int16)), i
+    # the first problem against the oracle's bound as well
+    if not quant:
+        check_bf16(got[0], a[0].cpu(), b[0].cpu(), sa[0].cpu(), sb[0].cpu())
+
+
+def test_grouped_linear_wrappers_equal_the_separate_calls(dev):
+    """fp8_linear_forward_grouped / fp8_linear_backward_grouped against the per-projection functions, with a bias vector in
+    one problem of the C call (bias is per problem) and with projections of different widths (falls back to separate calls)."""
+    from coat_amd import _hip
+    lin = _lin()
+    T, H = 384, 256
+    x, xt = rand_fp8((T, H), 1, E4).to(dev), rand_fp8((H, T), 2, E4).to(dev)
+    s = torch.tensor(0.031).bfloat16().to(dev)
+    ws = [rand_fp8((H, H), 10 + i, E4).to(dev) for i in range(3)]
+    wts = [rand_fp8((H, H), 20 + i, E4).to(dev) for i in range(3)]
+    sws = [torch.tensor(0.01 * (i + 1)).bfloat16().to(dev) for i in range(3)]
+    gs8 = [rand_fp8((T, H), 30 + i, E5).to(dev) for i in range(3)]
+    gts = [rand_fp8((H, T), 40 + i, E5).to(dev) for i in range(3)]
+    sgs = [torch.tensor(0.002 * (i + 1)).bfloat16().to(dev) for i in range(3)]
+    outs = lin.fp8_linear_forward_grouped(x, s, ws, sws, False, 16)
+    for o, w, sw in zip(outs, ws, sws):
+        assert torch.equal(o, lin.fp8_linear_forward(x, s, w, sw, False, 16))
+    outs = lin.fp8_linear_forward_grouped(x, s, ws[:2], sws[:2], True, 16)
+    for (q, qs), w, sw in zip(outs, ws, sws):
+        wq, wqs = lin.fp8_linear_forward(x, s, w, sw, True, 16)
+        assert torch.equal(q.view(torch.uint8), wq.view(torch.uint8)) and torch.equal(qs, wqs)
+    dxs, dws = lin.fp8_linear_backward_grouped(xt, s, gs8, sgs, gts, wts, sws, 16)
+    for i in range(3):
+        dx, dw = lin.fp8_linear_backward(xt, s, gs8[i], sgs[i], gts[i], wts[i], sws[i], 16)
+        assert torch.equal(dxs[i], dx) and torch.equal(dws[i], dw)
+    # grouped-query shapes: k / v narrower than q -> separate launches, same results
+    wk = rand_fp8((H // 4, H), 50, E4).to(dev)
+    outs = lin.fp8_linear_forward_grouped(x, s, [ws[0], wk], sws[:2], False, 16)
+    assert outs[1].shape == (T, H // 4) and torch.equal(outs[1], lin.fp8_linear_forward(x, s, wk, sws[1], False, 16))
+    # bias in the second problem only
+    lib = _hip.lib()
+    bias = torch.randn(H, generator=torch.Generator().manual_seed(7)).bfloat16().to(dev)
+    got = [torch.zeros((T, H), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+    _hip.check(lib.coat_fp8_gemm_grouped(2, _hip.ptr_array([x, x]), 0, _hip.ptr_array(ws[:2]), 0, _hip.ptr_array(got), None, 0,
+                                         _hip.ptr_array([s, s]), _hip.dt(s), _hip.ptr_array(sws[:2]), _hip.dt(sws[0]),
+                                         _hip.ptr_array([None, bias]), _hip.dt(bias), T, H, H, 0, _hip.stream(dev)), "grouped")
+    assert torch.equal(got[0], lin.fp8matmul(x, ws[0].t(), False, s, sws[0], 16))
+    assert torch.equal(got[1], lin.fp8matmul(x, ws[1].t(), False, s, sws[1], 16, bias))

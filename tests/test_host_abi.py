@@ -111,6 +111,16 @@ def test_argument_validation_of_the_remaining_entry_points_without_gpu():
     assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 1, p, 1, p, 1, None, 0, 64, 64, 64, 16, None) == ESHAPE    # quantized output without scales
     assert L.coat_fp8_gemm(p, 3, p, 0, p, None, 0, p, 1, p, 1, None, 0, 64, 64, 64, 16, None) == EINVAL    # unknown operand format
     assert L.coat_fp8_gemm(p, 0, p, 0, p, None, 0, p, 1, p, 1, None, 0, 0, 64, 64, 16, None) == 0          # empty
+    pa = (ctypes.c_void_p * 5)(*[p.value] * 5)      # host arrays of pointers for the grouped GEMM
+    pn = (ctypes.c_void_p * 2)(p.value, None)
+    po = (ctypes.c_void_p * 2)(p.value, odd.value)
+    assert L.coat_fp8_gemm_grouped(0, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 64, 16, None) == EINVAL   # no problem
+    assert L.coat_fp8_gemm_grouped(5, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 64, 16, None) == EINVAL   # more than four
+    assert L.coat_fp8_gemm_grouped(2, pa, 0, pn, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 64, 16, None) == EINVAL   # second B missing
+    assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, po, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 64, 16, None) == EALIGN   # second C misaligned
+    assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, pa, pn, 1, pa, 1, pa, 1, None, 0, 64, 64, 64, 16, None) == ESHAPE     # second scale output missing
+    assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 24, 16, None) == ESHAPE   # K % 16
+    assert L.coat_fp8_gemm_grouped(3, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 0, 64, 16, None) == 0         # empty
     # RoPE, cross-entropy, probe
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 24, 0, 0, 0, None) == ESHAPE                      # head_dim % 16
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 48, 0, None) == ESHAPE                     # pitch < heads * head_dim
