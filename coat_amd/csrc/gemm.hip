@@ -284,15 +284,22 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
 #define COAT_MFMA(FB_, FA_, J, I) \
     acc[J][I] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(FB_[J], FA_[I], acc[J][I], FMT_B, FMT_A, 0, 0, 0, 0)
     static_assert(TJ == 2 && NW == 8, "the schedule is written for eight waves of 128 x 64");
+    // The four groups of fragment reads are kept in this order (scheduling barriers): left to itself the compiler
+    // hoisted the address additions and issued the reads in another order in one instantiation of this kernel, whose
+    // K loop then ran 3 % slower with otherwise the same instructions (the loop sits at the LDS limit).
     auto mem_phase = [&]() {
 #pragma unroll
         for (int t = 0; t < 4; t++) fax[t] = load_fa(sl_frag, 0, t);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < TJ; t++) fbx[t] = load_fb(sl_frag, 0, t);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < 4; t++) fay[t] = load_fa(sl_frag, 1, t);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < TJ; t++) fby[t] = load_fb(sl_frag, 1, t);
+        __builtin_amdgcn_sched_barrier(0);
         sl_frag = sl_frag + 2 >= NUNIT ? sl_frag + 2 - NUNIT : sl_frag + 2;
         issue_slab();
         // every fragment has arrived before the barrier: the compute phase has nothing to wait for, and the slabs
