@@ -59,6 +59,10 @@ def new_max(device):
     device = torch.device(device)
     if device.type != "cuda":
         return torch.zeros(_hip.MAX_WORDS, dtype=torch.float32, device=device)
+    if torch.cuda.is_current_stream_capturing():
+        # under graph capture the zero fill has to be a node of the graph (a pool zeroed before the capture would keep the
+        # maxima of earlier replays), and memory of the graph's private pool must not be handed out after the capture
+        return torch.zeros(_hip.MAX_WORDS, dtype=torch.float32, device=device)
     key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
     pool = _MAX_POOL.get(key)
     if pool is None or pool[1] >= _MAX_POOL_SIZE:

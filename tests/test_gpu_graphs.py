@@ -1,0 +1,126 @@
+"""The C ABI under HIP graph capture: the entry points allocate nothing, never synchronise and enqueue kernels only (no
+memset nodes), so a chain of them can be captured once and replayed.  A graph of a forward chain (per-group quantize,
+RMSNorm with its per-tensor division, three projections in one grouped GEMM launch, fused SiLU * mul, per-tensor quantize
+with transpose, a plain GEMM) is replayed several times on new input data, with eager work and synchronisations of the
+program between the replays, and every replay is compared bit for bit with the same chain run eagerly."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _chain(x, w_rms, wq, ws, w_down, s_down):
+    """x bf16 [T, H] -> a list of output tensors.  Only stream-ordered work: no host reads of device data."""
+    import coat_amd.activation.real_quantization as rq
+    from coat_amd.activation.real_quantization import linear as lin
+    q, s = rq.fp8_quantize(x, 16, "E4M3")
+    ln_x, ln_s, ln_x_t, (_, rstd, _) = rq.fp8_rmsnorm_forward(q, s, w_rms, 16, 1e-5, transpose_output_2d=True)
+    (g_q, g_s), (u_q, u_s) = lin.fp8_linear_forward_grouped(ln_x, ln_s, wq[:2], ws[:2], True, 16)
+    y3 = lin.fp8_linear_forward_grouped(ln_x, ln_s, wq, ws, False, 16)
+    silu_x, silu_s, mul_x, mul_s, mul_x_t = rq.fp8_silu_mul_forward(g_q, g_s, u_q, u_s, 16, transpose_output_2d=True)
+    down = lin.fp8_linear_forward(mul_x, mul_s, w_down, s_down, False, 16)
+    pq, ps, pqt = rq.fp8_quantize_pertensor_transpose(down, 16, "E5M2", transpose_output_2d=True)
+    outs = [q, s, ln_x, ln_s, ln_x_t, rstd, g_q, g_s, u_q, u_s, *y3, silu_x, silu_s, mul_x, mul_s, mul_x_t, down, pq, ps, pqt]
+    return [o.view(torch.uint8) if o.dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else o for o in outs]
+
+
+def test_captured_chain_replays_bit_identically(dev):
+    import coat_amd.activation.real_quantization as rq
+    T, H = 512, 512
+    gen = torch.Generator(device=dev).manual_seed(3)
+    w_rms = (1 + 0.1 * torch.randn(H, generator=gen, device=dev)).bfloat16()
+    wq, ws = [], []
+    for i in range(3):
+        w = (torch.randn(H, H, generator=gen, device=dev) * 0.05).bfloat16()
+        q8, s8, _ = rq.fp8_quantize_pertensor_transpose(w, 16, "E4M3", transpose_output_2d=True)
+        wq.append(q8)
+        ws.append(s8)
+    w_down, s_down = wq[2], ws[2]
+    inputs = [(torch.randn(T, H, generator=gen, device=dev) * (0.5 + i)).bfloat16() for i in range(4)]
+    static_x = inputs[0].clone()
+
+    side = torch.cuda.Stream(device=dev)  # default priority
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):  # warm-up outside the capture (first-use attribute calls of the library, allocator)
+        for _ in range(2):
+            _chain(static_x, w_rms, wq, ws, w_down, s_down)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize(dev)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = _chain(static_x, w_rms, wq, ws, w_down, s_down)
+    torch.cuda.synchronize(dev)
+
+    for i, x in enumerate(inputs):
+        want = [o.clone() for o in _chain(x, w_rms, wq, ws, w_down, s_down)]  # eager work between the replays
+        torch.cuda.synchronize(dev)
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        assert len(static_out) == len(want)
+        for k, (got, ref) in enumerate(zip(static_out, want)):
+            assert torch.equal(got, ref), f"replay {i}: output {k} differs from the eager run"
+    # and the first input once more, after the others: nothing of an earlier replay may survive in the outputs
+    want = [o.clone() for o in _chain(inputs[0], w_rms, wq, ws, w_down, s_down)]
+    static_x.copy_(inputs[0])
+    graph.replay()
+    torch.cuda.synchronize(dev)
+    for k, (got, ref) in enumerate(zip(static_out, want)):
+        assert torch.equal(got, ref), f"last replay: output {k} differs from the eager run"
+
+
+def test_captured_backward_chain_replays_bit_identically(dev):
+    """The backward half of an MLP block under capture: fused SiLU * mul backward with its two per-tensor divisions, the
+    gate / up dgrads and wgrads as two grouped GEMM launches, the RMSNorm backward (partial rows in a workspace plus the
+    column sum) on the two dgrads, and the residual addition with its e5m2 quantization."""
+    import coat_amd.activation.real_quantization as rq
+    from coat_amd.activation.real_quantization import linear as lin
+    T, H, I = 512, 256, 768
+    gen = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn(T, H, generator=gen, device=dev).bfloat16()
+    w_rms = (1 + 0.1 * torch.randn(H, generator=gen, device=dev)).bfloat16()
+    q, s = rq.fp8_quantize(x, 16, "E4M3")
+    ln_x, ln_s, ln_x_t, (_, rstd, nw) = rq.fp8_rmsnorm_forward(q, s, w_rms, 16, 1e-5, transpose_output_2d=True)
+    wq, wqt, ws = [], [], []
+    for i in range(2):
+        w = (torch.randn(I, H, generator=gen, device=dev) * 0.05).bfloat16()
+        a8, s8, a8t = rq.fp8_quantize_pertensor_transpose(w, 16, "E4M3", transpose_output_2d=True)
+        wq.append(a8)
+        wqt.append(a8t)
+        ws.append(s8)
+    (g_q, g_s), (u_q, u_s) = lin.fp8_linear_forward_grouped(ln_x, ln_s, wq, ws, True, 16)
+    silu_x, silu_s, _, _, _ = rq.fp8_silu_mul_forward(g_q, g_s, u_q, u_s, 16, transpose_output_2d=True)
+    torch.cuda.synchronize(dev)
+
+    def backward(g, fp_grad):
+        (sg, sgs, sg_t), (ug, ugs, ug_t) = rq.fp8_silu_mul_backward(g_q, g_s, u_q, u_s, silu_x, silu_s, g, 16, "E5M2")
+        (d1, d2), (dw1, dw2) = lin.fp8_linear_backward_grouped(ln_x_t, ln_s, [sg, ug], [sgs, ugs], [sg_t, ug_t], wqt, ws, 16)
+        dx, dw = rq.fp8_rmsnorm_backward(q, s, (d1, d2), w_rms, rstd, 16, nw)
+        re_g, (in_g, in_sg, in_sg16) = rq.fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, dx, 16, "E5M2")
+        outs = [sg, sgs, sg_t, ug, ugs, ug_t, d1, d2, dw1, dw2, dx, dw, re_g, in_g, in_sg, in_sg16]
+        return [o.view(torch.uint8) if o.dtype in (torch.float8_e4m3fn, torch.float8_e5m2) else o for o in outs]
+
+    grads = [((torch.randn(T, I, generator=gen, device=dev) * 1e-2 * (i + 1)).bfloat16(),
+              (torch.randn(T, H, generator=gen, device=dev) * 1e-2).bfloat16()) for i in range(3)]
+    static_g, static_fp = grads[0][0].clone(), grads[0][1].clone()
+    side = torch.cuda.Stream(device=dev)  # default priority
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            backward(static_g, static_fp)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = backward(static_g, static_fp)
+    torch.cuda.synchronize(dev)
+    for i, (g, fp) in enumerate(grads + grads[:1]):
+        want = [o.clone() for o in backward(g, fp)]  # eager work between the replays
+        torch.cuda.synchronize(dev)
+        static_g.copy_(g)
+        static_fp.copy_(fp)
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        for k, (got, ref) in enumerate(zip(static_out, want)):
+            assert torch.equal(got, ref), f"replay {i}: output {k} differs from the eager run"
