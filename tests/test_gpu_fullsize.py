@@ -80,6 +80,27 @@ def test_gemm_llama_mlp_shapes(dev, M, N, K, fa):
         torch.backends.cuda.matmul.allow_tf32 = prev
 
 
+@pytest.mark.parametrize("count,M,N,K,fa,quant", [
+    (3, 8192, 5120, 5120, E4, False),    # 13B q / k / v forward: 3 x 640 tiles = 7.5 rounds of 256 tiles
+    (3, 5120, 5120, 8192, E5, False),    # their wgrads: 3 x 400 tiles
+    (2, 8192, 13824, 5120, E4, True),    # 13B gate / up forward through the quantizing epilogue: 2 x 1728 tiles
+])
+def test_grouped_gemm_llama_13b_shapes(dev, count, M, N, K, fa, quant):
+    """The grouped launches of the 13B decoder layer at 4 x 2048 tokens: every problem bit-identical to its own launch."""
+    from coat_amd.activation.real_quantization import linear
+    a = [randn(dev, (M, K), 20 + i, 1.0, torch.float32).to(fa) for i in range(count)]
+    b = [randn(dev, (N, K), 30 + i, 1.0, torch.float32).to(E4) for i in range(count)]
+    sa = [torch.tensor(0.02 + 0.001 * i, device=dev).bfloat16() for i in range(count)]
+    sb = [torch.tensor(0.013 + 0.002 * i, device=dev).bfloat16() for i in range(count)]
+    got = linear.fp8matmul_grouped(a, [x.t() for x in b], quant, sa, sb, 16)
+    for i in range(count):
+        want = linear.fp8matmul(a[i], b[i].t(), quant, sa[i], sb[i], 16)
+        if quant:
+            assert torch.equal(got[i][0].view(torch.uint8), want[0].view(torch.uint8)) and torch.equal(got[i][1], want[1]), i
+        else:
+            assert torch.equal(got[i], want), i
+
+
 def test_silu_mul_llama_mlp(dev):
     rq = _rq()
     M, N, QB = 8192, 11008, 16
