@@ -47,9 +47,9 @@ struct GemmProblem {
     const void* sb;
     const void* bias;   // [N] or nullptr
 };
-// The shape and the first problem come first: a wave reads its kernel arguments from host-visible memory when it starts,
-// and the plain GEMM then touches two 64-byte lines of them as it would without the group (with the seven pointers laid
-// out as arrays of four the same kernel ran 1.3 % slower on config 3).
+// The shape and the first problem come first: a wave fetches its kernel arguments when it starts (the host writes them per
+// launch, so they are not in any cache), and the plain GEMM then touches two 64-byte lines of them as it would without the
+// group (with the seven pointers laid out as arrays of four the same kernel ran 1.3 % slower on config 3).
 struct GemmArgs {
     int sa_dt, sb_dt, bias_dt;
     int M, N, K;
@@ -101,7 +101,7 @@ template <int LANE> __device__ __forceinline__ void write_lane_ptr(uint32_t& t, 
 // product of the two scales.
 template <int P> __device__ __forceinline__ void fill_table(uint32_t& t, const GemmArgs& G) {
     if constexpr (P < kMaxGroup) {
-        if (P < G.nprob) {  // (the arguments of unused problems are not even fetched: they are lines of host-visible memory)
+        if (P < G.nprob) {  // (the arguments of unused problems are not even fetched)
             write_lane_ptr<14 * P + 0>(t, G.P[P].A);
             write_lane_ptr<14 * P + 2>(t, G.P[P].B);
             write_lane_ptr<14 * P + 4>(t, G.P[P].C);
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
     // Grouped launch: the problems' pointers and scales are kept across the lanes of one VGPR (lane 14 p + 2 f and the
     // next: pointer f of problem p as two dwords; lane 56 + p: its combined scale) and fetched with v_readlane when a
     // tile begins: scalar registers for four problems are not to be had, and reading the kernel arguments at that point
-    // would put a round trip to host-visible memory into the loading role's path once per tile.
+    // would put a scalar load and its wait into the loading role's path once per tile.
     uint32_t ptab = 0;
     if (GROUPED) {
         static_assert(sizeof(GemmProblem) == 56 && kMaxGroup * 14 + kMaxGroup <= 64, "table fits the lanes of one register");
