@@ -183,6 +183,7 @@ def test_fp8matmul_scales_in_different_dtypes(dev):
     (2, 300, 272, 144, E5, E4, False),      # ragged tiles, partial last K-step, e5m2 gradients
     (2, 768, 512, 384, E4, E4, True),       # gate / up forward through the quantizing epilogue
     (4, 2304, 2048, 128, E5, E4, False),    # 4 x 72 tiles: more tiles than CUs, every XCD band spans problems
+    (3, 200, 208, 80, E4, E5, True),        # ragged tiles through the quantizing epilogue (scales stored one by one)
 ])
 def test_grouped_gemm_equals_separate_launches(dev, count, M, N, K, fa, fb, quant):
     """coat_fp8_gemm_grouped through the C ABI: every problem's output is bit-identical to coat_fp8_gemm on it."""
