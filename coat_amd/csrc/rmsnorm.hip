@@ -271,8 +271,11 @@ __global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__
 // they are added in wave order through LDS, 1024 columns at a time, into the block's partial row.
 // MULTI: up to two further gradients of the same tensor are added to dy (dy2, dy3).  A variant of its own, because the
 // extra loads in flight cost it the second resident block per CU, which the single-gradient kernel keeps.
+// Five chunks (the 5120 columns of the 13B shape) with several gradients need 268 registers; held to 256, i.e. to two
+// waves per SIMD with 12 registers spilled, the kernel takes 91 us per call in the 13B layer against 104 us with one wave
+// per SIMD and no spill (128.7 us as 5 of 8 chunks, loaded chunk by chunk).
 template <int KIND, int WDT, int CH, bool MULTI>
-__global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+__global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
                                                       const void* __restrict__ dy, const void* __restrict__ dy2,
                                                       const void* __restrict__ dy3, const void* __restrict__ w,
                                                       const float* __restrict__ rstd_in, void* __restrict__ dx,
@@ -337,7 +340,7 @@ __global__ __launch_bounds__(256) void k_rmsnorm_bwd(const uint8_t* __restrict__
                 g[c][0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
                 g[c][1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
             };
-            if constexpr (CH <= 4) {  // a whole row of one gradient at a time: two round trips instead of 2 x CH
+            if constexpr (CH <= 5) {  // a whole row of one gradient at a time: two round trips instead of 2 x CH
                 uint4 r[CH][2];
                 auto load_all = [&](const void* src) {
 #pragma unroll
@@ -445,7 +448,8 @@ static int rms_check(int64_t M, int64_t N, int QB) {
     return COAT_OK;
 }
 
-// Rows up to 8192 columns go to the wave-per-row kernels (CH = 4 or 8 chunks of 16 per lane), wider rows (up to 16384) to
+// Rows up to 8192 columns go to the wave-per-row kernels (CH = 4, 5 or 8 chunks of 16 per lane; 5 is the 5120 columns of
+// the 13B shape, which as 5 of 8 chunks ran at 0.6 of the rate of the 4096-column rows), wider rows (up to 16384) to
 // the block-per-row kernels.  KW = fp8 kind * 3 + weight dtype.
 #ifndef COAT_RMS_FWD_BLOCKS
 #define COAT_RMS_FWD_BLOCKS 768
@@ -471,6 +475,9 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
     case K * 3 + W:                                                                                                    \
         if (N <= 4096)                                                                                                 \
             hipLaunchKernelGGL((k_rmsnorm_fwd<K, W, 4>), dim3((unsigned)wave_blocks), dim3(256), 0, st, (const uint8_t*)x, s_x, \
+                               s_dtype, w, y, s_row, rstd, s_max, M, (int)N, QB, eps);                                 \
+        else if (N <= 5120)                                                                                            \
+            hipLaunchKernelGGL((k_rmsnorm_fwd<K, W, 5>), dim3((unsigned)wave_blocks), dim3(256), 0, st, (const uint8_t*)x, s_x, \
                                s_dtype, w, y, s_row, rstd, s_max, M, (int)N, QB, eps);                                 \
         else if (N <= 8192)                                                                                            \
             hipLaunchKernelGGL((k_rmsnorm_fwd<K, W, 8>), dim3((unsigned)wave_blocks), dim3(256), 0, st, (const uint8_t*)x, s_x, \
@@ -505,6 +512,9 @@ static int rms_backward_launch(const void* x, int fp8, const void* s_x, int s_dt
         if (N <= 4096) {                                                                                               \
             if (dy2) RMS_BWD_WAVE(K, W, 4, true);                                                                      \
             else RMS_BWD_WAVE(K, W, 4, false);                                                                         \
+        } else if (N <= 5120) {                                                                                        \
+            if (dy2) RMS_BWD_WAVE(K, W, 5, true);                                                                      \
+            else RMS_BWD_WAVE(K, W, 5, false);                                                                         \
         } else if (N <= 8192) {                                                                                        \
             if (dy2) RMS_BWD_WAVE(K, W, 8, true);                                                                      \
             else RMS_BWD_WAVE(K, W, 8, false);                                                                         \

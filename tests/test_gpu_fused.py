@@ -261,10 +261,12 @@ def test_fused_silu_mul_on_column_slices_and_joined_backward(dev, QBv):
     assert gs_.item() == ds_.item() and torch.equal(b(gq), b(dq)) and torch.equal(b(uqt), b(eqt))
 
 
-def test_rmsnorm_backward_sums_gradients_like_bf16_additions(dev):
-    """g given as a tuple: identical to adding the bf16 tensors first (the reference's callers do that with torch)."""
+@pytest.mark.parametrize("N", [1024, 5120, 4096 + 2048, 8192 + 1024])
+def test_rmsnorm_backward_sums_gradients_like_bf16_additions(dev, N):
+    """g given as a tuple: identical to adding the bf16 tensors first (the reference's callers do that with torch).  The
+    widths take the wave-per-row kernels with 4, 5 and 8 chunks per lane and the block-per-row kernel."""
     rq = _rq()
-    M, N = 96, 1024
+    M = 96
     x = rand(50, shape=(M, N))
     w = (1 + 0.1 * rand(51, shape=(N,)).float()).bfloat16()
     g1, g2, g3 = rand(52, 0.01, shape=(M, N)), rand(53, 0.01, shape=(M, N)), rand(54, 0.02, shape=(M, N))
