@@ -73,6 +73,20 @@ def new_max(device):
     return pool[0][i * _hip.MAX_WORDS:(i + 1) * _hip.MAX_WORDS]
 
 
+def scale_max(s):
+    """``s.max()`` for a tensor of (non-negative) scales, as a 0-dim tensor of its dtype: the scale with which a tensor
+    quantized per tensor was divided is the maximum of the per-group scale tensor that travels with it (reference
+    coat/models/coat_llama.py:474, :706).  One pass of the library's abs-max kernel instead of torch's reduction, which
+    takes a memset and a kernel of 12 us for these 4 MB and, under HIP graph capture, records a memset node."""
+    from ... import _hip
+    if not s.is_cuda or s.numel() == 0 or s.dtype not in (torch.bfloat16, torch.float32, torch.float16):
+        return s.max()
+    s = _hip.dense(s)
+    amax = new_max(s.device)
+    _hip.check(_hip.lib().coat_absmax(_hip.ptr(s), _hip.dt(s), _hip.ptr(amax), s.numel(), _hip.stream(s.device)), "scale_max")
+    return read_max(amax).to(s.dtype)
+
+
 def read_max(buf):
     """The maximum held by a ``new_max`` buffer, as a 0-dim fp32 tensor (for host-side code; the division kernels read
     the slots themselves)."""

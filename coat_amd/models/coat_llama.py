@@ -28,6 +28,7 @@ from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_If
                                             fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
                                             fp8_rmsnorm_backward, fp8_rmsnorm_forward, fp8_silu_mul_backward,
                                             fp8_silu_mul_forward, fp8_transpose)
+from ..activation.real_quantization.common import scale_max
 from ..utils._fp8_quantization_config import QuantizationConfig
 from ..utils._fp8_weightcache import FP8CacheWeightModule
 from ..utils._fp8manager import FP8Manager
@@ -235,7 +236,7 @@ class _CoatLlamaAfterAttentionResidual(torch.autograd.Function):
         group_size = ctx.group_size
         fwobits, layer_id, config, qargs = ctx.utils
         out_g = _as_e5m2_grad(out_g, fwobits)
-        out_gs_max = out_gs.max()
+        out_gs_max = scale_max(out_gs)
         out_g_t = fp8_transpose(out_g, transpose_output_2d=True)
         flash_x_t, flash_s = fp8_division_transpose(flash_x, group_size, fwobits["fabit"], flash_s, stochastic=False,
                                                     only_transposed=True)
@@ -304,7 +305,7 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
         rms_weight, rstd, num_warps = ctx.ln_utils
         fwobits, layer_id, config, qargs = ctx.utils
         out_g = _as_e5m2_grad(out_g, fwobits)
-        out_gs_max = out_gs.max()
+        out_gs_max = scale_max(out_gs)
         # down projection
         out_g_t = fp8_transpose(out_g, transpose_output_2d=True)
         w3_t = _backward_weight_t(w3_saved, w3_s, qargs, fwobits)

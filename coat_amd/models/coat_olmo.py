@@ -20,6 +20,7 @@ from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_If
                                             fp8_layernorm_noparam_forward, fp8_linear_backward, fp8_linear_forward,
                                             fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
                                             fp8_silu_mul_backward_joined, fp8_silu_mul_forward, fp8_transpose)
+from ..activation.real_quantization.common import scale_max
 from ..utils._fp8_quantization_config import QuantizationConfig
 from .coat_llama import (E4M3, _as_e4m3_input, _as_e5m2_grad, _backward_weight_t, _forward_weight, _ResidualBase,
                          apply_rotary_pos_emb, fused_qkv_rotary, fused_rotary, rotary_cos_sin)
@@ -143,7 +144,7 @@ class _CoatOLMoAfterAttentionResidual(torch.autograd.Function):
         group_size = ctx.group_size
         fwobits, layer_id, config, qargs = ctx.utils
         out_g = _as_e5m2_grad(out_g, fwobits)
-        out_gs_max = out_gs.max()
+        out_gs_max = scale_max(out_gs)
         out_g_t = fp8_transpose(out_g, transpose_output_2d=True)
         flash_x_t, flash_s = fp8_division_transpose(flash_x, group_size, fwobits["fabit"], flash_s, stochastic=False,
                                                     only_transposed=True)
@@ -209,7 +210,7 @@ class _CoatOLMoMLPResidual(torch.autograd.Function):
         mean, rstd, num_warps = ctx.ln_utils
         fwobits, layer_id, config, qargs = ctx.utils
         out_g = _as_e5m2_grad(out_g, fwobits)
-        out_gs_max = out_gs.max()
+        out_gs_max = scale_max(out_gs)
         out_g_t = fp8_transpose(out_g, transpose_output_2d=True)
         w2_t = _backward_weight_t(w2_saved, w2_s, qargs, fwobits)
         fc2_g, weight2_grad = fp8_linear_backward(mul_x_t, mul_s, out_g, out_gs_max, out_g_t, w2_t, w2_s, group_size)

@@ -124,3 +124,63 @@ def test_captured_backward_chain_replays_bit_identically(dev):
         torch.cuda.synchronize(dev)
         for k, (got, ref) in enumerate(zip(static_out, want)):
             assert torch.equal(got, ref), f"replay {i}: output {k} differs from the eager run"
+
+
+def test_captured_decoder_layer_step_replays_like_eager(dev):
+    """Forward + backward of a whole CoatLlamaDecoderLayer (FP8 linears, fused activations, norms, bf16 SDPA attention,
+    autograd in between) recorded into one graph and replayed on new inputs: output, input gradient and every weight
+    gradient equal the eager step's bit for bit.  (At this size the attention backward of this torch build is reproducible
+    run to run, which the comparison relies on; the FP8 path of the layer launches no memset: the scale maxima it needs
+    come from the library's kernels, not from torch reductions.)"""
+    from coat_amd.activation.real_quantization import Coat_quantize_bgn, Coat_quantize_end
+    from coat_amd.models.coat_llama import CoatLlamaConfig, CoatLlamaDecoderLayer
+    from coat_amd.utils._fp8manager import FP8Manager
+    torch.manual_seed(0)
+    cfg = CoatLlamaConfig(hidden_size=512, intermediate_size=1536, num_attention_heads=8)
+    layer = CoatLlamaDecoderLayer(cfg, 0)
+    for p in layer.parameters():
+        if p.dim() == 2:
+            torch.nn.init.normal_(p, std=0.02)
+        else:
+            p.data = 1 + 0.1 * torch.randn_like(p)
+    layer = layer.to(dev).to(torch.bfloat16)
+    layer.train()
+    bgn, end = Coat_quantize_bgn(layer.qargs).to(dev), Coat_quantize_end(layer.qargs).to(dev)
+    B, S, H = 2, 128, cfg.hidden_size
+    gen = torch.Generator(device=dev).manual_seed(9)
+    data = [((torch.randn(B, S, H, generator=gen, device=dev) * (1 + i)).bfloat16(),
+             (torch.randn(B, S, H, generator=gen, device=dev) * 1e-2 / (1 + i)).bfloat16()) for i in range(3)]
+    params = [p for _, p in sorted(layer.named_parameters())]
+    FP8Manager.is_first_microbatch = True
+
+    def step(xin, gy):
+        h, qh, sh = bgn(xin)
+        (h, qh, sh), = layer(h, qh, sh)
+        y = end(h, qh, sh)
+        grads = torch.autograd.grad(y, [xin] + params, gy)
+        return [y.detach(), *grads]
+
+    static_x = data[0][0].clone().requires_grad_(True)
+    static_gy = data[0][1].clone()
+    side = torch.cuda.Stream(device=dev)  # default priority
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(static_x, static_gy)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step(static_x, static_gy)
+    torch.cuda.synchronize(dev)
+    for i, (x, gy) in enumerate(data + data[:1]):
+        want = [o.clone() for o in step(x.clone().requires_grad_(True), gy)]  # eager work between the replays
+        torch.cuda.synchronize(dev)
+        with torch.no_grad():
+            static_x.copy_(x)
+            static_gy.copy_(gy)
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        assert len(static_out) == len(want) > 10
+        for k, (got, ref) in enumerate(zip(static_out, want)):
+            assert torch.equal(got, ref), f"replay {i}: tensor {k} differs from the eager step"
