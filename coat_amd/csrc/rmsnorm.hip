@@ -280,7 +280,9 @@ __global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd
                                                       const void* __restrict__ dy3, const void* __restrict__ w,
                                                       const float* __restrict__ rstd_in, void* __restrict__ dx,
                                                       float* __restrict__ dw_partial, int64_t M, int N, int qb) {
-    constexpr bool HOLD_W = WDT != kF32 && !MULTI;  // MULTI spends those registers on gradient loads in flight
+    // MULTI spends those registers on gradient loads in flight; with five chunks they decide between one and two waves per
+    // SIMD (61.3 -> 50.1 us at [8192, 5120]), with eight there is one wave either way and re-reading the weight costs 20 %
+    constexpr bool HOLD_W = WDT != kF32 && !MULTI && CH != 5;
     __shared__ float red[4][64 * 16];
     const int lane = threadIdx.x & 63, wv_id = threadIdx.x >> 6;
     const int64_t nwaves = (int64_t)gridDim.x * 4;
