@@ -452,7 +452,9 @@ static int rms_check(int64_t M, int64_t N, int QB) {
 
 // Rows up to 8192 columns go to the wave-per-row kernels (CH = 4, 5 or 8 chunks of 16 per lane; 5 is the 5120 columns of
 // the 13B shape, which as 5 of 8 chunks ran at 0.6 of the rate of the 4096-column rows), wider rows (up to 16384) to
-// the block-per-row kernels.  KW = fp8 kind * 3 + weight dtype.
+// the block-per-row kernels.  The forward changes over at 5120 columns already: with eight chunks a wave holds 256
+// registers and is alone on its SIMD, and the block-per-row kernel is faster ([8192, 8192]: 22 against 41 us); the
+// backward is faster wave by wave up to 8192 (110 against 136 us).  Both layouts give the same bits.  KW = fp8 kind * 3 + weight dtype.
 #ifndef COAT_RMS_FWD_BLOCKS
 #define COAT_RMS_FWD_BLOCKS 768
 #endif
@@ -480,9 +482,6 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
                                s_dtype, w, y, s_row, rstd, s_max, M, (int)N, QB, eps);                                 \
         else if (N <= 5120)                                                                                            \
             hipLaunchKernelGGL((k_rmsnorm_fwd<K, W, 5>), dim3((unsigned)wave_blocks), dim3(256), 0, st, (const uint8_t*)x, s_x, \
-                               s_dtype, w, y, s_row, rstd, s_max, M, (int)N, QB, eps);                                 \
-        else if (N <= 8192)                                                                                            \
-            hipLaunchKernelGGL((k_rmsnorm_fwd<K, W, 8>), dim3((unsigned)wave_blocks), dim3(256), 0, st, (const uint8_t*)x, s_x, \
                                s_dtype, w, y, s_row, rstd, s_max, M, (int)N, QB, eps);                                 \
         else                                                                                                           \
             hipLaunchKernelGGL((k_rmsnorm_fwd_block<K, W, 4>), dim3((unsigned)M), dim3(256), 0, st, (const uint8_t*)x, s_x, \
