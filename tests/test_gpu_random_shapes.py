@@ -55,3 +55,32 @@ def test_random_shapes_bit_exact(dev, seed):
     d = rq.fp8_dequantize(q, s, QB)
     wd = R.fp8_dequantize(wq, ws, QB)
     assert torch.equal(d.cpu(), wd), what
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_grouped_gemm_equals_separate_launches(dev, seed):
+    """Seeded random problem counts, shapes (ragged tiles, partial K-steps), operand formats and epilogues: every problem
+    of a grouped launch is bit-identical to its own launch."""
+    from coat_amd.activation.real_quantization import linear
+    rnd = random.Random(7000 + seed)
+    count = rnd.choice([2, 3, 4])
+    M = rnd.choice([16, 48, 256, 272, 520, 1040])
+    N = 16 * rnd.randint(1, 70)
+    K = 16 * rnd.randint(1, 40)
+    fa = rnd.choice([torch.float8_e4m3fn, torch.float8_e5m2])
+    fb = rnd.choice([torch.float8_e4m3fn, torch.float8_e5m2])
+    quant = rnd.random() < 0.4
+    g = torch.Generator().manual_seed(seed)
+    a = [torch.randn(M, K, generator=g).to(fa).to(dev) for _ in range(count)]
+    b = [torch.randn(N, K, generator=g).to(fb).to(dev) for _ in range(count)]
+    sa = [torch.tensor(rnd.uniform(1e-3, 1e-1)).bfloat16().to(dev) for _ in range(count)]
+    sb = [torch.tensor(rnd.uniform(1e-3, 1e-1)).bfloat16().to(dev) for _ in range(count)]
+    got = linear.fp8matmul_grouped(a, [x.t() for x in b], quant, sa, sb, 16)
+    what = (seed, count, M, N, K, fa, fb, quant)
+    for i in range(count):
+        want = linear.fp8matmul(a[i], b[i].t(), quant, sa[i], sb[i], 16)
+        if quant:
+            assert torch.equal(got[i][0].view(torch.uint8), want[0].view(torch.uint8)), what
+            assert torch.equal(got[i][1], want[1]), what
+        else:
+            assert torch.equal(got[i], want), what
