@@ -123,32 +123,42 @@ def make_quantize_workload(dev, torch, transpose, shape=(4096, 4096)):
 
 
 def make_gemm_workload(dev, torch, which, grad_format="e5m2"):
-    """The Llama-2-7B MLP up-projection at 8192 tokens, X [8192,4096] x W [11008,4096]; which = fwd | dgrad | wgrad (the three GEMMs of FP8Linear).
-    The gradient operand is e5m2 as the reference's default bobit; grad_format="e4m3" times the all-e4m3 variant."""
+    """The three GEMMs of FP8Linear at BASELINE config 3 on the config's own data: X [8192,4096] ~ N(0, 0.02),
+    W [11008,4096] ~ N(0, 0.02), grad_out [8192,11008] ~ N(0, 1e-2), bf16, each quantized with its per-tensor scale by
+    fp8_quantize_pertensor_transpose (what the module does), and the GEMM gets those codes and scales.
+    which = fwd | dgrad | wgrad.  The gradient is e5m2 as the reference's default bobit; grad_format="e4m3" times the
+    all-e4m3 variant."""
+    from coat_amd.activation.real_quantization._quantize_pertensor_transpose import fp8_quantize_pertensor_transpose
     from coat_amd.activation.real_quantization.linear import fp8matmul
 
-    E4 = torch.float8_e4m3fn
-    E5 = torch.float8_e5m2 if grad_format == "e5m2" else E4
+    gfmt = "E5M2" if grad_format == "e5m2" else "E4M3"
     T, K, N = 8192, 4096, 11008
-    gen = torch.Generator(device="cpu").manual_seed(0)
+    gen = torch.Generator(device=dev).manual_seed(0)
 
-    def rnd(shape, dtype, std):
-        return (torch.randn(shape, generator=gen) * std).to(dtype).to(dev)
+    def quantized(shape, std, fmt):
+        t = (torch.randn(shape, generator=gen, device=dev) * std).bfloat16()
+        return fp8_quantize_pertensor_transpose(t, 16, fmt, transpose_output_2d=True)
 
-    one = torch.tensor(0.01, dtype=torch.bfloat16, device=dev)
+    qx, sx, qxt = quantized((T, K), 0.02, "E4M3")
+    qw, sw, qwt = quantized((N, K), 0.02, "E4M3")
     if which == "fwd":      # Y[T,N] = X[T,K] W[N,K]^T
-        a, b, (M_, N_, K_) = rnd((T, K), E4, 1.0), rnd((N, K), E4, 1.0), (T, N, K)
-    elif which == "dgrad":  # dX[T,K] = G[T,N] Wt[K,N]^T, G is e5m2
-        a, b, (M_, N_, K_) = rnd((T, N), E5, 1.0), rnd((K, N), E4, 1.0), (T, K, N)
-    else:                   # dW[N,K] = Gt[N,T] Xt[K,T]^T
-        a, b, (M_, N_, K_) = rnd((N, T), E5, 1.0), rnd((K, T), E4, 1.0), (N, K, T)
+        a, b, sa, sb, (M_, N_, K_) = qx, qw, sx, sw, (T, N, K)
+    else:
+        qg, sg, qgt = quantized((T, N), 1e-2, gfmt)
+        if which == "dgrad":  # dX[T,K] = G[T,N] Wt[K,N]^T
+            a, b, sa, sb, (M_, N_, K_) = qg, qwt, sg, sw, (T, K, N)
+        else:                 # dW[N,K] = Gt[N,T] Xt[K,T]^T
+            a, b, sa, sb, (M_, N_, K_) = qgt, qxt, sg, sx, (N, K, T)
+    a, b = a.contiguous(), b.contiguous()
+    del qx, qxt, qw, qwt
 
     def step():
-        fp8matmul(a, b.t(), False, one, one, 16)
+        fp8matmul(a, b.t(), False, sa, sb, 16)
 
     flops = 2 * M_ * N_ * K_
     fmt = "e4m3 x e4m3" if which == "fwd" or grad_format == "e4m3" else "e5m2 x e4m3"
-    return step, flops, {"workload": f"fp8matmul {which}: [{M_},{K_}] x [{N_},{K_}]^T -> bf16, {fmt}, per-tensor scales",
+    return step, flops, {"workload": f"fp8matmul {which}: [{M_},{K_}] x [{N_},{K_}]^T -> bf16, {fmt}; operands = "
+                                     f"per-tensor-quantized X, W ~ N(0,0.02), grad_out ~ N(0,1e-2) with their own scales",
                          "M": M_, "N": N_, "K": K_, "kernel": "k_fp8_gemm"}
 
 

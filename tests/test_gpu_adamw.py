@@ -60,19 +60,33 @@ def test_plain_step_bit_exact(dev, n, pdtype):
                                st[k].view(torch.uint8) if st[k].dtype != torch.float32 else st[k]), (k, step)
 
 
+# Smallest fraction of groups whose centre agrees to 1e-5 (tensors of 64 groups or more).  Second moments are sums of
+# positive terms: all of them.  A first moment's group minimum is often what is left of beta1*m + (1-beta1)*g after a
+# cancellation, and carries the 1e-6 of the dequantized m as a 1e-4 of itself: measured 0.85.
+WELL_MIN = {"exp_avg": 0.80, "exp_avg_sq": 0.99}
+# Groups whose minimum comes out of such a cancellation: (scale rtol, code mismatch rate, fraction with another k)
+# (measured on [11008, 4096] slabs over ten steps: scale 2.1e-3 beyond k times the centre's own difference, codes
+# 0 .. 5.4e-5, another exponent on at most 1 of 420 groups)
+ILL_BARS = (1e-2, 2e-4, 1e-2)
+
+
 def compare_expand(pd, std, p, st, n, tag="", p_rtol=2e-6, p_atol=1e-9):
     """Stated tolerances for the expand step (hardware log2/exp2, ~1e-6 relative, against correctly rounded powf).
 
     params: fp32 rtol 2e-6 (atol 1e-9); bf16 within one bf16 ulp.
     The group minimum Mn is often the result of a cancellation beta1*m + (1-beta1)*g ~ 0, so its absolute error
     is ~1e-6 of the group maximum Mx, not of Mn: the centre c = sqrt(Mx*Mn) is therefore bounded through
-    |c^2 - c_ref^2| / c_ref^2 <= 4e-5 * Mx/Mn.  Groups whose c agrees to 1e-5 ("well conditioned", at least 80 %
-    of them) must in addition have: the same exponent k (all but 1e-3 of them), the new scale within rtol 1e-4,
-    codes different on < 1e-3 of their elements and by one code step at most."""
+    |c^2 - c_ref^2| / c_ref^2 <= 4e-5 * Mx/Mn for every group.  Groups whose c agrees to 1e-5 ("well conditioned":
+    every group of a second moment, 85 % of a first moment's; bars WELL_MIN) must have the same exponent k, every one
+    of them; the new scale within 6e-6 beyond what the centre's own difference explains (s = (Mx/c)^k / 448, so k times
+    it; measured 2.1e-6); codes different on at most 5e-5 of their elements (measured 0 .. 2.6e-5; a tensor too small for
+    a rate may have two such elements).  The other groups are held to ILL_BARS.  No code may differ by more than one
+    step.  Every measured value is printed (pytest -rP); all bars are checked before the test fails."""
     if p.dtype == torch.float32:
         assert torch.allclose(pd.cpu(), p, rtol=p_rtol, atol=p_atol), tag + " params"
     else:
         assert torch.allclose(pd.cpu().float(), p.float(), rtol=2.0 ** -7, atol=1e-30), tag + " params (bf16 ulp)"
+    failures = []
     for name in ("exp_avg", "exp_avg_sq"):
         c_g, c_c = std["sqrt_minmax_" + name].cpu().double(), st["sqrt_minmax_" + name].double()
         k_g, k_c = std["expand_" + name].cpu(), st["expand_" + name]
@@ -83,20 +97,38 @@ def compare_expand(pd, std, p, st, n, tag="", p_rtol=2e-6, p_atol=1e-9):
         assert (rel_c2 <= 4e-5 * ratio + 1e-6).all(), (tag, name, "centre", (rel_c2 / ratio).max().item())
         well = ((c_g - c_c).abs() <= 1e-5 * c_c) & finite_k
         ng = k_c.numel()
-        if ng >= 64:
-            assert well.float().mean().item() >= 0.8, (tag, name, well.float().mean().item())
-        same = (k_g == k_c) & well
-        assert (well & ~same).sum().item() <= max(1, int(1e-3 * ng)), (tag, name, "k", (well & ~same).sum().item())
-        assert torch.allclose(s_g[same], s_c[same], rtol=1e-4, atol=0), tag + " scale"
+        well_frac = well.float().mean().item()
+        if ng >= 64 and well_frac < WELL_MIN[name]:
+            failures.append((tag, name, "well", well_frac))
         pad = ng * 128 - n
-        cg = torch.nn.functional.pad(std[name].cpu().view(torch.uint8).flatten(), (0, pad)).reshape(ng, 128)[same]
-        cc = torch.nn.functional.pad(st[name].view(torch.uint8).flatten(), (0, pad)).reshape(ng, 128)[same]
-        neq = cg != cc
-        assert neq.sum().item() <= max(16, int(1e-3 * neq.numel())), (tag, name, "codes", neq.sum().item(), neq.numel())
-        if neq.any():  # one code step: neighbouring magnitudes with the same sign (or +0 / -0 against the smallest code)
-            a, b = cg[neq].int(), cc[neq].int()
-            assert ((a & 0x7F) - (b & 0x7F)).abs().max().item() <= 1, (tag, name, "code step")
-            assert (((a & 0x80) == (b & 0x80)) | (((a & 0x7F) + (b & 0x7F)) <= 1)).all(), (tag, name, "code sign")
+        codes_g = torch.nn.functional.pad(std[name].cpu().view(torch.uint8).flatten(), (0, pad)).reshape(ng, 128)
+        codes_c = torch.nn.functional.pad(st[name].view(torch.uint8).flatten(), (0, pad)).reshape(ng, 128)
+        for cls, groups, s_rtol, code_rate, k_rate in (("well", well, 6e-6, 5e-5, 0.0), ("cancelling", finite_k & ~well, *ILL_BARS)):
+            if not groups.any():
+                continue
+            same = (k_g == k_c) & groups
+            k_bad = (groups & ~same).sum().item()
+            # s = (Mx / c)^k / 448: a centre that differs by d moves the scale by k * d; what is left is the log2 / exp2 error
+            rel_c = (c_g[same] - c_c[same]).abs() / c_c[same]
+            s_rel = (s_g[same] - s_c[same]).abs() / s_c[same].abs()
+            s_err = (s_rel - k_c[same].double() * rel_c).clamp_min(0).max().item() if same.any() else 0.0
+            cg, cc = codes_g[same], codes_c[same]
+            neq = cg != cc
+            rate = neq.sum().item() / max(1, neq.numel())
+            print(f"expand {tag} {name} [{cls}: {groups.sum().item()} of {ng} groups]: k mismatches {k_bad}, "
+                  f"scale err beyond k * centre err {s_err:.2e} (raw {s_rel.max().item() if same.any() else 0.0:.2e}), "
+                  f"codes {neq.sum().item()} / {neq.numel()} = {rate:.2e}")
+            if k_bad > int(k_rate * groups.sum().item() + (1 if k_rate else 0)):
+                failures.append((tag, name, cls, "k", k_bad))
+            if s_err > s_rtol:
+                failures.append((tag, name, cls, "scale", s_err))
+            if neq.sum().item() > max(2, int(code_rate * neq.numel())):
+                failures.append((tag, name, cls, "codes", neq.sum().item(), neq.numel()))
+            if neq.any():  # one code step: neighbouring magnitudes with the same sign (or +0 / -0 against the smallest code)
+                a, b = cg[neq].int(), cc[neq].int()
+                assert ((a & 0x7F) - (b & 0x7F)).abs().max().item() <= 1, (tag, name, cls, "code step")
+                assert (((a & 0x80) == (b & 0x80)) | (((a & 0x7F) + (b & 0x7F)) <= 1)).all(), (tag, name, cls, "code sign")
+    assert not failures, failures
 
 
 @pytest.mark.parametrize("n", [128 * 512, 128 * 9 + 37, 127, 1])

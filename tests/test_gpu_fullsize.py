@@ -287,6 +287,57 @@ def test_rmsnorm_llama_hidden_slabs(dev):
         assert frac <= 6e-3 and ulp <= 2
 
 
+def test_fp8linear_config3_on_its_stated_data(dev):
+    """BASELINE config 3 as it is stated: FP8Linear forward + backward with X [4, 2048, 4096] ~ N(0, 0.02),
+    W [11008, 4096] ~ N(0, 0.02) and grad_out ~ N(0, 1e-2), all bf16, per-tensor quantized by the module itself
+    (reference rq/fp8linear.py:63-110).  Checked: the three per-tensor scales (bit-exact against the scale the
+    tensor's maximum fixes), q and q^T of X, W and dY on 256-row slabs against the oracle's division (bit-exact),
+    the module's saved tensors against those, and the three bf16 outputs on slabs against the float64 product of the
+    decoded operands within the GEMM bound."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    from test_gpu_layer_chain import gemm_close
+    from coat_amd.activation.real_quantization._quantize_pertensor_transpose import fp8_quantize_pertensor_transpose
+    from coat_amd.activation.real_quantization.fp8linear import FP8Linear
+    B, S, K, N = 4, 2048, 4096, 11008
+    x, w, gy = randn(dev, (B, S, K), 31, 0.02), randn(dev, (N, K), 32, 0.02), randn(dev, (B, S, N), 33, 1e-2)
+    layer = FP8Linear(K, N, bias=False, device=dev).to(torch.bfloat16)
+    with torch.no_grad():
+        layer.weight.copy_(w)
+    layer.train()
+    xd = x.clone().requires_grad_(True)
+    y = layer(xd)
+    saved = y.grad_fn.saved
+    y.backward(gy)
+    quant = {}
+    for name, t, fp8, mx in (("x", x.reshape(-1, K), "E4M3", 448.0), ("w", w, "E4M3", 448.0),
+                             ("g", gy.reshape(-1, N), "E5M2", 57344.0)):
+        q, s, qt = fp8_quantize_pertensor_transpose(t, 16, fp8, transpose_output_2d=True)
+        assert s.dtype == torch.bfloat16 and s.cpu().item() == _scale_of_amax(t.abs().max(), mx).item(), name
+        assert torch.equal(qt.view(torch.uint8), q.view(torch.uint8).t()), name + ": q^T is not the byte transpose of q"
+        for r0 in _slabs(t.shape[0]):
+            want, _ = R.fp8_division(t[r0:r0 + SLAB].cpu(), 16, fp8, s.cpu())
+            assert torch.equal(_b(q[r0:r0 + SLAB]).cpu(), _b(want)), (name, r0)
+        quant[name] = (q, s, qt)
+    # what the module quantized and saved is what the same calls return
+    u8 = torch.uint8
+    assert torch.equal(saved[0].view(u8), quant["x"][2].view(u8)) and torch.equal(saved[1], quant["x"][1])
+    assert torch.equal(saved[2].view(u8), quant["w"][2].view(u8)) and torch.equal(saved[3], quant["w"][1])
+    (qx, sx, qxt), (qw, sw, qwt), (qg, sg, qgt) = quant["x"], quant["w"], quant["g"]
+    y2, dx2, dw = y.detach().reshape(-1, N), xd.grad.reshape(-1, K), layer.weight.grad
+    for r0 in _slabs(B * S):
+        gemm_close(y2[r0:r0 + SLAB], qx[r0:r0 + SLAB], qw, sx, sw, f"config 3 forward rows {r0}")
+        gemm_close(dx2[r0:r0 + SLAB], qg[r0:r0 + SLAB], qwt, sg, sw, f"config 3 dgrad rows {r0}")
+    for r0 in _slabs(N):  # rows of the weight gradient = columns of the output gradient
+        gemm_close(dw[r0:r0 + SLAB], qgt[r0:r0 + SLAB], qxt, sg, sx, f"config 3 wgrad rows {r0}")
+    # the FP8 flow against the same linear in bf16: quantization noise only
+    ref = torch.nn.functional.linear(x, w)
+    rel = ((y.detach().float() - ref.float()).norm() / ref.float().norm()).item()
+    print(f"[measured] config 3 forward against bf16 F.linear: relative Frobenius {rel:.4f} (bar 0.06)")
+    assert rel < 0.06
+
+
 def test_adamw_ten_steps_llama_weight_slab(dev):
     """BASELINE config 2: ten CoatAdamW expand steps on fp32 [11008, 4096], lr 3e-4, betas (0.9, 0.95), wd 0.1, eps 1e-8.
     The GPU steps the whole tensor from the fresh state; before every step the first 4096 groups of its state are copied
