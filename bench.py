@@ -26,6 +26,44 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+PROBE_SRC = os.path.join(ROOT, "bench_probe.hip")
+PROBE_LIB = os.path.join(ROOT, "libcoat_bench_probe.so")
+_probe_lib = None
+
+
+def build_probe(verbose=True):
+    """Compiles bench_probe.hip (the copy / read / fill probe and the clock-probe instances of the GEMM kernel) into
+    libcoat_bench_probe.so beside this file.  Measurement code only: nothing of it is part of libcoat_hip.so."""
+    import subprocess
+
+    from coat_amd import build as hip_build
+
+    cmd = [hip_build.HIPCC, *hip_build.FLAGS, "-shared", "-I", ROOT, PROBE_SRC, "-o", PROBE_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on bench_probe.hip:\n" + r.stdout + r.stderr)
+    if verbose:
+        print(f"[bench] built {PROBE_LIB}")
+    return PROBE_LIB
+
+
+def probe_lib():
+    """The measurement library: loaded if it has been built (python -c 'import bench; bench.build_probe()' or
+    __graft_entry__.build()), built first otherwise."""
+    global _probe_lib
+    if _probe_lib is None:
+        import ctypes
+
+        if not os.path.exists(PROBE_LIB):
+            build_probe()
+        L = ctypes.CDLL(PROBE_LIB)
+        vp, i64 = ctypes.c_void_p, ctypes.c_int64
+        L.bench_hbm_probe.argtypes = [ctypes.c_int, vp, vp, i64, vp]
+        L.bench_gemm_clock.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, vp, vp]
+        L.bench_hbm_probe.restype = L.bench_gemm_clock.restype = ctypes.c_int
+        _probe_lib = L
+    return _probe_lib
+
 
 def adamw_bytes(numel):
     ngroups = (numel + 127) // 128
@@ -374,19 +412,20 @@ def make_layernorm_workload(dev, torch):
 
 
 def make_hbm_probe_workload(dev, torch, kind):
-    """What this box's HBM delivers to the simplest kernels on 1 GiB (coat_hbm_probe: one 16-byte access per lane,
+    """What this box's HBM delivers to the simplest kernels on 1 GiB (bench_hbm_probe of bench_probe.hip: one 16-byte access per lane,
     streaming loads): "copy" (1 GiB read + 1 GiB written), "read", "fill".  These are the practical ceilings the
     streaming kernels are compared with next to the nominal 8 TB/s."""
     from coat_amd import _hip
+    L = probe_lib()
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
     dst = torch.empty_like(src) if kind != "read" else torch.zeros(16, dtype=torch.uint8, device=dev)
     code = {"copy": 0, "read": 1, "fill": 2}[kind]
 
     def step():
-        _hip.check(_hip.lib().coat_hbm_probe(code, _hip.ptr(src), _hip.ptr(dst), n, _hip.stream(dev)), "hbm_probe")
+        _hip.check(L.bench_hbm_probe(code, _hip.ptr(src), _hip.ptr(dst), n, _hip.stream(dev)), "hbm_probe")
 
-    return step, (2 * n if kind == "copy" else n), {"workload": f"hbm_probe {kind}: coat_hbm_probe on 1 GiB",
+    return step, (2 * n if kind == "copy" else n), {"workload": f"hbm_probe {kind}: bench_hbm_probe on 1 GiB",
                                                       "kernel": "k_hbm_probe"}
 
 
@@ -682,31 +721,37 @@ def ramp_clocks(step, seconds, torch):
 
 
 def gemm_clock(dev, torch):
-    """The shader clock the FP8 GEMM really runs at.  Needs a probe build of the library:
-        COAT_HIPCC_FLAGS=-DCOAT_GEMM_PROBE COAT_LIB_OUT=/tmp/libcoat_probe.so python -m coat_amd.build
-        COAT_HIP_LIB=/tmp/libcoat_probe.so python bench.py --workload gemm_clock
-    Every block of k_fp8_gemm records its duration in shader clocks (s_memtime) and in ticks of the constant 100 MHz
-    counter (s_memrealtime); their ratio is the clock.  Operands N(0, 1) as in the gemm_* workloads, and all zeros."""
-    import ctypes
-
+    """The shader clock the FP8 GEMM really runs at.  bench_probe.hip instantiates the library's GEMM kernel with its
+    PROBE switch: every block records its duration in shader clocks (s_memtime) and in ticks of the constant 100 MHz
+    counter (s_memrealtime); their ratio is the clock.  Operands: the per-tensor-quantized config-3 tensors of the gemm_*
+    workloads, and all zeros."""
     from coat_amd import _hip
-    from coat_amd.activation.real_quantization.linear import fp8matmul
-    L = _hip.lib()
-    if not hasattr(L, "coat_gemm_set_probe"):
-        print("bench.py: --workload gemm_clock needs a library built with -DCOAT_GEMM_PROBE (see the docstring)", file=sys.stderr)
-        sys.exit(4)
+    from coat_amd.activation.real_quantization._quantize_pertensor_transpose import fp8_quantize_pertensor_transpose
+
+    L = probe_lib()
     probe = torch.zeros(2 * 256, dtype=torch.int64, device=dev)
-    L.coat_gemm_set_probe.argtypes = [ctypes.c_void_p]
-    L.coat_gemm_set_probe.restype = None
-    L.coat_gemm_set_probe(ctypes.c_void_p(probe.data_ptr()))
-    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
-    one = torch.tensor(0.01, dtype=torch.bfloat16, device=dev)
+    T, K, N = 8192, 4096, 11008
+    gen = torch.Generator(device=dev).manual_seed(0)
+
+    def quantized(shape, std, fmt):
+        t = (torch.randn(shape, generator=gen, device=dev) * std).bfloat16()
+        return fp8_quantize_pertensor_transpose(t, 16, fmt, transpose_output_2d=True)
+
+    qx, sx, qxt = quantized((T, K), 0.02, "E4M3")
+    qw, sw, qwt = quantized((N, K), 0.02, "E4M3")
+    qg, sg, qgt = quantized((T, N), 1e-2, "E5M2")
+    cases = (("fwd", qx, qw, sx, sw), ("dgrad", qg, qwt, sg, sw), ("wgrad", qgt, qxt, sg, sx),
+             ("dgrad_zero_operands", torch.zeros_like(qg), torch.zeros_like(qwt), sg, sw))
     out = {}
-    for name, (M, N, K), fa, zero in (("fwd", (8192, 11008, 4096), E4, False), ("dgrad", (8192, 4096, 11008), E5, False),
-                                      ("wgrad", (11008, 4096, 8192), E5, False), ("dgrad_zero_operands", (8192, 4096, 11008), E5, True)):
-        a = (torch.zeros if zero else torch.randn)(M, K, device=dev).to(fa)
-        b = (torch.zeros if zero else torch.randn)(N, K, device=dev).to(E4)
-        step = lambda: fp8matmul(a, b.t(), False, one, one, 16)  # noqa: E731
+    for name, a, b, sa, sb in cases:
+        a, b = a.contiguous(), b.contiguous()
+        (M, Kd), Nd = a.shape, b.shape[0]
+        c = torch.empty((M, Nd), dtype=torch.bfloat16, device=dev)
+
+        def step():
+            _hip.check(L.bench_gemm_clock(_hip.ptr(a), _hip.fp8(a.dtype), _hip.ptr(b), _hip.ptr(c), _hip.ptr(sa), _hip.ptr(sb),
+                                          M, Nd, Kd, _hip.ptr(probe), _hip.stream(dev)), "bench_gemm_clock")
+
         ramp_clocks(step, 2.0, torch)
         ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
         ev[0].record()
@@ -716,15 +761,16 @@ def gemm_clock(dev, torch):
         torch.cuda.synchronize()
         ms = ev[0].elapsed_time(ev[1]) / 50
         p = probe.cpu().view(-1, 2).double()
-        tiles = ((M + 255) // 256) * ((N + 255) // 256)
-        ideal = tiles * ((K + 127) // 128) * 2048 / 256  # MFMA clocks per CU if the matrix pipes never waited
+        tiles = ((M + 255) // 256) * ((Nd + 255) // 256)
+        ideal = tiles * ((Kd + 127) // 128) * 2048 / 256  # MFMA clocks per CU if the matrix pipes never waited
         mhz = p[:, 0] / p[:, 1] * 100.0
-        out[name] = {"us_per_launch": round(ms * 1e3, 1), "tflops": round(2 * M * N * K / ms / 1e9, 0),
+        out[name] = {"us_per_launch": round(ms * 1e3, 1), "tflops": round(2 * M * Nd * Kd / ms / 1e9, 0),
                      "shader_clock_mhz_mean": round(mhz.mean().item()), "shader_clock_mhz_min": round(mhz.min().item()),
                      "shader_clock_mhz_max": round(mhz.max().item()), "block_shader_clocks_mean": round(p[:, 0].mean().item()),
                      "mfma_clocks_ideal_per_cu": round(ideal), "mfma_busy_of_block_clocks": round(ideal / p[:, 0].mean().item(), 4),
                      "peak_at_this_clock_tflops": round(256 * 8192 * mhz.mean().item() / 1e6, 0)}
-    print(json.dumps({"workload": "gemm_clock", "gemm": out}))
+    print(json.dumps({"workload": "gemm_clock", "operands": "per-tensor-quantized X, W ~ N(0,0.02), grad_out ~ N(0,1e-2) (config 3)",
+                      "gemm": out}))
 
 
 METRIC = "quantize+AdamW GB/s (% HBM peak); FP8 GEMM TFLOPS; 7B-layer fwd+bwd ms"

@@ -9,12 +9,13 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# COAT_HIP_LIB: another build of the same library (an experiment or probe build made with COAT_LIB_OUT=... python -m coat_amd.build)
+# COAT_HIP_LIB: another build of the same library (an experiment build made with COAT_LIB_OUT=... python -m coat_amd.build)
 LIB_PATH = os.environ.get("COAT_HIP_LIB") or os.path.join(_HERE, "libcoat_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
 MAX_SLOTS, MAX_SLOT_STRIDE = 16, 32  # COAT_MAX_SLOTS, COAT_MAX_SLOT_STRIDE of include/coat_hip.h
 MAX_WORDS = MAX_SLOTS * MAX_SLOT_STRIDE
+ABI_VERSION = 3  # COAT_ABI_VERSION of include/coat_hip.h: a library built from another header is refused
 E4M3, E5M2 = 0, 1
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
@@ -34,7 +35,6 @@ SIGNATURES = {
     "coat_fp8_layernorm_division": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_silu_mul_forward_bf16": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_product_division": [_vp, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i64, _i64, _vp],
-    "coat_hbm_probe": [_i, _vp, _vp, _i64, _vp],
     "coat_fp8_division_from_max": [_vp, _i, _vp, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_division_stochastic": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _u64, _vp],
     "coat_fp8_transpose": [_vp, _vp, _i64, _i64, _vp],
@@ -60,6 +60,7 @@ SIGNATURES = {
                                    _i64, _i64, _vp],
     "coat_rope_bf16": [_vp, _vp, _vp, _vp, _i64, _f, _vp, _i64, _i, _i, _i, _i, _i64, _i64, _vp],
     "coat_fp8_gemm": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _i, _vp],
+    "coat_fp8_gemm_residual": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _vp],
     "coat_fp8_gemm_grouped": [_i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _i, _vp],
     "coat_fp8_adamw_expand_step": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _i,
                                    _i64, _i64, _vp],
@@ -82,6 +83,10 @@ def lib():
             fn = getattr(L, name)
             fn.argtypes = argtypes
             fn.restype = _i
+        L.coat_abi_version.restype = _i
+        if L.coat_abi_version() != ABI_VERSION:
+            raise RuntimeError(f"coat_amd: {LIB_PATH} has ABI version {L.coat_abi_version()}, this package needs "
+                               f"{ABI_VERSION}; rebuild it with `python -m coat_amd.build`")
         L.coat_version.restype = ctypes.c_char_p
         L.coat_status_string.argtypes = [_i]
         L.coat_status_string.restype = ctypes.c_char_p

@@ -61,6 +61,63 @@ def fp8matmul(a, b, output_quantize, scale_a, scale_b, QB, bias=None, stochastic
     return (c, scale_c) if output_quantize else c
 
 
+def fp8matmul_add(a, b, residual, scale_a, scale_b, fp8type=None, QB=16, bias=None):
+    """``fp8matmul(a, b, False, ...)`` followed by the addition of the bf16 tensor ``residual``, in one kernel:
+    returns ``y = bf16(float(product) + float(residual))`` and, with ``fp8type``, ``(y, (q, s))`` where q / s are the
+    1 x 16 per-group FP8 codes and bf16 scales of the fp32 sum: what ``fp8_add_Ifp_Ifp_Ofp_Og16(residual, product, fp8type,
+    16)`` returns (reference add_fwd.py:162-213 after linear.py:172-250), bit for bit.  Falls back to the two kernels for
+    shapes the fused epilogue does not take."""
+    from .add_fwd import fp8_add_Ifp_Ifp_Ofp_Og16
+    from .common import as_fp8_dtype
+    lead = a.shape[:-1]
+    a2 = a.reshape(-1, a.shape[-1])
+    r2 = residual.reshape(-1, residual.shape[-1])
+    N = b.shape[1]
+    fused = (residual.dtype == torch.bfloat16 and N % 8 == 0 and (fp8type is None or (QB == 16 and N % 16 == 0))
+             and tuple(r2.shape) == (a2.shape[0], N))
+    if not fused:
+        prod = fp8matmul(a2, b, False, scale_a, scale_b, QB, bias)
+        if fp8type is None:
+            return (prod + r2).reshape(*lead, N)
+        y, (q, sq) = fp8_add_Ifp_Ifp_Ofp_Og16(r2, prod, fp8type, QB)
+        return y.reshape(*lead, N), (q.reshape(*lead, N), sq.reshape(*lead, N // QB))
+    assert a2.shape[1] == b.shape[0], "Incompatible dimensions"
+    a2, r2 = _hip.dense(a2), _hip.dense(r2)
+    bn = _hip.dense(_k_contiguous_rows(b))
+    M, K = a2.shape
+    for t in (scale_a, scale_b):
+        if t.numel() != 1:
+            raise ValueError("fp8matmul takes per-tensor (single element) scales")
+    scale_a = scale_a if scale_a.is_cuda else scale_a.to(a2.device)
+    scale_b = scale_b if scale_b.is_cuda else scale_b.to(a2.device)
+    if bias is not None:
+        bias = _hip.dense(bias)
+    y = torch.empty((M, N), device=a2.device, dtype=torch.bfloat16)
+    q = sq = None
+    kind = 0
+    if fp8type is not None:
+        fp8type = as_fp8_dtype(fp8type)
+        q = torch.empty((M, N), device=a2.device, dtype=fp8type)
+        sq = torch.empty((M, N // 16), device=a2.device, dtype=torch.bfloat16)
+        kind = _OUT_KIND[fp8type]
+    _hip.check(_hip.lib().coat_fp8_gemm_residual(
+        _hip.ptr(a2), _hip.fp8(a2.dtype), _hip.ptr(bn), _hip.fp8(bn.dtype), _hip.ptr(r2), _hip.ptr(y), _hip.ptr(q), _hip.ptr(sq),
+        kind, _hip.ptr(scale_a), _hip.dt(scale_a), _hip.ptr(scale_b), _hip.dt(scale_b), _hip.ptr(bias),
+        _hip.dt(bias) if bias is not None else 0, M, N, K, _hip.stream(a2.device)), "fp8matmul_add")
+    y = y.reshape(*lead, N)
+    if fp8type is None:
+        return y
+    return y, (q.reshape(*lead, N), sq.reshape(*lead, N // 16))
+
+
+def fp8_linear_forward_add(x, s, w, s_w, residual, fp8type, QB, bias=None):
+    """``fp8_add_Ifp_Ifp_Ofp_Og16(residual, fp8_linear_forward(x, s, w, s_w, False, QB, bias), fp8type, QB)`` in one
+    kernel: the projection that closes a residual branch (reference coat_llama.py:440-441, :673-674)."""
+    assert s.numel() == 1, f"X uses per-tensor quantization in linear forward, but the scale shape is {s.shape}"
+    assert s_w.numel() == 1, f"W uses per-tensor quantization in linear forward, but the scale shape is {s_w.shape}"
+    return fp8matmul_add(x, w.t(), residual, s, s_w, fp8type, QB, bias)
+
+
 _MAX_GROUP = 4  # problems per grouped launch (kMaxGroup of the kernel)
 
 

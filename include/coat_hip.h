@@ -45,11 +45,14 @@ enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.f
 #define COAT_MAX_SLOT_STRIDE 32
 #define COAT_MAX_WORDS (COAT_MAX_SLOTS * COAT_MAX_SLOT_STRIDE)
 
+/* Bumped whenever an entry point's argument list or the size of a buffer it writes changes (2: every s_max / amax
+ * argument became COAT_MAX_WORDS words; 3: coat_fp8_gemm_residual and coat_fp8_rmsnorm_backward_add added,
+ * coat_hbm_probe removed).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
+ * loads the library. */
+#define COAT_ABI_VERSION 3
+int coat_abi_version(void);
 const char* coat_version(void);
 const char* coat_status_string(int status);
-/* Memory-bandwidth probe for the benchmarks (no counterpart in the reference): kind 0 copies bytes from src to dst,
- * 1 reads src (dst: 4 writable bytes), 2 fills dst; one 16-byte access per lane, bytes % 16 == 0. */
-int coat_hbm_probe(int kind, const void* src, void* dst, int64_t bytes, void* stream);
 
 /* ---- quantize family -------------------------------------------------------------------------- */
 
@@ -255,6 +258,17 @@ int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* si
 int coat_fp8_gemm(const void* a, int fmt_a, const void* b, int fmt_b, void* c, void* c_scale, int out_kind,
                   const void* scale_a, int sa_dtype, const void* scale_b, int sb_dtype, const void* bias, int bias_dtype,
                   int64_t M, int64_t N, int64_t K, int QB, void* stream);
+
+/* The same product followed by the addition of a bf16 tensor, as one kernel (no counterpart function in the reference,
+ * which runs fp8matmul, rq/linear.py:172, and then a tensor addition: rq/add_fwd.py:162 fp8_add_Ifp_Ifp_Ofp_Og16 after the
+ * output and down projections, coat/models/coat_llama.py:440-441, :673-674; plain bf16 `+` for the gradients that reach one
+ * tensor, :328, :742).  t = bf16 of the product as coat_fp8_gemm stores it; v = float(t) + float(residual) in fp32;
+ * c = bf16(v).  out_kind 1 / 2: also c_q = e4m3 / e5m2 codes of v per 1 x 16 group with scale (amax + 1e-10) / fp8max and
+ * c_scale = the bf16 scales [M, N/16] (add_fwd.py:107-137), bit-identical to running the two kernels.  residual bf16 [M,N]
+ * may be c itself (accumulation in place).  N % 8 == 0 (N % 16 == 0 with out_kind 1 / 2), N < 2^22. */
+int coat_fp8_gemm_residual(const void* a, int fmt_a, const void* b, int fmt_b, const void* residual, void* c, void* c_q,
+                           void* c_scale, int out_kind, const void* scale_a, int sa_dtype, const void* scale_b,
+                           int sb_dtype, const void* bias, int bias_dtype, int64_t M, int64_t N, int64_t K, void* stream);
 
 /* `count` (1 .. 4) such products of one shape and one pair of formats in one launch: problem i is
  * (a[i], b[i], c[i], c_scale[i], scale_a[i], scale_b[i], bias[i]); the seven arrays are host arrays of `count` device

@@ -219,6 +219,50 @@ def test_grouped_gemm_equals_separate_launches(dev, count, M, N, K, fa, fb, quan
         check_bf16(got[0], a[0].cpu(), b[0].cpu(), sa[0].cpu(), sb[0].cpu())
 
 
+@pytest.mark.parametrize("M,N,K,fa,fb,out,with_bias", [
+    (512, 512, 256, E4, E4, "E4M3", False),     # whole tiles, packed scale stores
+    (300, 272, 144, E4, E4, "E4M3", True),      # ragged tile rows / columns, partial last K-step, scales stored one by one
+    (1100, 1040, 272, E5, E4, "E5M2", False),   # more tiles than one round of a small grid, e5m2 operand and e5m2 codes
+    (512, 520, 128, E4, E5, None, False),       # bf16 sum only, rows of N % 16 == 8
+    (4352, 2064, 400, E5, E4, None, True),      # more tiles than CUs (the ring runs across tile boundaries)
+    (2304, 2048, 128, E4, E4, "E4M3", False),   # 72 whole tiles
+])
+def test_gemm_with_residual_equals_gemm_then_add(dev, M, N, K, fa, fb, out, with_bias):
+    """coat_fp8_gemm_residual against the two kernels it replaces: the bf16 product of coat_fp8_gemm, then the residual
+    addition (fp8_add_Ifp_Ifp_Ofp_Og16, or torch's bf16 addition when no FP8 copy is asked for).  Bit-identical sums,
+    codes and scales; also with the residual tensor as the output (accumulation in place)."""
+    from coat_amd.activation.real_quantization.add_fwd import fp8_add_Ifp_Ifp_Ofp_Og16
+    lin = _lin()
+    a, b = rand_fp8((M, K), 61, fa).to(dev), rand_fp8((N, K), 62, fb).to(dev)
+    sa, sb = torch.tensor(0.021).bfloat16().to(dev), torch.tensor(0.0127).float().to(dev)
+    res = (torch.randn(M, N, generator=torch.Generator().manual_seed(63)) * 1.5).bfloat16().to(dev)
+    res[::7, ::5] *= 40
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(64)).bfloat16().to(dev) if with_bias else None
+    prod = lin.fp8matmul(a, b.t(), False, sa, sb, 16, bias)
+    if out is None:
+        want = prod + res
+        got = lin.fp8matmul_add(a, b.t(), res, sa, sb, None, 16, bias)
+        assert got.dtype == torch.bfloat16 and torch.equal(got, want)
+        # in place through the C ABI: the residual is the output
+        from coat_amd import _hip
+        acc = res.clone()
+        _hip.check(_hip.lib().coat_fp8_gemm_residual(
+            _hip.ptr(a), _hip.fp8(fa), _hip.ptr(b), _hip.fp8(fb), _hip.ptr(acc), _hip.ptr(acc), None, None, 0, _hip.ptr(sa),
+            _hip.dt(sa), _hip.ptr(sb), _hip.dt(sb), _hip.ptr(bias), _hip.dt(bias) if with_bias else 0, M, N, K,
+            _hip.stream(dev)), "gemm_residual in place")
+        assert torch.equal(acc, want)
+        return
+    want_y, (want_q, want_s) = fp8_add_Ifp_Ifp_Ofp_Og16(res, prod, out, 16)
+    got_y, (got_q, got_s) = lin.fp8matmul_add(a, b.t(), res, sa, sb, out, 16, bias)
+    assert torch.equal(got_y, want_y), "bf16 sum"
+    assert got_q.dtype == want_q.dtype and torch.equal(got_q.view(torch.uint8), want_q.view(torch.uint8)), "codes of the sum"
+    assert torch.equal(got_s.view(torch.int16), want_s.view(torch.int16)), "group scales of the sum"
+    # and the oracle on the same product (the addition itself is bit-exact against the CPU restatement)
+    oy, (oq, os_) = R.fp8_add_Ifp_Ifp_Ofp_Og16(res.cpu(), prod.cpu(), out, 16)
+    assert torch.equal(got_y.cpu(), oy) and torch.equal(got_q.cpu().view(torch.uint8), oq.view(torch.uint8))
+    assert torch.equal(got_s.cpu(), os_)
+
+
 def test_grouped_linear_wrappers_equal_the_separate_calls(dev):
     """fp8_linear_forward_grouped / fp8_linear_backward_grouped against the per-projection functions, with a bias vector in
     one problem of the C call (bias is per problem) and with projections of different widths (falls back to separate calls)."""

@@ -23,6 +23,8 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(L, name), f"{name} declared in include/coat_hip.h but not exported"
     assert set(_hip.SIGNATURES) <= declared
     assert b"gfx950" in L.coat_version()
+    abi = int(re.search(r"#define\s+COAT_ABI_VERSION\s+(\d+)", open(os.path.join(ROOT, "include", "coat_hip.h")).read()).group(1))
+    assert L.coat_abi_version() == abi == _hip.ABI_VERSION and str(abi).encode() in L.coat_version()
     assert b"128 per-group" in L.coat_status_string(-4)
 
 
@@ -121,14 +123,12 @@ def test_argument_validation_of_the_remaining_entry_points_without_gpu():
     assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, pa, pn, 1, pa, 1, pa, 1, None, 0, 64, 64, 64, 16, None) == ESHAPE     # second scale output missing
     assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 24, 16, None) == ESHAPE   # K % 16
     assert L.coat_fp8_gemm_grouped(3, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 0, 64, 16, None) == 0         # empty
-    # RoPE, cross-entropy, probe
+    # RoPE, cross-entropy
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 24, 0, 0, 0, None) == ESHAPE                      # head_dim % 16
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 48, 0, None) == ESHAPE                     # pitch < heads * head_dim
     assert L.coat_cross_entropy_forward(p, 0, 8, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # stride < columns
     assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # mean without a count
     assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, p, 4, 16, -100, 0.0, 0.0, 7, 0.0, 0, None) == EINVAL
-    assert L.coat_hbm_probe(0, p, p, 40, None) == EINVAL                                                   # bytes % 16
-    assert L.coat_hbm_probe(3, p, p, 64, None) == EINVAL
 
 
 def test_quantization_config_defaults():
