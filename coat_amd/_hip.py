@@ -51,6 +51,8 @@ SIGNATURES = {
     "coat_fp8_add_bwd": [_vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
     "coat_fp8_rmsnorm_forward": [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i64, _i64, _i, _f, _vp],
     "coat_fp8_rmsnorm_backward": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _vp],
+    "coat_fp8_rmsnorm_backward_add": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i64, _i64,
+                                      _i, _vp],
     "coat_fp8_rmsnorm_backward_static": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp],
     "coat_fp8_layernorm_forward": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _f, _vp],
     "coat_fp8_layernorm_backward": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i,

@@ -13,13 +13,13 @@ from .func_layernorm_noparam import fp8_layernorm_noparam_backward, fp8_layernor
 from .func_layernorm_param import fp8_layernorm_param_backward, fp8_layernorm_param_forward
 from .silu_mul import (fp8_silu_mul_backward, fp8_silu_mul_backward_joined, fp8_silu_mul_forward,
                        fp8_silu_mul_forward_from_bf16)
-from .func_rmsnorm import fp8_rmsnorm_backward, fp8_rmsnorm_forward
+from .func_rmsnorm import fp8_rmsnorm_backward, fp8_rmsnorm_backward_add, fp8_rmsnorm_forward
 from .gelu_bwd import fp8_gelu_backward
 from .gelu_fwd import fp8_gelu_forward
 from .mul_bwd import fp8_mul_backward
 from .mul_fwd import fp8_mul_forward
 from .silu_bwd import fp8_silu_backward
 from .silu_fwd import fp8_silu_forward
-from .linear import (fp8_linear_backward, fp8_linear_backward_grouped, fp8_linear_forward, fp8_linear_forward_grouped,
-                     fp8matmul_grouped)
+from .linear import (fp8_linear_backward, fp8_linear_backward_grouped, fp8_linear_forward, fp8_linear_forward_add,
+                     fp8_linear_forward_grouped, fp8matmul_add, fp8matmul_grouped)
 from .func_quantize import Coat_quantize_bgn, Coat_quantize_end

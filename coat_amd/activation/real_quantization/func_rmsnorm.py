@@ -41,6 +41,26 @@ def fp8_rmsnorm_backward(x, s_x, g, w, v, QB, num_warps):
     ``g`` may also be a tuple of two or three bf16 gradients of the normalised tensor: the kernel then uses
     ``g[0] + g[1] (+ g[2])`` with the roundings of that chain of bf16 additions (what the reference's modules compute
     before the call, coat/models/coat_llama.py:328 and :742), without the separate passes over the tensors."""
+    return _rmsnorm_backward(x, s_x, g, w, v, QB, None, None, False)
+
+
+def fp8_rmsnorm_backward_add(x, s_x, g, w, v, QB, num_warps, residual_grad, fp8type, stochastic=False):
+    """``fp8_rmsnorm_backward`` followed by ``fp8_add_Ifp_Ifp_Ofp_Opt(residual_grad, dx, QB, fp8type)`` with the
+    addition inside the backward kernel (the reference runs them one after the other, coat/models/coat_llama.py:331-339 and
+    :745-754): dx is rounded to bf16 as it would be stored and added to the bf16 ``residual_grad`` in fp32.
+    Returns ``(y, (q, s_max, s_pg), dw)``: the bf16 sum, its per-tensor FP8 codes with their scale, the per-group scales
+    of the sum, and the weight gradient; all bit-identical to the two calls."""
+    from .add_bwd import fp8_add_Ifp_Ifp_Ofp_Opt
+    from .common import as_fp8_dtype
+    N = x.shape[-1]
+    if N > 8192 or residual_grad.dtype != torch.bfloat16:  # rows the wave-per-row kernels do not take: the two kernels
+        dx, dw = _rmsnorm_backward(x, s_x, g, w, v, QB, None, None, False)
+        y, quant = fp8_add_Ifp_Ifp_Ofp_Opt(residual_grad, dx, QB, fp8type, stochastic=stochastic)
+        return y, quant, dw
+    return _rmsnorm_backward(x, s_x, g, w, v, QB, residual_grad, as_fp8_dtype(fp8type), stochastic)
+
+
+def _rmsnorm_backward(x, s_x, g, w, v, QB, residual_grad, fp8type, stochastic):
     x, s_x, batch = prep_pg(x, s_x)
     extra = [None, None]
     if isinstance(g, (tuple, list)):
@@ -61,8 +81,20 @@ def fp8_rmsnorm_backward(x, s_x, g, w, v, QB, num_warps):
     dw = torch.empty((N,), dtype=w.dtype, device=w.device)
     nparts = min(_DW_PARTIALS, M)
     partial = torch.empty((nparts, N), dtype=torch.float32, device=w.device)
-    _hip.check(_hip.lib().coat_fp8_rmsnorm_backward(
+    if residual_grad is None:
+        _hip.check(_hip.lib().coat_fp8_rmsnorm_backward(
+            _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(g), _hip.ptr(extra[0]), _hip.ptr(extra[1]),
+            _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd),
+            _hip.ptr(dx), _hip.ptr(dw), _hip.ptr(partial), nparts, M, N, QB, _hip.stream(x.device)), "fp8_rmsnorm_backward")
+        return restore(dx, batch), dw
+    r = prep_bf16(residual_grad)
+    if r.shape != g.shape:
+        raise ValueError("the residual gradient must have the gradient's shape")
+    s_pg = torch.empty((M, N // QB), dtype=torch.bfloat16, device=x.device)
+    s_max = new_max(x.device)
+    _hip.check(_hip.lib().coat_fp8_rmsnorm_backward_add(
         _hip.ptr(x), _hip.fp8(x.dtype), _hip.ptr(s_x), _hip.dt(s_x), _hip.ptr(g), _hip.ptr(extra[0]), _hip.ptr(extra[1]),
-        _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd),
-        _hip.ptr(dx), _hip.ptr(dw), _hip.ptr(partial), nparts, M, N, QB, _hip.stream(x.device)), "fp8_rmsnorm_backward")
-    return restore(dx, batch), dw
+        _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd), _hip.ptr(r), _hip.ptr(dx), _hip.ptr(s_pg), _hip.ptr(s_max), _hip.fp8(fp8type),
+        _hip.ptr(dw), _hip.ptr(partial), nparts, M, N, QB, _hip.stream(x.device)), "fp8_rmsnorm_backward_add")
+    q, s_q, _ = _division(dx, fp8type, s_max, True, False, "fp8_rmsnorm_backward_add", stochastic, max_as=torch.bfloat16)
+    return restore(dx, batch), (restore(q, batch), s_q, restore(s_pg, batch)), dw

@@ -19,6 +19,7 @@
 // The MFMA takes the B tile as its first operand, so a lane ends up holding 4 consecutive n for one m per accumulator
 // quad: bf16 rows are packed 4 at a time, and a 1 x 16 quantization group is two quads in each of the lanes l, l^32.
 #pragma once
+#include <type_traits>
 #include "coat_device.h"
 #include "coat_host.h"
 
@@ -377,22 +378,28 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
         constexpr int KIND = EPI == kEpiResQuantE5M2 ? kE5M2 : kE4M3;
         const uint8_t* const r_tile = (const uint8_t*)G.res + ((int64_t)m0 * G.N + n0) * 2;
         uint8_t* const cq_tile = (uint8_t*)G.Cq + ((int64_t)m0 * G.N + n0);
-        uint4 rres[2][TJ][2];  // the residual runs of accumulator row-block i (slot i & 1); the next block's are in flight
+        // FULL (wave-uniform): the wave's 128 x 64 lie inside the matrix and there is no bias, so no load, store or
+        // addition is conditional; edge tiles take the guarded instance of the same code.
+        auto residual_epilogue = [&](auto full_c) {
+        constexpr bool FULL = decltype(full_c)::value;
+        constexpr int RD = 2;
+        uint4 rres[RD][TJ][2];  // the residual runs of accumulator row-block i (slot i % RD); the next blocks' are in flight
         auto load_res = [&](int i) {
 #pragma unroll
             for (int j = 0; j < TJ; j++)
 #pragma unroll
                 for (int qp = 0; qp < 2; qp++) {
                     // unconditional load (a load under a branch is waited for on the spot); lanes outside read the tile's origin
-                    const bool in = i * 32 < m_lim && j * 32 + 16 * qp < n_lim;
+                    const bool in = FULL || (i * 32 < m_lim && j * 32 + 16 * qp < n_lim);
                     const uint32_t off = (uint32_t)(((i * 32) * G.N + j * 32 + 16 * qp) * 2) + c_lane_off;
-                    rres[i & 1][j][qp] = *(const uint4*)(r_tile + (in ? off : 0u));
+                    rres[i % RD][j][qp] = *(const uint4*)(r_tile + (in ? off : 0u));
                 }
         };
-        load_res(0);
+#pragma unroll
+        for (int i = 0; i < RD - 1; i++) load_res(i);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            if (i < 3) load_res(i + 1);
+            if (i + RD - 1 < 4) load_res(i + RD - 1);
             uint32_t spack[TJ] = {};
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
@@ -400,7 +407,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                 float v[16];
 #pragma unroll
                 for (int r = 0; r < 16; r++) v[r] = acc[j][i][r] * scale;
-                if (biasp) {
+                if (!FULL && biasp) {
 #pragma unroll
                     for (int q = 0; q < 4; q++)
 #pragma unroll
@@ -417,7 +424,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                     const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
                     const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
                     const uint32_t t[4] = {s0[0], s1[0], s0[1], s1[1]};  // columns j*32 + 16*qp + 8*half .. + 7 of the row
-                    const uint4 rv = rres[i & 1][j][qp];
+                    const uint4 rv = rres[i % RD][j][qp];
                     const uint32_t ru[4] = {rv.x, rv.y, rv.z, rv.w};
                     float f[8];
 #pragma unroll
@@ -425,7 +432,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                         f[2 * k] = bf16lo(t[k]) + bf16lo(ru[k]);
                         f[2 * k + 1] = bf16hi(t[k]) + bf16hi(ru[k]);
                     }
-                    const bool in = i * 32 < m_lim && j * 32 + 16 * qp < n_lim;
+                    const bool in = FULL || (i * 32 < m_lim && j * 32 + 16 * qp < n_lim);
                     if (in) {
                         uint8_t* base = c_tile + ((int64_t)(i * 32) * G.N + j * 32 + 16 * qp) * 2;
                         *(uint4*)(base + c_lane_off) = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]),
@@ -446,7 +453,7 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                         if (in) {  // N % 16 == 0: a group is inside or outside as a whole
                             uint8_t* base = cq_tile + ((int64_t)(i * 32) * G.N + j * 32 + 16 * qp);
                             *(uint2*)(base + q_lane_off) = make_uint2(w0, w1);
-                            if (half == 0 && !pack_scales) {
+                            if (half == 0 && !(FULL || pack_scales)) {
                                 uint8_t* sbase = s_tile + ((int64_t)(i * 32) * (G.N >> 4) + j * 2 + qp) * 2;
                                 *(uint16_t*)(sbase + s_lane_off) = (uint16_t)f2bf16(sg);
                             }
@@ -455,11 +462,17 @@ __global__ __launch_bounds__(512) void k_fp8_gemm(GemmArgs G) {
                     }
                 }
             }
-            if (QUANT && pack_scales && half == 0 && i * 32 < m_lim) {
+            if (QUANT && (FULL || pack_scales) && half == 0 && (FULL || i * 32 < m_lim)) {
                 uint8_t* sbase = s_tile + (int64_t)(i * 32) * (G.N >> 4) * 2;
                 *(uint2*)(sbase + s_lane_off) = make_uint2(spack[0], spack[1]);
             }
         }
+        };
+        // uniform over the wave: every row and column of its sub-tile exists, rows of the scale tensor can take 8-byte stores
+        const bool full = m0 + wm * 128 + 128 <= G.M && n0 + wn * (TJ * 32) + TJ * 32 <= G.N && !biasp &&
+                          (!QUANT || pack_scales);
+        if (full) residual_epilogue(std::true_type{});
+        else residual_epilogue(std::false_type{});
     } else if constexpr (EPI != kEpiBf16 && QBE > 16) {
         // Groups of 32 or 64 columns (reference linear.py:139-164 is generic in the group size): a row's 32 columns of
         // one accumulator tile sit in lanes l and l ^ 32, its 64 columns of the wave in the two tiles of those lanes, so

@@ -274,15 +274,26 @@ __global__ __launch_bounds__(256) void k_rmsnorm_fwd(const uint8_t* __restrict__
 // Five chunks (the 5120 columns of the 13B shape) with several gradients need 268 registers; held to 256, i.e. to two
 // waves per SIMD with 12 registers spilled, the kernel takes 91 us per call in the 13B layer against 104 us with one wave
 // per SIMD and no spill (128.7 us as 5 of 8 chunks, loaded chunk by chunk).
-template <int KIND, int WDT, int CH, bool MULTI>
-__global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+// ADD: the residual-gradient addition that follows in the layer (reference add_bwd.py:107-135 after
+// func_rmsnorm.py:121-196) happens here: dx is rounded to bf16 as it would be stored, `radd` (bf16 [M, N]) is added in
+// fp32, and what goes out is bf16 of the sum, the bf16 scale (amax + 1e-10) / fp8max of every 1 x qb group of the fp32 sum
+// and the maximum of those scales (fp32) for the per-tensor division that follows.
+struct RmsAddArgs {
+    const void* radd;   // bf16 [M, N]
+    void* s_pg;         // bf16 [M, N / qb]
+    float* s_max;       // COAT_MAX_WORDS
+    int kind_out;       // kE4M3 / kE5M2: the FP8 format the scales are for
+};
+template <int KIND, int WDT, int CH, bool MULTI, bool ADD = false>
+__global__ __launch_bounds__(256, ((CH == 5 && MULTI) || (ADD && CH == 4)) ? 2 : 1) void k_rmsnorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
                                                       const void* __restrict__ dy, const void* __restrict__ dy2,
                                                       const void* __restrict__ dy3, const void* __restrict__ w,
                                                       const float* __restrict__ rstd_in, void* __restrict__ dx,
-                                                      float* __restrict__ dw_partial, int64_t M, int N, int qb) {
+                                                      float* __restrict__ dw_partial, int64_t M, int N, int qb,
+                                                      RmsAddArgs A) {
     // MULTI spends those registers on gradient loads in flight; with five chunks they decide between one and two waves per
     // SIMD (61.3 -> 50.1 us at [8192, 5120]), with eight there is one wave either way and re-reading the weight costs 20 %
-    constexpr bool HOLD_W = WDT != kF32 && !MULTI && CH != 5;
+    constexpr bool HOLD_W = WDT != kF32 && !MULTI && CH != 5 && !ADD;
     __shared__ float red[4][64 * 16];
     const int lane = threadIdx.x & 63, wv_id = threadIdx.x >> 6;
     const int64_t nwaves = (int64_t)gridDim.x * 4;
@@ -303,6 +314,7 @@ __global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd
     for (int c = 0; c < CH; c++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[c][i] = 0.0f;
+    float wave_max = 0.0f;  // ADD: largest group scale this lane has seen
     for (int64_t row = (int64_t)blockIdx.x * 4 + wv_id; row < M; row += nwaves) {
         const int64_t row_off = row * N;
         RowRaw<CH> raw;
@@ -317,6 +329,14 @@ __global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd
                 g[c][1] = gp[1];
             }
         }
+        // ADD: the residual gradient, two chunks in flight: chunk 0 is requested before the row is reduced, chunk c + 1
+        // before chunk c is used (a whole row of it in registers costs the kernel its second wave per SIMD).
+        uint4 ra[2][2];
+        auto load_radd = [&](int c) {
+            const int col = min((c * 64 + lane) * 16, N - 16);
+            const uint4* p = (const uint4*)((const uint16_t*)A.radd + row_off + col);
+            ra[c & 1][0] = p[0]; ra[c & 1][1] = p[1];
+        };
         const float rstd = rstd_in[row];
         if constexpr (MULTI) {
             // further gradients of the same tensor, summed the way a chain of bf16 tensor additions would:
@@ -385,6 +405,7 @@ __global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd
                 }
             }
         }
+        if constexpr (ADD) load_radd(0);
         float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int c = 0; c < CH; c++) {
@@ -405,9 +426,13 @@ __global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd
             }
         }
         const float c1 = row_sum4(part) / (float)N;
+        float gmax[ADD ? CH : 1] = {};  // ADD: max |sum| of the lane's chunk c (0 for a chunk past the row's end)
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int col = (c * 64 + lane) * 16;
+            if constexpr (ADD) {
+                if (c + 1 < CH) load_radd(c + 1);
+            }
             if (col < N) {
                 float xv[16], wvv[16], gv[16], o[16];
                 decode16<KIND>(raw.codes[c], scale_from_raw(raw.sc[c], s_dt), xv);
@@ -416,9 +441,39 @@ __global__ __launch_bounds__(256, (CH == 5 && MULTI) ? 2 : 1) void k_rmsnorm_bwd
                 unpack_w16<kBF16>(g[c], gv);
 #pragma unroll
                 for (int i = 0; i < 16; i++) o[i] = ((wvv[i] * gv[i]) - ((xv[i] * rstd) * c1)) * rstd;
+                if constexpr (ADD) {
+                    float rg[16];
+                    unpack_w16<kBF16>(ra[c & 1], rg);
+#pragma unroll
+                    for (int i = 0; i < 16; i++) o[i] = rg[i] + round_to<kBF16>(o[i]);
+                    float am = fmaxf(fabsf(o[0]), fabsf(o[1]));
+#pragma unroll
+                    for (int i = 2; i < 16; i++) am = fmaxf(am, fabsf(o[i]));
+                    gmax[c] = am;
+                }
                 store_bf16_16(dx, row_off + col, o);
             }
         }
+        if constexpr (ADD) {
+            const int lpg = qb >> 4;  // lanes per group: neighbouring lanes hold neighbouring chunks
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                const float am = cluster_max_rt(gmax[c], lpg);
+                const float sg = A.kind_out == kE5M2 ? group_scale<kE5M2>(am) : group_scale<kE4M3>(am);
+                const int col = (c * 64 + lane) * 16;
+                if (col < N) {
+                    if ((lane & (lpg - 1)) == 0) ((uint16_t*)A.s_pg)[row * (N / qb) + col / qb] = (uint16_t)f2bf16(sg);
+                    wave_max = fmaxf(wave_max, sg);
+                }
+            }
+        }
+    }
+    if constexpr (ADD) {  // one lazy atomic per block
+        __shared__ float wmax[4];
+        wave_max = cluster_max<64>(wave_max);
+        if (lane == 0) wmax[wv_id] = wave_max;
+        __syncthreads();
+        if (threadIdx.x == 0) atomic_max_nonneg(max_slot(A.s_max), fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3])));
     }
     // the block's partial row: waves added in index order, 1024 columns per round
 #pragma unroll
@@ -498,27 +553,36 @@ extern "C" int coat_fp8_rmsnorm_forward(const void* x, int fp8, const void* s_x,
 // Shared by the two backward entry points: dx kernel on min(n_partial, M) blocks, then the column sum of their partial rows.
 static int rms_backward_launch(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
                                const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
-                               float* dw_partial, int64_t n_partial, int64_t M, int64_t N, int QB, hipStream_t st) {
+                               float* dw_partial, int64_t n_partial, int64_t M, int64_t N, int QB, hipStream_t st,
+                               const RmsAddArgs* add = nullptr) {
     RMS_CHECK_ENUMS()
     // one partial row per block: min(n_partial, M) blocks of the block-per-row kernel, min(n_partial, ceil(M / 4)) blocks
     // of four row-owning waves otherwise
     const int64_t rows_per_block = N <= 8192 ? 4 : 1;
     const int64_t want = (M + rows_per_block - 1) / rows_per_block;
     const int64_t grid = n_partial < want ? n_partial : want;
+    if (add && N > 8192) return COAT_ESHAPE;  // the fused addition exists in the wave-per-row kernels only
+    const RmsAddArgs no_add = {};
 #define RMS_BWD_WAVE(K, W, CHV, MU)                                                                                    \
-    hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, CHV, MU>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, s_dtype, \
-                       dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB)
+    {                                                                                                                  \
+        if (add)                                                                                                       \
+            hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, CHV, MU, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, \
+                               s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB, *add);                   \
+        else                                                                                                           \
+            hipLaunchKernelGGL((k_rmsnorm_bwd<K, W, CHV, MU, false>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, \
+                               s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB, no_add);                 \
+    }
 #define RMS_BWD(K, W)                                                                                                  \
     case K * 3 + W:                                                                                                    \
         if (N <= 4096) {                                                                                               \
-            if (dy2) RMS_BWD_WAVE(K, W, 4, true);                                                                      \
-            else RMS_BWD_WAVE(K, W, 4, false);                                                                         \
+            if (dy2) RMS_BWD_WAVE(K, W, 4, true)                                                                       \
+            else RMS_BWD_WAVE(K, W, 4, false)                                                                          \
         } else if (N <= 5120) {                                                                                        \
-            if (dy2) RMS_BWD_WAVE(K, W, 5, true);                                                                      \
-            else RMS_BWD_WAVE(K, W, 5, false);                                                                         \
+            if (dy2) RMS_BWD_WAVE(K, W, 5, true)                                                                       \
+            else RMS_BWD_WAVE(K, W, 5, false)                                                                          \
         } else if (N <= 8192) {                                                                                        \
-            if (dy2) RMS_BWD_WAVE(K, W, 8, true);                                                                      \
-            else RMS_BWD_WAVE(K, W, 8, false);                                                                         \
+            if (dy2) RMS_BWD_WAVE(K, W, 8, true)                                                                       \
+            else RMS_BWD_WAVE(K, W, 8, false)                                                                          \
         } else {                                                                                                       \
             hipLaunchKernelGGL((k_rmsnorm_bwd_block<K, W, 4>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t*)x, s_x, \
                                s_dtype, dy, dy2, dy3, w, rstd, dx, dw_partial, M, (int)N, QB);                         \
@@ -561,6 +625,23 @@ extern "C" int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x
     if (!coat_aligned16(dw_partial)) return COAT_EALIGN;
     return rms_backward_launch(x, fp8, s_x, s_dtype, dy, dy2, dy3, w, w_dtype, rstd, dx, dw, dw_partial, n_partial, M, N, QB,
                                (hipStream_t)stream);
+}
+
+extern "C" int coat_fp8_rmsnorm_backward_add(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
+                                             const void* dy2, const void* dy3, const void* w, int w_dtype,
+                                             const float* rstd, const void* residual_grad, void* y, void* s_pg,
+                                             float* s_max, int fp8_out, void* dw, float* dw_partial, int n_partial,
+                                             int64_t M, int64_t N, int QB, void* stream) {
+    if (int e = rms_check(M, N, QB)) return e;
+    if (N > 8192 || QB > 1024) return COAT_ESHAPE;
+    if (M * N == 0) return COAT_OK;
+    if (!dw_partial || n_partial <= 0 || !residual_grad || !s_pg || !s_max) return COAT_EINVAL;
+    if (fp8_out != COAT_E4M3 && fp8_out != COAT_E5M2) return COAT_EINVAL;
+    if (int e = rms_backward_check(x, s_x, dy, dy2, dy3, w, rstd, y, dw)) return e;
+    if (!coat_aligned16(dw_partial) || !coat_aligned16(residual_grad)) return COAT_EALIGN;
+    const RmsAddArgs add = {residual_grad, s_pg, s_max, fp8_out == COAT_E5M2 ? kE5M2 : kE4M3};
+    return rms_backward_launch(x, fp8, s_x, s_dtype, dy, dy2, dy3, w, w_dtype, rstd, y, dw, dw_partial, n_partial, M, N, QB,
+                               (hipStream_t)stream, &add);
 }
 
 // ------------------------------------------------------------------------------------------------ no allocation

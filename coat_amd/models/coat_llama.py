@@ -24,9 +24,10 @@ import torch.nn.functional as F
 from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt, fp8_division,
                                             fp8_division_transpose, fp8_linear_backward, fp8_linear_backward_grouped,
-                                            fp8_linear_forward, fp8_linear_forward_grouped,
+                                            fp8_linear_forward, fp8_linear_forward_add, fp8_linear_forward_grouped,
                                             fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
-                                            fp8_rmsnorm_backward, fp8_rmsnorm_forward, fp8_silu_mul_backward,
+                                            fp8_rmsnorm_backward, fp8_rmsnorm_backward_add, fp8_rmsnorm_forward,
+                                            fp8_silu_mul_backward,
                                             fp8_silu_mul_forward, fp8_transpose)
 from ..activation.real_quantization.common import scale_max
 from ..utils._fp8_quantization_config import QuantizationConfig
@@ -187,9 +188,9 @@ class _CoatLlamaBeforeAttentionResidual(torch.autograd.Function):
         dgrads, wgrads = fp8_linear_backward_grouped(ln_x_t, ln_s, g8s, gss, g8_ts, w_ts, list(ctx.weight[1::2]), group_size)
         del g8s, g8_ts, w_ts
         # fc1_g = dgrads[0] + dgrads[1] + dgrads[2] (reference :328), summed inside the kernel with the same roundings
-        in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, tuple(dgrads), rms_weight, rstd, group_size, num_warps)
-        re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],
-                                                                stochastic=False)
+        # and fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g) (:331-339) inside the same kernel
+        re_g, (in_g, in_sg, in_sg_g16), rms_weight_grad = fp8_rmsnorm_backward_add(
+            in_x, in_s, tuple(dgrads), rms_weight, rstd, group_size, num_warps, fp_grad, fwobits["babit"], stochastic=False)
         # the per-group scale tensor is returned as the "gradient" of the forward scales so that shapes match;
         # the consumer takes its maximum, which is the scale in_g was quantized with
         return (re_g, in_g.view(E4M3), in_sg_g16,
@@ -220,8 +221,8 @@ class _CoatLlamaAfterAttentionResidual(torch.autograd.Function):
     def forward(ctx, re_x, flash_x, w4_origin, w4, w4_t, w4_s, group_size, fwobits, layer_id, config, qargs):
         flash_qx, flash_s, _ = fp8_quantize_pertensor(flash_x, group_size, fwobits["fabit"])
         w8 = _forward_weight(w4_origin, w4, w4_s, qargs, fwobits)
-        fc4_x = fp8_linear_forward(flash_qx, flash_s, w8, w4_s, False, group_size)
-        fp_x, (out_x, out_s) = fp8_add_Ifp_Ifp_Ofp_Og16(re_x, fc4_x, flash_qx.dtype, group_size)
+        # fp8_linear_forward + fp8_add_Ifp_Ifp_Ofp_Og16 of the reference (:440-441): the addition runs in the GEMM epilogue
+        fp_x, (out_x, out_s) = fp8_linear_forward_add(flash_qx, flash_s, w8, w4_s, re_x, flash_qx.dtype, group_size)
         # the bf16 attention output is saved (not its FP8 copy): its transpose is re-quantized in backward
         ctx.save_for_backward(flash_x, flash_s)
         ctx.weight = (w4_origin, w4_s) if qargs.weight_memory_efficient else (w4_t, w4_s)
@@ -284,9 +285,9 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
         # one kernel for fp8_silu_forward + fp8_mul_forward of the reference (:664-668), same tensors
         silu_x, silu_s, mul_x, mul_s, mul_x_t = fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, group_size,
                                                                       transpose_output_2d=True)
-        fc3_x = fp8_linear_forward(mul_x, mul_s, _forward_weight(w3_origin, w3, w3_s, qargs, fwobits), w3_s, False,
-                                   group_size)
-        fp_x, (out_x, out_s) = fp8_add_Ifp_Ifp_Ofp_Og16(re_x, fc3_x, mul_x.dtype, group_size)
+        # fp8_linear_forward + fp8_add_Ifp_Ifp_Ofp_Og16 of the reference (:673-674) in one kernel
+        fp_x, (out_x, out_s) = fp8_linear_forward_add(mul_x, mul_s, _forward_weight(w3_origin, w3, w3_s, qargs, fwobits),
+                                                      w3_s, re_x, mul_x.dtype, group_size)
         ctx.save_for_backward(in_x, in_s, ln_x_t, ln_s, gate_x, gate_s, up_x, up_s, silu_x, silu_s, mul_x_t, mul_s)
         if qargs.weight_memory_efficient:
             ctx.weight = (w1_origin, w1_s, w2_origin, w2_s, w3_origin, w3_s)
@@ -322,9 +323,9 @@ class _CoatLlamaMLPResidual(torch.autograd.Function):
         (fc1_g, fc2_g), (weight1_grad, weight2_grad) = fp8_linear_backward_grouped(
             ln_x_t, ln_s, [silu_g, mul_g2], [silu_gs, mul_gs2], [silu_g_t, mul_g2_t], [w1_t, w2_t], [w1_s, w2_s], group_size)
         # fc_g = fc1_g + fc2_g (reference :742), summed inside the kernel
-        in_g, rms_weight_grad = fp8_rmsnorm_backward(in_x, in_s, (fc1_g, fc2_g), rms_weight, rstd, group_size, num_warps)
-        re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],
-                                                                stochastic=False)
+        # and fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g) (:745-754) inside the same kernel
+        re_g, (in_g, in_sg, in_sg_g16), rms_weight_grad = fp8_rmsnorm_backward_add(
+            in_x, in_s, (fc1_g, fc2_g), rms_weight, rstd, group_size, num_warps, fp_grad, fwobits["babit"], stochastic=False)
         return (re_g, in_g.view(E4M3), in_sg_g16,
                 weight1_grad, None, None, None, weight2_grad, None, None, None, weight3_grad, None, None, None,
                 rms_weight_grad, None, None, None, None, None, None)

@@ -18,6 +18,7 @@ from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt,
                                             fp8_division_transpose, fp8_layernorm_noparam_backward,
                                             fp8_layernorm_noparam_forward, fp8_linear_backward, fp8_linear_forward,
+                                            fp8_linear_forward_add,
                                             fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
                                             fp8_silu_mul_backward_joined, fp8_silu_mul_forward, fp8_transpose)
 from ..activation.real_quantization.common import scale_max
@@ -127,9 +128,9 @@ class _CoatOLMoAfterAttentionResidual(torch.autograd.Function):
     @staticmethod
     def forward(ctx, re_x, flash_x, w2_origin, w2, w2_t, w2_s, group_size, fwobits, layer_id, config, qargs):
         flash_qx, flash_s, _ = fp8_quantize_pertensor(flash_x, group_size, fwobits["fabit"])
-        fc2_x = fp8_linear_forward(flash_qx, flash_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits), w2_s, False,
-                                   group_size)
-        fp_x, (out_x, out_s) = fp8_add_Ifp_Ifp_Ofp_Og16(re_x, fc2_x, flash_qx.dtype, group_size)
+        # projection + residual addition (fp8_linear_forward then fp8_add_Ifp_Ifp_Ofp_Og16 in the reference) in one kernel
+        fp_x, (out_x, out_s) = fp8_linear_forward_add(flash_qx, flash_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits),
+                                                      w2_s, re_x, flash_qx.dtype, group_size)
         # the bf16 attention output is saved (not its FP8 copy): its transpose is re-quantized in backward (:331)
         ctx.save_for_backward(flash_x, flash_s)
         ctx.weight = (w2_origin, w2_s) if qargs.weight_memory_efficient else (w2_t, w2_s)
@@ -189,9 +190,9 @@ class _CoatOLMoMLPResidual(torch.autograd.Function):
         up_s, gate_s = fc1_s.chunk(2, dim=-1)
         silu_x, silu_s, mul_x, mul_s, mul_x_t = fp8_silu_mul_forward(gate_x, gate_s, up_x, up_s, group_size,
                                                                     transpose_output_2d=True)
-        fc2_x = fp8_linear_forward(mul_x, mul_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits), w2_s, False,
-                                   group_size)
-        fp_x, (out_x, out_s) = fp8_add_Ifp_Ifp_Ofp_Og16(re_x, fc2_x, mul_x.dtype, group_size)
+        # projection + residual addition in one kernel, as above
+        fp_x, (out_x, out_s) = fp8_linear_forward_add(mul_x, mul_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits),
+                                                      w2_s, re_x, mul_x.dtype, group_size)
         ctx.save_for_backward(in_x, in_s, ln_x_t, ln_s, gate_x, gate_s, up_x, up_s, silu_x, silu_s, mul_x_t, mul_s)
         if qargs.weight_memory_efficient:
             ctx.weight = (w1_origin, w1_s, w2_origin, w2_s)

@@ -200,6 +200,17 @@ int coat_fp8_product_division(const void* a, const void* s_a, int sa_dtype, cons
 int coat_fp8_rmsnorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
                               const void* dy3, const void* w, int w_dtype, const float* rstd, void* dx, void* dw,
                               float* dw_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream);
+/* coat_fp8_rmsnorm_backward followed by the residual-gradient addition rq/add_bwd.py:147 fp8_add_Ifp_Ifp_Ofp_Opt (kernel
+ * :107-135), as one kernel (the reference runs the two one after the other, coat/models/coat_llama.py:331-339, :745-754):
+ * dx is rounded to bf16 as coat_fp8_rmsnorm_backward stores it, v = float(residual_grad) + float(dx) in fp32,
+ * y = bf16(v) [M,N]; s_pg = bf16 scales (amax + 1e-10) / fp8max(fp8_out) of the 1 x QB groups of v [M, N/QB]; the largest
+ * fp32 group scale is merged into s_max (COAT_MAX_WORDS, zero-filled by the caller), from which
+ * coat_fp8_division_from_max of y gives the per-tensor codes.  Bit-identical to the two entry points.  N <= 8192. */
+int coat_fp8_rmsnorm_backward_add(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* dy2,
+                                  const void* dy3, const void* w, int w_dtype, const float* rstd,
+                                  const void* residual_grad, void* y, void* s_pg, float* s_max, int fp8_out, void* dw,
+                                  float* dw_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream);
+
 /* No counterpart in the reference.  For callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): coat_fp8_rmsnorm_backward without the workspace argument.  The partial rows live in a
  * device array inside the library, COAT_RMSNORM_STATIC_PARTIALS x COAT_RMSNORM_STATIC_FULL_N floats (16 MiB per GPU, held

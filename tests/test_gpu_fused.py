@@ -279,6 +279,36 @@ def test_rmsnorm_backward_sums_gradients_like_bf16_additions(dev, N):
         assert torch.equal(dx_t, dx_s) and torch.equal(dw_t, dw_s)
 
 
+@pytest.mark.parametrize("M,N,QBv,fp8out", [(96, 1024, 16, "E5M2"), (1504, 4096, 16, "E5M2"), (208, 5120, 16, "E5M2"),
+                                            (96, 4096 + 2048, 64, "E4M3"), (64, 8192 + 1024, 16, "E5M2")])
+def test_rmsnorm_backward_with_residual_addition_equals_the_two_kernels(dev, M, N, QBv, fp8out):
+    """fp8_rmsnorm_backward_add against fp8_rmsnorm_backward followed by fp8_add_Ifp_Ifp_Ofp_Opt, with one, two and three
+    gradients: the bf16 sum, the per-group scales, the per-tensor scale, the codes and dw, bit for bit; the addition
+    itself against the oracle.  Widths take the 4-, 5- and 8-chunk kernels; the widest falls back to the two kernels."""
+    rq = _rq()
+    from coat_amd.activation.real_quantization.func_rmsnorm import fp8_rmsnorm_backward_add
+    x = rand(70, shape=(M, N))
+    w = (1 + 0.1 * rand(71, shape=(N,)).float()).bfloat16().to(dev)
+    gs = [rand(72 + i, 0.01 * (i + 1), shape=(M, N)).to(dev) for i in range(3)]
+    res = rand(76, 0.02, shape=(M, N))
+    res[::5, ::3] *= 30
+    res = res.to(dev)
+    q, s = rq.fp8_quantize(x.to(dev), QBv, "E4M3")
+    _, _, _, (_, rstd, nw) = rq.fp8_rmsnorm_forward(q, s, w, QBv, 1e-5, transpose_output_2d=True)
+    for n in (1, 2, 3):
+        g = tuple(gs[:n]) if n > 1 else gs[0]
+        dx, dw = rq.fp8_rmsnorm_backward(q, s, g, w, rstd, QBv, nw)
+        want_y, (want_q, want_s, want_pg) = rq.fp8_add_Ifp_Ifp_Ofp_Opt(res, dx, QBv, fp8out)
+        got_y, (got_q, got_s, got_pg), got_dw = fp8_rmsnorm_backward_add(q, s, g, w, rstd, QBv, nw, res, fp8out)
+        assert torch.equal(got_y, want_y), (n, "sum")
+        assert torch.equal(got_pg.view(torch.int16), want_pg.view(torch.int16)), (n, "group scales")
+        assert got_s.dtype == want_s.dtype and got_s.item() == want_s.item(), (n, "tensor scale")
+        assert torch.equal(b(got_q), b(want_q)) and torch.equal(got_dw, dw), (n, "codes / dw")
+        oy, (oq, os_, opg) = R.fp8_add_Ifp_Ifp_Ofp_Opt(res.cpu(), dx.cpu(), QBv, fp8out)
+        assert torch.equal(got_y.cpu(), oy) and torch.equal(got_pg.cpu(), opg) and os_.item() == got_s.item()
+        assert torch.equal(b(got_q), oq.view(torch.uint8))
+
+
 def test_larger_groups_and_float32_scales(dev):
     rq = _rq()
     x1, x2 = rand(13, shape=(128, 512)), rand(14, shape=(128, 512))

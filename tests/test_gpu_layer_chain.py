@@ -118,6 +118,37 @@ class Recorder:
         # of the reference that it stands for, so the checks below read like the reference's call sequence
         monkeypatch.setattr(L, "fp8_linear_forward_grouped", self._wrap_forward_grouped(L.fp8_linear_forward_grouped))
         monkeypatch.setattr(L, "fp8_linear_backward_grouped", self._wrap_backward_grouped(L.fp8_linear_backward_grouped))
+        from coat_amd.activation.real_quantization import func_rmsnorm as _rms
+        from coat_amd.activation.real_quantization import linear as _linear
+        monkeypatch.setattr(L, "fp8_rmsnorm_backward_add", self._wrap_backward_add(L.fp8_rmsnorm_backward_add, _rms.fp8_rmsnorm_backward))
+        monkeypatch.setattr(L, "fp8_linear_forward_add", self._wrap_forward_add(L.fp8_linear_forward_add, _linear.fp8_linear_forward))
+
+    def _wrap_backward_add(self, fn, plain_backward):
+        """The RMSNorm backward adds the residual gradient before it stores.  Logged as the reference's two calls: the
+        backward (dx from a separate launch of the plain kernel on the same operands) and the addition of that dx, whose
+        logged result is what the fused kernel returned: the oracle's addition of the logged dx must reproduce it bit
+        for bit."""
+        def wrapper(x, s_x, g, w, v, QB, num_warps, residual_grad, fp8type, stochastic=False):
+            y, quant, dw = fn(x, s_x, g, w, v, QB, num_warps, residual_grad, fp8type, stochastic=stochastic)
+            dx, dw_plain = plain_backward(x, s_x, g, w, v, QB, num_warps)
+            assert torch.equal(dw, dw_plain)
+            self.calls.append(("fp8_rmsnorm_backward", (x, s_x, g, w, v, QB, num_warps), {}, (dx, dw)))
+            self.calls.append(("fp8_add_Ifp_Ifp_Ofp_Opt", (residual_grad, dx, QB, fp8type), {"stochastic": stochastic}, (y, quant)))
+            return y, quant, dw
+        return wrapper
+
+    def _wrap_forward_add(self, fn, plain_linear):
+        """The projection that closes a residual branch adds the residual in its epilogue.  It is logged as the reference's
+        two calls: the projection (its bf16 product taken from a separate launch of the same GEMM on the same operands) and
+        the addition of that product, whose logged result is what the fused kernel returned.  The checks on the addition
+        (bit for bit against the oracle's addition of the logged product) therefore hold the fused kernel to the chain."""
+        def wrapper(x, s, w, s_w, residual, fp8type, QB, bias=None):
+            out = fn(x, s, w, s_w, residual, fp8type, QB, bias)
+            product = plain_linear(x, s, w, s_w, False, QB, bias)
+            self.calls.append(("fp8_linear_forward", (x, s, w, s_w, False, QB), {}, product))
+            self.calls.append(("fp8_add_Ifp_Ifp_Ofp_Og16", (residual, product, fp8type, QB), {}, out))
+            return out
+        return wrapper
 
     def _wrap_forward_grouped(self, fn):
         def wrapper(x, s, w_list, s_w_list, output_quantize, QB):
