@@ -1,4 +1,6 @@
 """Constants of the FP8 op library (reference: coat/activation/real_quantization/common.py:20-31)."""
+import threading
+
 import torch
 
 SCALE_MIN_THRES = 1e-10
@@ -46,6 +48,7 @@ def no_stochastic(stochastic, why):
 
 _MAX_POOL = {}
 _MAX_POOL_SIZE = 64
+_MAX_POOL_LOCK = threading.Lock()  # host threads may call the entry points together (autograd's backward threads do)
 
 
 def new_max(device):
@@ -64,13 +67,15 @@ def new_max(device):
         # maxima of earlier replays), and memory of the graph's private pool must not be handed out after the capture
         return torch.zeros(_hip.MAX_WORDS, dtype=torch.float32, device=device)
     key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
-    pool = _MAX_POOL.get(key)
-    if pool is None or pool[1] >= _MAX_POOL_SIZE:
-        pool = [torch.zeros(_MAX_POOL_SIZE * _hip.MAX_WORDS, dtype=torch.float32, device=device), 0]
-        _MAX_POOL[key] = pool
-    i = pool[1]
-    pool[1] = i + 1
-    return pool[0][i * _hip.MAX_WORDS:(i + 1) * _hip.MAX_WORDS]
+    with _MAX_POOL_LOCK:  # the slot counter and the dictionary are shared by the threads that use one device and stream
+        pool = _MAX_POOL.get(key)
+        if pool is None or pool[1] >= _MAX_POOL_SIZE:
+            pool = [torch.zeros(_MAX_POOL_SIZE * _hip.MAX_WORDS, dtype=torch.float32, device=device), 0]
+            _MAX_POOL[key] = pool
+        i = pool[1]
+        pool[1] = i + 1
+        buf = pool[0]
+    return buf[i * _hip.MAX_WORDS:(i + 1) * _hip.MAX_WORDS]
 
 
 def scale_max(s):

@@ -122,20 +122,44 @@ _MAX_GROUP = 4  # problems per grouped launch (kMaxGroup of the kernel)
 
 
 def fp8matmul_grouped(a_list, b_list, output_quantize, scale_a_list, scale_b_list, QB):
-    """``[fp8matmul(a, b, output_quantize, sa, sb, QB) for ...]`` in one launch when every problem has the same shape
-    and formats (2-D ``a``, no bias): the q / k / v or gate / up projections of a layer and their backward products.
+    """``[fp8matmul(a, b, output_quantize, sa, sb, QB) for ...]`` with the problems that share a shape and formats (2-D
+    ``a``, no bias) in one launch each: the q / k / v or gate / up projections of a layer and their backward products.
     The results are bit-identical to the separate calls; on the persistent grid the problems' tiles form one sequence,
-    so a partial last round of tiles is paid once per group.  Anything else falls back to the separate calls."""
+    so a partial last round of tiles is paid once per group.  Problems of different shapes form groups of their own
+    (grouped-query attention: k and v share a launch, q takes its own); a problem alone in its group, or one the
+    grouped kernel does not take, is a separate call."""
     n = len(a_list)
     assert n == len(b_list) == len(scale_a_list) == len(scale_b_list)
-    same = (1 < n <= _MAX_GROUP and all(a.dim() == 2 and a.is_contiguous() for a in a_list)
-            and len({(tuple(a.shape), a.dtype, tuple(b.shape), b.dtype, b.t().is_contiguous())
-                     for a, b in zip(a_list, b_list)}) == 1 and b_list[0].t().is_contiguous()
-            and len({s.dtype for s in scale_a_list}) == 1 and len({s.dtype for s in scale_b_list}) == 1
-            and all(s.numel() == 1 and s.is_cuda for s in (*scale_a_list, *scale_b_list)))
-    if not same:
-        return [fp8matmul(a, b, output_quantize, sa, sb, QB)
-                for a, b, sa, sb in zip(a_list, b_list, scale_a_list, scale_b_list)]
+
+    def signature(i):
+        a, b, sa, sb = a_list[i], b_list[i], scale_a_list[i], scale_b_list[i]
+        if not (a.dim() == 2 and a.is_contiguous() and b.t().is_contiguous() and sa.numel() == 1 and sb.numel() == 1
+                and sa.is_cuda and sb.is_cuda):
+            return None
+        return (tuple(a.shape), a.dtype, tuple(b.shape), b.dtype, sa.dtype, sb.dtype)
+
+    groups = {}
+    for i in range(n):
+        sig = signature(i)
+        groups.setdefault(sig if sig is not None else ("alone", i), []).append(i)
+    out = [None] * n
+    for sig, idx in groups.items():
+        for at in range(0, len(idx), _MAX_GROUP):
+            part = idx[at:at + _MAX_GROUP]
+            if len(part) == 1 or sig[0] == "alone":
+                for i in part:
+                    out[i] = fp8matmul(a_list[i], b_list[i], output_quantize, scale_a_list[i], scale_b_list[i], QB)
+            else:
+                res = _matmul_group([a_list[i] for i in part], [b_list[i] for i in part], output_quantize,
+                                    [scale_a_list[i] for i in part], [scale_b_list[i] for i in part], QB)
+                for i, r in zip(part, res):
+                    out[i] = r
+    return out
+
+
+def _matmul_group(a_list, b_list, output_quantize, scale_a_list, scale_b_list, QB):
+    """One launch for 2 .. 4 problems of one shape, one pair of formats and one pair of scale dtypes."""
+    n = len(a_list)
     a_list = [_hip.dense(a) for a in a_list]
     bn_list = [_hip.dense(b.t()) for b in b_list]
     M, K = a_list[0].shape

@@ -462,7 +462,7 @@ extern "C" int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, c
                                          int64_t N, int QB, int64_t in_pitch, int64_t s_pitch, void* stream) {
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !q_silu || !s_silu || !s_max)) return COAT_EINVAL;  // y may be NULL
     SiluMulArgs A = {gate, s_gate, up, s_up, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr,
-                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0, kBF16};
+                     nullptr, nullptr, nullptr, nullptr};
     return silu_mul_launch(A, false, fp8, fp8, M, N, QB, s_dtype, in_pitch, s_pitch, 0, (hipStream_t)stream);
 }
 
@@ -474,7 +474,7 @@ extern "C" int coat_fp8_silu_mul_forward_bf16(const void* gate, const void* up, 
     if ((M > 0 && N > 0) && (!gate || !up || !q_gate || !s_gate || !q_up || !s_up || !q_silu || !s_silu || !s_max))
         return COAT_EINVAL;  // y may be NULL
     SiluMulArgs A = {gate, nullptr, up, nullptr, nullptr, nullptr, nullptr, q_silu, s_silu, y, nullptr, s_max, nullptr,
-                     q_gate, s_gate, q_up, s_up, 0, 0, 0, kBF16};
+                     q_gate, s_gate, q_up, s_up};
     return silu_mul_launch(A, false, fp8, fp8, M, N, QB, COAT_BF16, 0, 0, 0, (hipStream_t)stream);
 }
 
@@ -486,6 +486,6 @@ extern "C" int coat_fp8_silu_mul_backward(const void* gate, const void* s_gate, 
     if ((M > 0 && N > 0) && (!gate || !s_gate || !up || !s_up || !silu || !s_silu || !g || !y_gate || !s_max_gate || !y_up || !s_max_up))
         return COAT_EINVAL;
     SiluMulArgs A = {gate, s_gate, up, s_up, silu, s_silu, g, nullptr, nullptr, y_gate, y_up, s_max_gate, s_max_up,
-                     nullptr, nullptr, nullptr, nullptr, 0, 0, 0, kBF16};
+                     nullptr, nullptr, nullptr, nullptr};
     return silu_mul_launch(A, true, fp8_in, fp8_out, M, N, QB, s_dtype, in_pitch, s_pitch, y_pitch, (hipStream_t)stream);
 }

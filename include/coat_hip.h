@@ -144,8 +144,8 @@ int coat_fp8_add_bwd(const void* x1, const void* x2, void* y, void* s_y, float* 
  * (forward: rq/silu_fwd.py:152 then rq/mul_fwd.py:191) and round-trip the bf16 gradient of the product (backward:
  * rq/mul_bwd.py:221 then rq/silu_bwd.py:170).  No single counterpart in the reference; used by the MLP module.
  * forward: q_silu / s_silu = per-group FP8 SiLU(gate) with bf16 scales (saved for backward), y = bf16 product of the
- * dequantized SiLU and up (may be NULL: the maximum alone, for coat_fp8_product_division), *s_max = max of the product's
- * fp32 group scales (fp8 = format of gate / up / silu). */
+ * dequantized SiLU and up (may be NULL: the maximum alone, for coat_fp8_product_division), s_max (COAT_MAX_WORDS words,
+ * as above) receives the max of the product's fp32 group scales (fp8 = format of gate / up / silu). */
 int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* up, const void* s_up, int fp8,
                               int s_dtype, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M, int64_t N,
                               int QB, int64_t in_pitch, int64_t s_pitch, void* stream);
@@ -155,8 +155,9 @@ int coat_fp8_silu_mul_forward(const void* gate, const void* s_gate, const void* 
 int coat_fp8_silu_mul_forward_bf16(const void* gate, const void* up, int fp8, void* q_gate, void* s_gate, void* q_up,
                                    void* s_up, void* q_silu, void* s_silu, void* y, float* s_max, int64_t M, int64_t N,
                                    int QB, void* stream);
-/* backward: y_up = bf16(g * silu), y_gate = bf16(silu'(gate) * bf16(g * up)); *s_max_* = max of their fp32 group
- * scales for the format fp8_out (the per-tensor division that follows is coat_fp8_division).
+/* backward: y_up = bf16(g * silu), y_gate = bf16(silu'(gate) * bf16(g * up)); s_max_gate / s_max_up (COAT_MAX_WORDS
+ * words each) receive the max of their fp32 group scales for the format fp8_out (the per-tensor division that follows is
+ * coat_fp8_division_from_max).
  * Row pitches in elements, 0 = contiguous: in_pitch / s_pitch for gate, up and their scales when they are the two column
  * halves of a fused projection's output (coat/models/coat_olmo.py:520-523 chunks and copies them), y_pitch (backward
  * only) for y_gate / y_up written side by side into one [M, 2N] tensor (coat_olmo.py:600 concatenates them). */
@@ -217,7 +218,9 @@ int coat_fp8_rmsnorm_backward_add(const void* x, int fp8, const void* s_x, int s
  * until the process ends); the call allocates and frees nothing.  It uses coat_rmsnorm_static_partials(N) partial rows
  * (512 up to N = 8192, 256 beyond), so dx and dw equal those of coat_fp8_rmsnorm_backward called with that n_partial.
  * N > 16384 is rejected with COAT_ESHAPE, as everywhere.  All calls on one GPU share the array: calls that overlap on one
- * GPU (two streams, two threads) race on it; calls on one stream are ordered and need no clearing in between. */
+ * GPU (two streams, two threads) race on it; calls on one stream are ordered and need no clearing in between.  The first
+ * call on a device looks up the array's address (hipGetSymbolAddress): make one call on that device before capturing a
+ * graph that contains this entry point. */
 #define COAT_RMSNORM_STATIC_PARTIALS 512
 #define COAT_RMSNORM_STATIC_FULL_N 8192
 static inline int coat_rmsnorm_static_partials(int64_t N) {

@@ -178,45 +178,53 @@ def test_fp8matmul_scales_in_different_dtypes(dev):
     assert torch.equal(cq.cpu().view(torch.uint8), wq.view(torch.uint8)) and torch.equal(cs.cpu(), ws)
 
 
-@pytest.mark.parametrize("count,M,N,K,fa,fb,quant", [
-    (3, 512, 512, 256, E4, E4, False),      # q / k / v forward: 12 tiles, problems change inside a block's walk
-    (2, 300, 272, 144, E5, E4, False),      # ragged tiles, partial last K-step, e5m2 gradients
-    (2, 768, 512, 384, E4, E4, True),       # gate / up forward through the quantizing epilogue
-    (4, 2304, 2048, 128, E5, E4, False),    # 4 x 72 tiles: more tiles than CUs, every XCD band spans problems
-    (3, 200, 208, 80, E4, E5, True),        # ragged tiles through the quantizing epilogue (scales stored one by one)
+@pytest.mark.parametrize("count,M,N,K,fa,fb,quant,qb,with_bias", [
+    (3, 512, 512, 256, E4, E4, False, 16, (0, 0, 0)),      # q / k / v forward: 12 tiles, problems change inside a block's walk
+    (2, 300, 272, 144, E5, E4, False, 16, (0, 0)),         # ragged tiles, partial last K-step, e5m2 gradients
+    (2, 768, 512, 384, E4, E4, True, 16, (0, 0)),          # gate / up forward through the quantizing epilogue
+    (4, 2304, 2048, 128, E5, E4, False, 16, (0, 0, 0, 0)), # 4 x 72 tiles: more tiles than CUs, every XCD band spans problems
+    (3, 200, 208, 80, E4, E5, True, 16, (0, 0, 0)),        # ragged tiles through the quantizing epilogue (scales stored one by one)
+    (3, 300, 272, 144, E4, E4, False, 16, (1, 0, 1)),      # a bias vector in the first and third problem only
+    (2, 520, 320, 208, E5, E4, True, 32, (0, 1)),          # e5m2 codes in groups of 32 columns, ragged tiles, one bias
+    (3, 264, 448, 96, E4, E4, True, 64, (0, 0, 0)),        # groups of 64 columns
 ])
-def test_grouped_gemm_equals_separate_launches(dev, count, M, N, K, fa, fb, quant):
-    """coat_fp8_gemm_grouped through the C ABI: every problem's output is bit-identical to coat_fp8_gemm on it."""
-    import ctypes
+def test_grouped_gemm_equals_separate_launches(dev, count, M, N, K, fa, fb, quant, qb, with_bias):
+    """coat_fp8_gemm_grouped through the C ABI: every problem's output is bit-identical to coat_fp8_gemm on it, with
+    per-problem bias pointers (NULL for some) and with the 16-, 32- and 64-column quantizing epilogues."""
     from coat_amd import _hip
     lib = _hip.lib()
     a = [rand_fp8((M, K), 100 + i, fa).to(dev) for i in range(count)]
     b = [rand_fp8((N, K), 200 + i, fb).to(dev) for i in range(count)]
     sa = [torch.tensor(0.02 + 0.003 * i).bfloat16().to(dev) for i in range(count)]
     sb = [torch.tensor(0.013 - 0.002 * i).float().to(dev) for i in range(count)]
+    bias = [torch.randn(N, generator=torch.Generator().manual_seed(300 + i)).bfloat16().to(dev) if with_bias[i] else None
+            for i in range(count)]
+    any_bias = any(with_bias)
     kind = {E4: 1, E5: 2}[fa] if quant else 0
     odt = fa if quant else torch.bfloat16
     want = [torch.empty((M, N), dtype=odt, device=dev) for _ in range(count)]
     got = [torch.zeros((M, N), dtype=torch.uint8, device=dev).view(odt) if quant else torch.zeros((M, N), dtype=odt, device=dev)
            for _ in range(count)]
-    want_s = [torch.empty((M, N // 16), dtype=torch.bfloat16, device=dev) for _ in range(count)] if quant else None
-    got_s = [torch.zeros((M, N // 16), dtype=torch.bfloat16, device=dev) for _ in range(count)] if quant else None
+    want_s = [torch.empty((M, N // qb), dtype=torch.bfloat16, device=dev) for _ in range(count)] if quant else None
+    got_s = [torch.zeros((M, N // qb), dtype=torch.bfloat16, device=dev) for _ in range(count)] if quant else None
     st = _hip.stream(dev)
     for i in range(count):
         _hip.check(lib.coat_fp8_gemm(_hip.ptr(a[i]), _hip.fp8(fa), _hip.ptr(b[i]), _hip.fp8(fb), _hip.ptr(want[i]),
                                      _hip.ptr(want_s[i]) if quant else None, kind, _hip.ptr(sa[i]), _hip.dt(sa[i]),
-                                     _hip.ptr(sb[i]), _hip.dt(sb[i]), None, 0, M, N, K, 16 if quant else 0, st), "gemm")
+                                     _hip.ptr(sb[i]), _hip.dt(sb[i]), _hip.ptr(bias[i]), _hip.BF16 if bias[i] is not None else 0,
+                                     M, N, K, qb if quant else 0, st), "gemm")
     _hip.check(lib.coat_fp8_gemm_grouped(count, _hip.ptr_array(a), _hip.fp8(fa), _hip.ptr_array(b), _hip.fp8(fb),
                                          _hip.ptr_array(got), _hip.ptr_array(got_s) if quant else None, kind,
-                                         _hip.ptr_array(sa), _hip.dt(sa[0]), _hip.ptr_array(sb), _hip.dt(sb[0]), None, 0,
-                                         M, N, K, 16 if quant else 0, st), "gemm_grouped")
+                                         _hip.ptr_array(sa), _hip.dt(sa[0]), _hip.ptr_array(sb), _hip.dt(sb[0]),
+                                         _hip.ptr_array(bias) if any_bias else None, _hip.BF16 if any_bias else 0,
+                                         M, N, K, qb if quant else 0, st), "gemm_grouped")
     for i in range(count):
         assert torch.equal(got[i].view(torch.uint8), want[i].view(torch.uint8)), i
         if quant:
             assert torch.equal(got_s[i].view(torch.int16), want_s[i].view(torch.int16)), i
     # the first problem against the oracle's bound as well
     if not quant:
-        check_bf16(got[0], a[0].cpu(), b[0].cpu(), sa[0].cpu(), sb[0].cpu())
+        check_bf16(got[0], a[0].cpu(), b[0].cpu(), sa[0].cpu(), sb[0].cpu(), bias[0].cpu() if bias[0] is not None else None)
 
 
 @pytest.mark.parametrize("M,N,K,fa,fb,out,with_bias", [
@@ -288,10 +296,12 @@ def test_grouped_linear_wrappers_equal_the_separate_calls(dev):
     for i in range(3):
         dx, dw = lin.fp8_linear_backward(xt, s, gs8[i], sgs[i], gts[i], wts[i], sws[i], 16)
         assert torch.equal(dxs[i], dx) and torch.equal(dws[i], dw)
-    # grouped-query shapes: k / v narrower than q -> separate launches, same results
-    wk = rand_fp8((H // 4, H), 50, E4).to(dev)
-    outs = lin.fp8_linear_forward_grouped(x, s, [ws[0], wk], sws[:2], False, 16)
-    assert outs[1].shape == (T, H // 4) and torch.equal(outs[1], lin.fp8_linear_forward(x, s, wk, sws[1], False, 16))
+    # grouped-query shapes: k / v narrower than q -> q in a launch of its own, k and v together; same results, same order
+    wk, wv = rand_fp8((H // 4, H), 50, E4).to(dev), rand_fp8((H // 4, H), 51, E4).to(dev)
+    outs = lin.fp8_linear_forward_grouped(x, s, [ws[0], wk, wv], sws, False, 16)
+    assert outs[0].shape == (T, H) and outs[1].shape == outs[2].shape == (T, H // 4)
+    for o, w, sw in zip(outs, (ws[0], wk, wv), sws):
+        assert torch.equal(o, lin.fp8_linear_forward(x, s, w, sw, False, 16))
     # bias in the second problem only
     lib = _hip.lib()
     bias = torch.randn(H, generator=torch.Generator().manual_seed(7)).bfloat16().to(dev)

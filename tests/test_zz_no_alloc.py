@@ -80,3 +80,54 @@ def test_static_entry_point_rejects_what_it_cannot_hold(dev):
     assert L.coat_fp8_rmsnorm_backward_static(*args, 16, 4096 + 8, 16, None) == -2
     assert L.coat_fp8_rmsnorm_backward_static(*args, 0, 4096, 16, None) == 0      # empty: nothing to do
     assert L.coat_fp8_rmsnorm_backward_static(p, 0, p, 1, None, None, None, p, 1, p, p, p, 16, 4096, 16, None) == -1
+
+
+def test_static_entry_point_under_graph_capture(dev):
+    """What the entry point is for: one call recorded into a HIP graph (after a warm-up call outside the capture, which
+    performs the once-per-device lookup of the scratch array's address) and replayed on new gradients, with eager work
+    of the program between the replays; every replay bit-identical to the workspace entry point run eagerly."""
+    from coat_amd import _hip
+    L = _hip.lib()
+    M, N = 1024, 4096
+    qx, sx, w, rstd, grads = _inputs(dev, M, N, 11, 2)
+    gen = torch.Generator().manual_seed(12)
+    new_grads = [[(torch.randn(M, N, generator=gen) * (1e-2 * (r + 1))).bfloat16().to(dev) for _ in range(2)] for r in range(3)]
+    static_g = [g.clone() for g in grads]
+    dx = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    dw = torch.empty((N,), dtype=w.dtype, device=dev)
+    rows = min(512, (512 * 8192) // N)
+
+    def call_static():
+        rc = L.coat_fp8_rmsnorm_backward_static(_hip.ptr(qx), _hip.fp8(qx.dtype), _hip.ptr(sx), _hip.dt(sx), _hip.ptr(static_g[0]),
+                                                _hip.ptr(static_g[1]), None, _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd),
+                                                _hip.ptr(dx), _hip.ptr(dw), M, N, 16, _hip.stream(dev))
+        assert rc == 0, rc
+
+    def eager(gs):
+        dx0 = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        dw0 = torch.empty((N,), dtype=w.dtype, device=dev)
+        partial = torch.empty((rows, N), dtype=torch.float32, device=dev)
+        rc = L.coat_fp8_rmsnorm_backward(_hip.ptr(qx), _hip.fp8(qx.dtype), _hip.ptr(sx), _hip.dt(sx), _hip.ptr(gs[0]), _hip.ptr(gs[1]),
+                                         None, _hip.ptr(w), _hip.dt(w), _hip.ptr(rstd), _hip.ptr(dx0), _hip.ptr(dw0),
+                                         _hip.ptr(partial), rows, M, N, 16, _hip.stream(dev))
+        assert rc == 0, rc
+        return dx0, dw0
+
+    side = torch.cuda.Stream(device=dev)  # default priority
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        call_static()  # warm-up: the address lookup happens here, outside the capture
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call_static()
+    torch.cuda.synchronize(dev)
+    for gs in new_grads:
+        want_dx, want_dw = eager(gs)  # eager work (which also allocates) between the replays
+        torch.cuda.synchronize(dev)
+        for dst, src in zip(static_g, gs):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        assert torch.equal(dx, want_dx) and torch.equal(dw, want_dw)
