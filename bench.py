@@ -672,41 +672,26 @@ def cpu_baseline_rmsnorm(torch, nbytes_full):
 
 
 def cpu_baseline_layer(torch, size):
-    """The same decoder layer in fp32 torch on the host (F.rms_norm / F.linear / SDPA / F.silu, forward + backward) on one
-    sequence of 256 tokens; ms scaled by tokens to the 4 x 2048 of the GPU run (attention, 5 % of the work, scales worse)."""
-    import torch.nn.functional as F
+    """The layer as the chain of the CPU oracle's operations (oracle/layer_ref.py: the reference's call order through
+    norm, quantized projections, SiLU * up, residual adds and their backward, fp32 SDPA in between), forward + backward
+    on one sequence of 256 tokens with every host core torch uses; ms scaled by tokens to the 4 x 2048 of the GPU run
+    (attention, a few per cent of the work, scales worse; the weights' re-quantization does not scale at all)."""
+    from oracle import layer_ref
 
     H, heads, I = (4096, 32, 11008) if size == "7b" else (5120, 40, 13824)
-    S, hd = 256, H // heads
+    S = 256
     gen = torch.Generator().manual_seed(0)
-    W = {n: (torch.randn(shape, generator=gen) * 0.02).requires_grad_(True) for n, shape in
+    W = {n: (torch.randn(shape, generator=gen) * 0.02).bfloat16() for n, shape in
          (("q", (H, H)), ("k", (H, H)), ("v", (H, H)), ("o", (H, H)), ("gate", (I, H)), ("up", (I, H)), ("down", (H, I)))}
-    n1, n2 = torch.ones(H, requires_grad=True), torch.ones(H, requires_grad=True)
-    x = torch.randn(1, S, H, generator=gen)
-    gy = torch.randn(1, S, H, generator=gen) * 1e-2
-
-    def step():
-        for t in list(W.values()) + [n1, n2]:
-            t.grad = None
-        xin = x.clone().requires_grad_(True)
-        h = F.rms_norm(xin, (H,), n1, 1e-5)
-        q, k, v = (F.linear(h, W[n]).view(1, S, heads, hd).transpose(1, 2) for n in ("q", "k", "v"))
-        a = F.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(1, S, H)
-        x1 = xin + F.linear(a, W["o"])
-        h2 = F.rms_norm(x1, (H,), n2, 1e-5)
-        y = x1 + F.linear(F.silu(F.linear(h2, W["gate"])) * F.linear(h2, W["up"]), W["down"])
-        y.backward(gy)
-
-    step()
-    ts = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        step()
-        ts.append(time.perf_counter() - t0)
-    ms = _median(ts) * 1e3
+    W["norm1"], W["norm2"] = torch.ones(H).bfloat16(), torch.ones(H).bfloat16()
+    x = torch.randn(S, H, generator=gen).bfloat16()
+    gy = (torch.randn(S, H, generator=gen) * 1e-2).bfloat16()
+    t0 = time.perf_counter()
+    layer_ref.decoder_layer_step(x, gy, W, heads, 1)
+    ms = (time.perf_counter() - t0) * 1e3
     return {"value": round(ms * 8192 / S, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"fp32 torch layer of the same shape (RoPE left out), forward + backward on 1 x {S} tokens: {ms:.1f} ms, "
-                      f"median of 3 runs, scaled by 8192 / {S} tokens"}
+            "sample": f"oracle chain of the layer (oracle/layer_ref.py), forward + backward on 1 x {S} tokens: {ms:.0f} ms, "
+                      f"one run, scaled by 8192 / {S} tokens"}
 
 
 def ramp_clocks(step, seconds, torch):
