@@ -32,6 +32,7 @@ struct AdamArgs {
     float one_minus_beta1, one_minus_beta2;
     float correction1, correction2_sqrt;  // 1 - beta1^step, sqrt(1 - beta2^step), evaluated on the host
     float expand_min;
+    float inv_expand_min;  // 1 / expand_min when expand_min is a power of two (the division is then a multiplication), else 0
 };
 
 __device__ __forceinline__ float log2_hw(float x) { return __builtin_amdgcn_logf(x); }
@@ -387,11 +388,33 @@ __device__ __forceinline__ void adamw_expand_wave(void* __restrict__ params, con
     const float Mx_m = (float)((double)mx_m + 1e-30), Mn_m = (float)((double)mn_m + 1e-30);
     const float Mx_v = (float)((double)mx_v + 1e-30), Mn_v = (float)((double)mn_v + 1e-30);
     const float ratio_m = Mx_m / Mn_m, ratio_v = Mx_v / Mn_v;
-    const float cn_m = sqrtf(Mx_m) * sqrtf(Mn_m), cn_v = sqrtf(Mx_v) * sqrtf(Mn_v);
-    const float k_m = floorf((kLog2RatioUpperBound / log2_hw(ratio_m)) * A.expand_min) / A.expand_min;
-    const float k_v = floorf((kLog2RatioUpperBound / log2_hw(ratio_v)) * A.expand_min) / A.expand_min;
-    const float snew_m = pow_full(Mx_m / cn_m, k_m) / 448.0f;
-    const float snew_v = pow_full(Mx_v / cn_v, k_v) / 448.0f;
+    // Group constants.  The same IEEE results with fewer instructions where the operands allow it (decided once per wave;
+    // these constants are a quarter of the kernel's instructions, and every lane of a group computes them):
+    //   sqrtf          hardware approximation + one correction step (sqrt_cr_normal: normal operands >= 2^-96)
+    //   x / expand_min multiplication by the reciprocal when expand_min is a power of two (exact)
+    //   x / 448        reciprocal constant + two FMAs (div_by_fp8max: finite x with a normal quotient)
+    float cn_m, cn_v, k_m, k_v;
+    const bool easy = __all(Mn_m >= 0x1p-96f && Mn_v >= 0x1p-96f && Mx_m < INFINITY && Mx_v < INFINITY) && A.inv_expand_min > 0.0f;
+    if (easy) {
+        cn_m = sqrt_cr_normal(Mx_m) * sqrt_cr_normal(Mn_m);
+        cn_v = sqrt_cr_normal(Mx_v) * sqrt_cr_normal(Mn_v);
+        k_m = floorf((kLog2RatioUpperBound / log2_hw(ratio_m)) * A.expand_min) * A.inv_expand_min;
+        k_v = floorf((kLog2RatioUpperBound / log2_hw(ratio_v)) * A.expand_min) * A.inv_expand_min;
+    } else {
+        cn_m = sqrtf(Mx_m) * sqrtf(Mn_m);
+        cn_v = sqrtf(Mx_v) * sqrtf(Mn_v);
+        k_m = floorf((kLog2RatioUpperBound / log2_hw(ratio_m)) * A.expand_min) / A.expand_min;
+        k_v = floorf((kLog2RatioUpperBound / log2_hw(ratio_v)) * A.expand_min) / A.expand_min;
+    }
+    const float pw_m = pow_full(Mx_m / cn_m, k_m), pw_v = pow_full(Mx_v / cn_v, k_v);
+    float snew_m, snew_v;
+    if (__all(pw_m >= 0x1p-100f && pw_m < INFINITY && pw_v >= 0x1p-100f && pw_v < INFINITY)) {
+        snew_m = div_by_fp8max<kE4M3>(pw_m);
+        snew_v = div_by_fp8max<kE4M3>(pw_v);
+    } else {
+        snew_m = pw_m / 448.0f;
+        snew_v = pw_v / 448.0f;
+    }
     const bool odd_out = __builtin_amdgcn_ballot_w64(!(k_m > 0.0f && k_m < INFINITY) || !(k_v > 0.0f && k_v < INFINITY) ||
                                                      !(snew_m > 0.0f && snew_m < INFINITY) ||
                                                      !(snew_v > 0.0f && snew_v < INFINITY)) != 0;
@@ -470,6 +493,7 @@ static int adamw_common(void* params, const void* grads, int p_dtype, void* exp_
     A.correction1 = 1.0f - (float)pow((double)beta1, (double)(float)step);
     A.correction2_sqrt = sqrtf(1.0f - (float)pow((double)beta2, (double)(float)step));
     A.expand_min = (float)expand_min;
+    A.inv_expand_min = (expand_min > 0 && (expand_min & (expand_min - 1)) == 0) ? 1.0f / (float)expand_min : 0.0f;
     const int64_t waves = (ngroups + 7) / 8;
     const int64_t blocks = (waves + 3) / 4;
     hipStream_t st = (hipStream_t)stream;
