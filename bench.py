@@ -386,7 +386,7 @@ def make_olmo_workload(dev, torch):
     gemm_flops = 3 * 2 * B * S * (4 * D * D + D * hidden + D * hidden // 2)
     return step_fp8, step_bf16, gemm_flops, {
         "workload": f"CoatOLMoSequentialBlock fwd+bwd, OLMo-7B shape (d_model {D}, heads {heads}, mlp_hidden_size {hidden}), "
-                    f"batch {B} x seq {S}, FP8 linears/activations/LayerNorm, bf16 SDPA attention",
+                    f"batch {B} x seq {S}, FP8 linears/activations/LayerNorm, bf16 attention (this library's forward kernel, torch's backward)",
         "tokens": B * S, "gemm_flops": gemm_flops}
 
 
@@ -497,7 +497,7 @@ def make_layer_workload(dev, torch, size, cache_weights=False):
     gemm_flops = 3 * 2 * B * S * (4 * H * H + 3 * H * I)
     return step_fp8, step_bf16, gemm_flops, {
         "workload": f"CoatLlamaDecoderLayer fwd+bwd, Llama-2-{size.upper()} shape (H {H}, heads {heads}, I {I}), "
-                    f"batch {B} x seq {S}, FP8 linears/activations/norms, bf16 SDPA attention"
+                    f"batch {B} x seq {S}, FP8 linears/activations/norms, bf16 attention (this library's forward kernel, torch's backward)"
                     + (", FP8 weights cached across micro-batches" if cache_weights else ""),
         "tokens": B * S, "gemm_flops": gemm_flops}
 
@@ -805,7 +805,26 @@ def measure_layer(name, args, dev, torch, cpu):
     return rec
 
 
+def make_attention_workload(dev, torch):
+    """The bf16 attention forward of the 7B decoder layer: batch 4, 32 heads, 2048 tokens, head dimension 128, causal; q / k / v
+    as the projections leave them ([B, S, H, 128] seen as [B, H, S, 128]).  One step = one launch of the MFMA kernel.  FLOPs: the two products over the visible (lower-triangular) half, 2 * 2 * B * H * S^2 / 2 * 128."""
+    from coat_amd.models._attention import attention_forward
+
+    B, H, S, D = 4, 32, 2048, 128
+    gen = torch.Generator(device=dev).manual_seed(0)
+    q, k, v = [torch.randn(B, S, H, D, generator=gen, device=dev).bfloat16().transpose(1, 2) for _ in range(3)]
+
+    def step():
+        attention_forward(q, k, v, causal=True)
+
+    return step, 2 * 2 * B * H * S * S * D // 2, {
+        "workload": f"attention forward bf16, causal, batch {B} x {H} heads x {S} tokens x head_dim {D} (k_attn_fwd)",
+        "kernel": "k_attn_fwd", "batch": B, "heads": H, "seq": S, "head_dim": D}
+
+
 def make_stream_workload(name, args, dev, torch):
+    if name == "attention":
+        return make_attention_workload(dev, torch)
     if name in ("adamw", "adamw_plain"):
         return make_adamw_workload(dev, (11008, 4096), torch, expand=name == "adamw")
     if name == "adamw_class":
@@ -830,7 +849,7 @@ def make_stream_workload(name, args, dev, torch):
 def measure_stream(name, args, dev, torch, cpu):
     """One workload whose step is a short chain of launches: K steps between two synchronisations for `value`, HIP events
     on the launch stream around the same K back-to-back launches for the average launch duration of the roofline."""
-    is_gemm = name.startswith("gemm")
+    is_gemm = name.startswith("gemm") or name == "attention"  # MFMA-bound legs: `nbytes` holds FLOPs
     step, nbytes, cfg = make_stream_workload(name, args, dev, torch)
     ramp_clocks(step, args.ramp_seconds, torch)
     for _ in range(args.warmup):
@@ -865,13 +884,13 @@ def measure_stream(name, args, dev, torch, cpu):
     ms_per_step = avg_ms if prepare else wall * 1e3 / args.steps
     value = nbytes / (ms_per_step * 1e-3) / 1e9
     achieved = nbytes / (avg_ms * 1e-3) / 1e9
-    unit, peak, bound = ("TFLOP/s", 5000.0, "mfma") if is_gemm else ("GB/s", HBM_PEAK_GBS, "hbm")
+    unit, peak, bound = ("TFLOP/s", 2500.0 if name == "attention" else 5000.0, "mfma") if is_gemm else ("GB/s", HBM_PEAK_GBS, "hbm")
     if is_gemm:  # nbytes holds FLOPs for the GEMM workloads; report TFLOP/s
         value, achieved = value / 1e3, achieved / 1e3
     traffic = MEASURED_TRAFFIC.get("adamw" if name == "adamw_class" else name) if args.shape == [4096, 4096] else None
     rec = {
         "value": round(value, 2), "unit": unit, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
-        "dtype": "fp8" if is_gemm else ("f32" if name.startswith("adamw") else "bf16"), "config": cfg,
+        "dtype": "bf16" if name == "attention" else "fp8" if is_gemm else ("f32" if name.startswith("adamw") else "bf16"), "config": cfg,
         "roofline": {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": traffic[0] if traffic else None,
                      "traffic_source": (traffic[1] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in a separate run, not this run)") if traffic else None,
@@ -886,7 +905,7 @@ def measure_stream(name, args, dev, torch, cpu):
             rec["cpu_baseline"] = cpu_baseline_adamw(torch)
         elif name in ("quantize", "quantize_transpose") and args.shape == [4096, 4096]:
             rec["cpu_baseline"] = cpu_baseline_quantize(torch, name == "quantize_transpose", nbytes)
-        elif is_gemm:
+        elif name.startswith("gemm"):
             rec["cpu_baseline"] = cpu_baseline_gemm(torch, name.split("_")[1])
         elif name == "silu_mul":
             rec["cpu_baseline"] = cpu_baseline_silu_mul(torch, nbytes)
@@ -896,7 +915,7 @@ def measure_stream(name, args, dev, torch, cpu):
 
 
 # the default run: the headline workload (BASELINE configuration 2) plus one record per remaining leg of the metric
-EXTRAS = ("quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "silu_mul", "rmsnorm", "layer_7b", "layer_13b")
+EXTRAS = ("quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad", "gemm_wgrad", "silu_mul", "rmsnorm", "attention", "layer_7b", "layer_13b")
 
 
 def main():
@@ -907,7 +926,7 @@ def main():
     ap.add_argument("--workload", default="all",
                     choices=["all", "gemm_clock", "adamw", "adamw_class", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad",
                              "gemm_wgrad", "linear", "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr",
-                             "division_transpose", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b"],
+                             "division_transpose", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b", "attention"],
                     help="all (default): the headline AdamW step as `value` plus an `extra` record for every other leg of the metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", type=int, nargs=2, default=[4096, 4096], metavar=("M", "N"),

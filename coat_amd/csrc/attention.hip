@@ -9,17 +9,19 @@
 // 32 w .. 32 w + 31, all 128 dimensions.  Keys are walked in tiles of 64.  Both products are computed transposed, so that
 // the accumulator layout of the first is the operand layout of the second:
 //   S^T[key, query] = K Q^T      A = K tile rows (a lane reads 16 contiguous bytes of a key's row), B = Q (registers)
-//   O^T[dim, query] = V^T P^T    A = V^T tile rows (16 contiguous bytes of a dimension's row of keys), B = P^T
+//   O^T[dim, query] = V^T P^T    A = V^T fragments (8 keys of one dimension per lane), B = P^T
 // In both results a lane holds one query (column lane % 32), so the running maximum, the running sum and the rescaling
 // of O are per-lane scalars; the only cross-lane step of the softmax is one swap between lane l and lane l + 32, which
 // hold the two halves of a query's keys.  P^T needs no layout change either: the contraction over keys may run in any
 // order as long as both operands agree, and one v_permlane32_swap per two packed registers puts keys 16 j + 8 h .. + 7 into
-// half-wave h, which is what a 16-byte read of a V^T row delivers.
-// V^T (keys contiguous) does not exist in the projections' output: k_attn_transpose_v writes it once per call,
-// [batch, kv_heads, 128, seq padded to 64].
-// K and V^T tiles go from global memory into a two-stage LDS ring without passing through registers
-// (buffer_load_dwordx4 ... lds); 16-byte chunks are XOR-swizzled with the row so that the fragment reads are free of
-// bank conflicts.  Blocks are ordered so that the blocks of one (batch, head) run on one XCD (one L2) one after the other,
+// half-wave h, which is what two transposing reads of the V tile deliver.
+// V^T (keys contiguous) does not exist in memory, and is never formed: the V tile lies in LDS as it lies in memory
+// (a key's 128 dimensions per row) and its fragments are read with ds_read_b64_tr_b16, the transposing LDS read of
+// gfx950: 16 lanes point at 4 keys x 16 dimensions (lane i at key i / 4, dimensions 4 (i % 4) .. + 3) and lane j receives the
+// 4 keys of dimension j.
+// K and V tiles go from global memory into a two-stage LDS ring without passing through registers
+// (buffer_load_dwordx4 ... lds); 16-byte chunks (K) and 32-byte pieces (V) are XOR-swizzled with the row so that the
+// fragment reads are free of bank conflicts.  Blocks are ordered so that the blocks of one (batch, head) run on one XCD (one L2) one after the other,
 // longest first (under the causal mask a block's work grows with its position).
 #include <math.h>
 
@@ -36,18 +38,18 @@ typedef __attribute__((address_space(3))) void* lds_ptr3_t;
 constexpr int kHeadDim = 128;
 constexpr int kBlockQ = 128, kTileK = 64;
 constexpr int kKTileBytes = kTileK * kHeadDim * 2;   // 64 keys x 256 bytes
-constexpr int kVTileBytes = kHeadDim * kTileK * 2;   // 128 dims x 128 bytes
+constexpr int kVTileBytes = kTileK * kHeadDim * 2;   // 64 keys x 256 bytes
 constexpr int kStageBytes = kKTileBytes + kVTileBytes;
 constexpr int kAttnLdsBytes = 2 * kStageBytes;       // 64 KiB: two blocks per CU
 
 struct AttnArgs {
     const uint16_t* q;
     const uint16_t* k;
-    const uint16_t* vt;   // [batch, kv_heads, 128, s_pad]
+    const uint16_t* v;
     uint16_t* out;
     float* lse;           // [batch, heads, seq], natural logarithm
-    int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, o_sb, o_ss, o_sh;  // element strides: batch, token, head
-    int batch, heads, kv_heads, seq, s_pad;
+    int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh;  // element strides: batch, token, head
+    int batch, heads, kv_heads, seq;
     float scale_log2e;    // softmax scale * log2(e)
 };
 
@@ -92,37 +94,50 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
 
     // ---- tile loads (global -> LDS)
     const uint16_t* kbase = A.k + b * A.k_sb + kvh * A.k_sh;
-    const uint16_t* vbase = A.vt + ((int64_t)(b * A.kv_heads + kvh) * kHeadDim) * A.s_pad;
+    const uint16_t* vbase = A.v + b * A.v_sb + kvh * A.v_sh;
     const v4i_t k_rsrc = attn_rsrc(kbase, (uint32_t)(((int64_t)(A.seq - 1) * A.k_ss + kHeadDim) * 2));
-    const v4i_t v_rsrc = attn_rsrc(vbase, (uint32_t)((int64_t)kHeadDim * A.s_pad * 2));
+    const v4i_t v_rsrc = attn_rsrc(vbase, (uint32_t)(((int64_t)(A.seq - 1) * A.v_ss + kHeadDim) * 2));
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr3_t)lds;
-    // K: one instruction = 4 rows of 256 bytes; lane i fills position i % 16 of row i / 16 with the chunk that belongs there
-    // V^T: one instruction = 8 rows of 128 bytes; lane i fills position i % 8 of row i / 8
+    // one instruction = 4 rows (keys) of 256 bytes; lane i fills position i % 16 of row i / 16 with the chunk that belongs
+    // there: K position p holds chunk p ^ (row & 15); V position p holds chunk ((p / 2) ^ (row & 7)) * 2 + p % 2 (32-byte
+    // pieces stay whole: a transposing read takes 32 contiguous bytes of each of 4 keys).  Keys past the end read zeros.
     int k_off[4], v_off[4];
 #pragma unroll
     for (int x = 0; x < 4; x++) {
-        const int krow = 4 * (4 * wave + x) + (lane >> 4);
-        k_off[x] = krow * (int)(A.k_ss * 2) + (((lane & 15) ^ (krow & 15)) << 4);
-        const int vrow = 8 * (4 * wave + x) + (lane >> 3);
-        v_off[x] = vrow * (A.s_pad * 2) + (((lane & 7) ^ ((vrow >> 1) & 7)) << 4);
+        const int row = 4 * (4 * wave + x) + (lane >> 4), p = lane & 15;
+        k_off[x] = row * (int)(A.k_ss * 2) + ((p ^ (row & 15)) << 4);
+        v_off[x] = row * (int)(A.v_ss * 2) + ((((((p >> 1) ^ (row & 7)) << 1) | (p & 1))) << 4);
     }
     auto issue_tile = [&](int t, int stage) {
         const uint32_t kdst = lds_base + stage * kStageBytes + (4 * wave) * 1024;
         const uint32_t vdst = kdst + kKTileBytes;
-        const int kt_off = t * kTileK * (int)(A.k_ss * 2), vt_off = t * kTileK * 2;
+        const int kt_off = t * kTileK * (int)(A.k_ss * 2), vt_off = t * kTileK * (int)(A.v_ss * 2);
 #pragma unroll
         for (int x = 0; x < 4; x++) attn_lds_dma16(k_rsrc, kdst + x * 1024, k_off[x] + kt_off);
 #pragma unroll
         for (int x = 0; x < 4; x++) attn_lds_dma16(v_rsrc, vdst + x * 1024, v_off[x] + vt_off);
     };
-    // fragment addresses inside a stage: K row l32 (+ 32 kt), chunk 2 c + h32; V^T row l32 (+ 32 dt), chunk 2 j + h32
+    // K fragment (A operand of S^T): row l32 (+ 32 kt), chunk 2 c + h32
     auto k_frag = [&](int stage, int kt, int c) -> v8bf {
         const int row = 32 * kt + l32;
         return *(const v8bf*)(lds + stage * kStageBytes + row * 256 + (((2 * c + h32) ^ (row & 15)) << 4));
     };
+    // V^T fragment (A operand of O^T): dimension 32 dt + l32, keys 16 j + 8 h32 .. + 7, through two transposing reads.
+    // Within a group of 16 lanes, lane i points at key (16 j + 8 h32) + i / 4 (+ 4 for the second read), dimensions
+    // d0 + 4 (i % 4) .. + 3 with d0 = 32 dt + 16 * (group % 2); lane i then receives dimension d0 + i of 4 consecutive keys.
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4s* lds_v4s_ptr;
+    const int tr_i = lane & 15, tr_dim = 16 * ((lane >> 4) & 1) + 4 * (tr_i & 3), tr_key = 8 * h32 + (tr_i >> 2);
     auto v_frag = [&](int stage, int dt, int j) -> v8bf {
-        const int row = 32 * dt + l32;
-        return *(const v8bf*)(lds + stage * kStageBytes + kKTileBytes + row * 128 + (((2 * j + h32) ^ ((row >> 1) & 7)) << 4));
+        const int dim = 32 * dt + tr_dim, key = 16 * j + tr_key;
+        const uint8_t* base = lds + stage * kStageBytes + kKTileBytes + ((dim & 15) << 1);
+        const uint8_t* a0 = base + key * 256 + (((dim >> 4) ^ (key & 7)) << 5);
+        const uint8_t* a1 = base + (key + 4) * 256 + (((dim >> 4) ^ ((key + 4) & 7)) << 5);
+        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a0);
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a1);
+        typedef short v8s __attribute__((ext_vector_type(8)));
+        const v8s both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(v8bf, both);
     };
 
     v16f o_acc[4];
@@ -231,72 +246,29 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
     }
 }
 
-// v [batch, seq, kv_heads, 128] (strides given) -> vt [batch, kv_heads, 128, s_pad], columns seq .. s_pad - 1 zero.
-// One block = 64 keys x 128 dimensions of one (batch, head), through LDS.
-__global__ __launch_bounds__(256) void k_attn_transpose_v(const uint16_t* __restrict__ v, uint16_t* __restrict__ vt, int64_t v_sb,
-                                                          int64_t v_ss, int64_t v_sh, int kv_heads, int seq, int s_pad) {
-    __shared__ uint16_t tile[kTileK][kHeadDim + 2];
-    const int t = blockIdx.x, bh = blockIdx.y;
-    const int b = bh / kv_heads, hd = bh % kv_heads;
-    const uint16_t* src = v + b * v_sb + hd * v_sh;
-    // 64 rows x 16 chunks of 16 bytes: four per thread
-#pragma unroll
-    for (int it = 0; it < 4; it++) {
-        const int job = threadIdx.x + 256 * it, row = job >> 4, ch = job & 15;
-        const int key = t * kTileK + row;
-        uint4 val = make_uint4(0, 0, 0, 0);
-        if (key < seq) val = *(const uint4*)(src + (int64_t)key * v_ss + ch * 8);
-        uint32_t* dst = (uint32_t*)&tile[row][ch * 8];  // rows are 260 bytes apart: 4-byte aligned
-        dst[0] = val.x; dst[1] = val.y; dst[2] = val.z; dst[3] = val.w;
-    }
-    __syncthreads();
-    // 128 dims x 8 chunks of 8 keys: four per thread
-    uint16_t* dstb = vt + ((int64_t)bh * kHeadDim) * s_pad + t * kTileK;
-#pragma unroll
-    for (int it = 0; it < 4; it++) {
-        const int job = threadIdx.x + 256 * it, dim = job >> 3, kc = job & 7;
-        uint32_t w[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) w[e] = (uint32_t)tile[kc * 8 + 2 * e][dim] | ((uint32_t)tile[kc * 8 + 2 * e + 1][dim] << 16);
-        *(uint4*)(dstb + (int64_t)dim * s_pad + kc * 8) = make_uint4(w[0], w[1], w[2], w[3]);
-    }
-}
-
 }  // namespace coat
 
 using namespace coat;
 
-extern "C" int coat_attention_transpose_v(const void* v, void* vt, int64_t batch, int64_t seq, int64_t kv_heads, int64_t head_dim,
-                                          int64_t v_sb, int64_t v_ss, int64_t v_sh, int64_t s_pad, void* stream) {
-    if (batch < 0 || seq < 0 || kv_heads <= 0) return COAT_EINVAL;
-    if (head_dim != kHeadDim || s_pad % kTileK != 0 || s_pad < seq) return COAT_ESHAPE;
-    if (batch * seq == 0) return COAT_OK;
-    if (!v || !vt) return COAT_EINVAL;
-    if (!coat_aligned16(v) || !coat_aligned16(vt) || v_ss % 8 != 0 || v_sh % 8 != 0 || v_sb % 8 != 0) return COAT_EALIGN;
-    if (batch * kv_heads >= 65536 || s_pad / kTileK >= ((int64_t)1 << 31)) return COAT_ESHAPE;
-    hipLaunchKernelGGL(k_attn_transpose_v, dim3((unsigned)(s_pad / kTileK), (unsigned)(batch * kv_heads)), dim3(256), 0,
-                       (hipStream_t)stream, (const uint16_t*)v, (uint16_t*)vt, v_sb, v_ss, v_sh, (int)kv_heads, (int)seq, (int)s_pad);
-    return coat_launch_status();
-}
-
-extern "C" int coat_attention_forward_bf16(const void* q, const void* k, const void* vt, void* out, float* lse, int64_t batch,
+extern "C" int coat_attention_forward_bf16(const void* q, const void* k, const void* v, void* out, float* lse, int64_t batch,
                                            int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int64_t q_sb,
-                                           int64_t q_ss, int64_t q_sh, int64_t k_sb, int64_t k_ss, int64_t k_sh, int64_t o_sb,
-                                           int64_t o_ss, int64_t o_sh, int64_t s_pad, float scale, int causal, void* stream) {
+                                           int64_t q_ss, int64_t q_sh, int64_t k_sb, int64_t k_ss, int64_t k_sh, int64_t v_sb,
+                                           int64_t v_ss, int64_t v_sh, int64_t o_sb, int64_t o_ss, int64_t o_sh, float scale,
+                                           int causal, void* stream) {
     if (batch < 0 || seq < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0) return COAT_EINVAL;
-    if (head_dim != kHeadDim || s_pad % kTileK != 0 || s_pad < seq) return COAT_ESHAPE;
+    if (head_dim != kHeadDim) return COAT_ESHAPE;
     if (batch * seq == 0) return COAT_OK;
-    if (!q || !k || !vt || !out) return COAT_EINVAL;
-    if (!coat_aligned16(q) || !coat_aligned16(k) || !coat_aligned16(vt) || !coat_aligned16(out)) return COAT_EALIGN;
-    for (int64_t s : {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, o_sb, o_ss, o_sh})
+    if (!q || !k || !v || !out) return COAT_EINVAL;
+    if (!coat_aligned16(q) || !coat_aligned16(k) || !coat_aligned16(v) || !coat_aligned16(out)) return COAT_EALIGN;
+    for (int64_t s : {q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh})
         if (s % 8 != 0 || s < 0) return COAT_EALIGN;
-    // 32-bit byte offsets inside one (batch, head) of k and of vt
-    if (seq * k_ss * 2 >= ((int64_t)1 << 31) || (int64_t)kHeadDim * s_pad * 2 >= ((int64_t)1 << 31)) return COAT_ESHAPE;
+    // 32-bit byte offsets inside one (batch, head) of k and of v
+    if ((seq + kTileK) * k_ss * 2 >= ((int64_t)1 << 31) || (seq + kTileK) * v_ss * 2 >= ((int64_t)1 << 31)) return COAT_ESHAPE;
     AttnArgs A;
-    A.q = (const uint16_t*)q; A.k = (const uint16_t*)k; A.vt = (const uint16_t*)vt; A.out = (uint16_t*)out; A.lse = lse;
+    A.q = (const uint16_t*)q; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v; A.out = (uint16_t*)out; A.lse = lse;
     A.q_sb = q_sb; A.q_ss = q_ss; A.q_sh = q_sh; A.k_sb = k_sb; A.k_ss = k_ss; A.k_sh = k_sh;
-    A.o_sb = o_sb; A.o_ss = o_ss; A.o_sh = o_sh;
-    A.batch = (int)batch; A.heads = (int)heads; A.kv_heads = (int)kv_heads; A.seq = (int)seq; A.s_pad = (int)s_pad;
+    A.v_sb = v_sb; A.v_ss = v_ss; A.v_sh = v_sh; A.o_sb = o_sb; A.o_ss = o_ss; A.o_sh = o_sh;
+    A.batch = (int)batch; A.heads = (int)heads; A.kv_heads = (int)kv_heads; A.seq = (int)seq;
     A.scale_log2e = scale * 1.4426950408889634f;
     const int64_t nqb = (seq + kBlockQ - 1) / kBlockQ;
     const int64_t grid = ((batch * heads + 7) / 8) * 8 * nqb;

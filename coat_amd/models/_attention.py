@@ -2,7 +2,7 @@
 
 The reference calls the flash-attn library here (coat/models/coat_llama.py:960-971 through transformers).  The forward
 of the case the layers use (bf16, causal, no mask, no dropout, head dimension 128) is this library's MFMA kernel
-(``coat_attention_forward_bf16``: online softmax, K and V^T tiles through LDS); its backward is torch's
+(``coat_attention_forward_bf16``: online softmax, K and V tiles through LDS); its backward is torch's
 memory-efficient attention backward, which takes the forward's output and log-sum-exp.  Everything else goes to
 ``torch.nn.functional.scaled_dot_product_attention`` with the backend order that is fastest on MI355X: on this ROCm
 build torch picks its "flash" backend by default, while for the layers' shapes (batch 4, 32 heads, 2048 tokens) its
@@ -32,16 +32,12 @@ def attention_forward(q, k, v, causal=True, scale=None, need_lse=True):
     for t in (q, k, v):
         if t.stride(3) != 1 or any(s % 8 for s in t.stride()[:3]) or t.data_ptr() % 16:
             raise ValueError("attention_forward: the head dimension must be contiguous and rows 16-byte aligned")
-    s_pad = (S + 63) // 64 * 64
     lib, st = _hip.lib(), _hip.stream(q.device)
-    vt = torch.empty((B, Hkv, D, s_pad), dtype=torch.bfloat16, device=q.device)
-    _hip.check(lib.coat_attention_transpose_v(_hip.ptr(v), _hip.ptr(vt), B, S, Hkv, D, *_strides_bshd(v), s_pad, st),
-               "attention transpose_v")
     out = torch.empty((B, S, H, D), dtype=torch.bfloat16, device=q.device).transpose(1, 2)
     lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device) if need_lse else None
-    _hip.check(lib.coat_attention_forward_bf16(_hip.ptr(q), _hip.ptr(k), _hip.ptr(vt), _hip.ptr(out), _hip.ptr(lse), B, H, Hkv, S, D,
-                                               *_strides_bshd(q), *_strides_bshd(k), *_strides_bshd(out), s_pad, scale,
-                                               1 if causal else 0, st), "attention forward")
+    _hip.check(lib.coat_attention_forward_bf16(_hip.ptr(q), _hip.ptr(k), _hip.ptr(v), _hip.ptr(out), _hip.ptr(lse), B, H, Hkv, S, D,
+                                               *_strides_bshd(q), *_strides_bshd(k), *_strides_bshd(v), *_strides_bshd(out),
+                                               scale, 1 if causal else 0, st), "attention forward")
     return out, lse
 
 

@@ -46,7 +46,7 @@ enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.f
 #define COAT_MAX_WORDS (COAT_MAX_SLOTS * COAT_MAX_SLOT_STRIDE)
 
 /* Bumped whenever an entry point's argument list or the size of a buffer it writes changes (2: every s_max / amax
- * argument became COAT_MAX_WORDS words; 3: coat_fp8_gemm_residual, coat_fp8_rmsnorm_backward_add and the attention entry points added,
+ * argument became COAT_MAX_WORDS words; 3: coat_fp8_gemm_residual, coat_fp8_rmsnorm_backward_add and coat_attention_forward_bf16 added,
  * coat_hbm_probe removed).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
  * loads the library. */
 #define COAT_ABI_VERSION 3
@@ -263,19 +263,16 @@ int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* si
 /* ---- bf16 attention (forward) ------------------------------------------------------------------------
  * The attention between the FP8 projections: the reference calls the flash-attn library here
  * (coat/models/coat_llama.py:960-971, used by LlamaAttentionWithoutLinear :981-1074).
- * out = softmax(q k^T * scale (+ causal mask)) v per (batch, head); q, k, out bf16 [batch, seq, heads, 128] addressed
+ * out = softmax(q k^T * scale (+ causal mask)) v per (batch, head); q, k, v, out bf16 [batch, seq, heads, 128] addressed
  * through element strides (batch, token, head; the head dimension is contiguous; all strides multiples of 8), so the
- * projections' outputs are used where they lie.  k has kv_heads heads (heads % kv_heads == 0).  vt is v transposed per
- * head, bf16 [batch, kv_heads, 128, s_pad] with s_pad = seq rounded up to 64 and zeros in the padding: written by
- * coat_attention_transpose_v from v [batch, seq, kv_heads, 128] (strides v_sb, v_ss, v_sh).  lse (may be NULL): fp32
- * [batch, heads, seq], natural logarithm of each query's sum of exponentials, as backward kernels expect it.
+ * projections' outputs are used where they lie.  k and v have kv_heads heads (heads % kv_heads == 0).  lse (may be
+ * NULL): fp32 [batch, heads, seq], natural logarithm of each query's sum of exponentials, as backward kernels expect it.
  * head_dim must be 128. */
-int coat_attention_transpose_v(const void* v, void* vt, int64_t batch, int64_t seq, int64_t kv_heads, int64_t head_dim,
-                               int64_t v_sb, int64_t v_ss, int64_t v_sh, int64_t s_pad, void* stream);
-int coat_attention_forward_bf16(const void* q, const void* k, const void* vt, void* out, float* lse, int64_t batch,
+int coat_attention_forward_bf16(const void* q, const void* k, const void* v, void* out, float* lse, int64_t batch,
                                 int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int64_t q_sb, int64_t q_ss,
-                                int64_t q_sh, int64_t k_sb, int64_t k_ss, int64_t k_sh, int64_t o_sb, int64_t o_ss,
-                                int64_t o_sh, int64_t s_pad, float scale, int causal, void* stream);
+                                int64_t q_sh, int64_t k_sb, int64_t k_ss, int64_t k_sh, int64_t v_sb, int64_t v_ss,
+                                int64_t v_sh, int64_t o_sb, int64_t o_ss, int64_t o_sh, float scale, int causal,
+                                void* stream);
 
 /* ---- GEMM -------------------------------------------------------------------------------------------
  * rq/linear.py:172 fp8matmul (kernel :61-169): C[M,N] = (A[M,K] . B[N,K]^T) * (float(*scale_a) * float(*scale_b))
