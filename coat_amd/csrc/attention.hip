@@ -145,7 +145,15 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o_acc[dt][r] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;  // running maximum (log2 domain) and this lane's part of the running sum
+    // Softmax state.  m_ref: the reference maximum of this lane's query, in raw score units; every exponent is taken
+    // relative to it, and it is raised (and the accumulators rescaled, for the whole wave) when a tile's maximum exceeds it
+    // by more than kLazy log2 units after scaling.  With kLazy = 0 the largest probability of a row is exactly 1, as in the
+    // textbook recurrence; a threshold of 8 rescales a few times per block instead of once per tile and was 4 % faster at
+    // 4 x 32 x 2048, but then the largest probabilities are rounded to bf16 like all the others and rows with few keys lose
+    // a bit (max |out - ref| 1.7e-2 instead of 0.8e-2 on unit-variance values), so it is not used.
+    constexpr float kLazy = 0.0f;
+    float m_ref = -INFINITY, l_run = 0.0f;
+    const float c2 = A.scale_log2e;
 
     issue_tile(0, 0);
     for (int t = 0; t < nsteps; t++) {
@@ -168,46 +176,49 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
             for (int c = 0; c < 8; c++)
                 s_acc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(stage, kt, c), qf[c], s_acc[kt], 0, 0, 0);
         }
-        // ---- scale, mask, running maximum
+        // ---- mask (edge tiles only) and the tile's maximum per query, on the raw scores (the scale is positive)
         const bool edge = (CAUSAL && key0 + kTileK - 1 > q0 + wave * 32) || key0 + kTileK > A.seq;  // wave-uniform
-        float mx = -INFINITY;
+        if (edge) {
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+            for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                float s = s_acc[kt][r] * A.scale_log2e;
-                if (edge) {
+                for (int r = 0; r < 16; r++) {
                     const int key = key0 + 32 * kt + 8 * (r >> 2) + 4 * h32 + (r & 3);
-                    if ((CAUSAL && key > my_q) || key >= A.seq) s = -INFINITY;
+                    if ((CAUSAL && key > my_q) || key >= A.seq) s_acc[kt][r] = -INFINITY;
                 }
-                s_acc[kt][r] = s;
-                mx = fmaxf(mx, s);
-            }
+        }
+        float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
+#pragma unroll
+        for (int r = 1; r < 16; r++) mx = fmaxf(mx, fmaxf(s_acc[0][r], s_acc[1][r]));
         {
             const auto sw = __builtin_amdgcn_permlane32_swap(f2u(mx), f2u(mx), false, false);
             mx = fmaxf(u2f(sw[0]), u2f(sw[1]));
         }
-        const float m_new = fmaxf(m_run, mx);  // finite: key 0 is visible to every query
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        // ---- P = exp2(S - m), packed to bf16 as the B operand of O^T = V^T P^T
-        float psum = 0.0f;
-        uint32_t pk[2][8];
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s_acc[kt][r] - m_new), p1 = __builtin_amdgcn_exp2f(s_acc[kt][r + 1] - m_new);
-                psum += p0 + p1;
-                pk[kt][r >> 1] = pack_bf16x2(p0, p1);
-            }
-        l_run = l_run * alpha + psum;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        // raise the reference where the tile exceeds it by more than kLazy (always on the first tile, from -inf)
+        if (__builtin_amdgcn_ballot_w64((mx - m_ref) * c2 > kLazy) != 0) {
+            const float m_new = fmaxf(m_ref, mx);  // finite: key 0 is visible to every query
+            const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * c2);
+            m_ref = m_new;
+            l_run *= alpha;
 #pragma unroll
             for (int dt = 0; dt < 4; dt++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) o_acc[dt][r] *= alpha;
         }
+        // ---- P = exp2(S c - m c), packed to bf16 as the B operand of O^T = V^T P^T
+        const float mc = -m_ref * c2;
+        uint32_t pk[2][8];
+        float ps0 = 0.0f, ps1 = 0.0f;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(s_acc[kt][r], c2, mc)), p1 = __builtin_amdgcn_exp2f(fmaf(s_acc[kt][r + 1], c2, mc));
+                ps0 += p0;
+                ps1 += p1;
+                pk[kt][r >> 1] = pack_bf16x2(p0, p1);
+            }
+        l_run += ps0 + ps1;
         // ---- O^T += V^T P^T, 16 keys per instruction: chunk j = 2 kt + u takes accumulator registers 8 u .. 8 u + 7
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
@@ -242,7 +253,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
                     make_uint2(pack_bf16x2(o[4 * g] * inv_l, o[4 * g + 1] * inv_l), pack_bf16x2(o[4 * g + 2] * inv_l, o[4 * g + 3] * inv_l));
             }
         if (h32 == 0 && A.lse)
-            A.lse[((int64_t)b * A.heads + head) * A.seq + my_q] = (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
+            A.lse[((int64_t)b * A.heads + head) * A.seq + my_q] = (m_ref * c2 + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
     }
 }
 
