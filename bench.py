@@ -306,7 +306,7 @@ class Bf16DecoderLayer:
 
     def __call__(self, x):
         import torch.nn.functional as F
-        from coat_amd.models._attention import sdpa
+        from coat_amd.models._attention import torch_sdpa as sdpa  # torch's fastest backend here, forward and backward
         from coat_amd.models.coat_llama import fused_rotary
         p, torch = self.p, self.torch
         B, S, H = x.shape
@@ -333,7 +333,7 @@ class Bf16OLMoBlock:
 
     def __call__(self, x):
         import torch.nn.functional as F
-        from coat_amd.models._attention import sdpa
+        from coat_amd.models._attention import torch_sdpa as sdpa  # torch's fastest backend here, forward and backward
         from coat_amd.models.coat_llama import fused_rotary
         p = self.p
         B, S, D = x.shape

@@ -66,10 +66,16 @@ def _own_kernel_applies(q, k, v, attn_mask, dropout_p, is_causal):
                                                    for t in (q, k, v)))
 
 
-def sdpa(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False):
+def torch_sdpa(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False):
+    """torch's own attention, forward and backward, with the backend order above (what the layers used before this
+    library had a forward kernel, and what a plain bf16 torch layer uses)."""
     if not q.is_cuda:
         return F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal)
-    if _own_kernel_applies(q, k, v, attn_mask, dropout_p, is_causal):
-        return _CausalAttention.apply(q, k, v)
     with sdpa_kernel(BACKEND_PRIORITY, set_priority=True):
         return F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal)
+
+
+def sdpa(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False):
+    if _own_kernel_applies(q, k, v, attn_mask, dropout_p, is_causal):
+        return _CausalAttention.apply(q, k, v)
+    return torch_sdpa(q, k, v, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal)
