@@ -60,9 +60,9 @@ SIGNATURES = {
     "coat_fp8_silu_mul_forward": [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i64, _i64, _vp],
     "coat_fp8_silu_mul_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _i64,
                                    _i64, _i64, _vp],
-    "coat_rope_bf16": [_vp, _vp, _vp, _vp, _i64, _f, _vp, _i64, _i, _i, _i, _i, _i64, _i64, _vp],
+    "coat_rope_bf16": [_vp, _vp, _vp, _vp, _i64, _f, _vp, _i64, _i, _i, _i, _i, _i64, _i64, _vp, _i, _vp],
     "coat_attention_forward_bf16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
-                                    _i64, _i64, _i64, _i64, _i64, _f, _i, _vp],
+                                    _i64, _i64, _i64, _i64, _i64, _f, _i, _vp, _i, _vp],
     "coat_fp8_gemm": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _i, _vp],
     "coat_fp8_gemm_residual": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _vp],
     "coat_fp8_gemm_grouped": [_i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i64, _i64, _i64, _i, _vp],

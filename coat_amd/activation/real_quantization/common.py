@@ -78,6 +78,26 @@ def new_max(device):
     return buf[i * _hip.MAX_WORDS:(i + 1) * _hip.MAX_WORDS]
 
 
+def tag_scale_max(t, buf, fp8type):
+    """Producer side of a hand-over: ``buf`` (a ``new_max`` buffer) holds the maximum of the fp32 group scales of the
+    bf16 tensor ``t`` for the FP8 format ``fp8type``, merged by the kernel that wrote ``t`` (the RoPE backward, the
+    attention forward).  The tag travels with the tensor object, through the autograd engine too."""
+    t._coat_scale_max = (buf, fp8type, t._version)
+    return t
+
+
+def known_scale_max(t, fp8type):
+    """Consumer side: the tagged buffer if ``t`` still is the tensor its producer wrote (same object, not modified in
+    place since, same format), else None, and the caller runs its own scale pass."""
+    tag = getattr(t, "_coat_scale_max", None)
+    if tag is None:
+        return None
+    buf, kind, version = tag
+    if kind != fp8type or version != t._version or buf.device != t.device or t.dtype != torch.bfloat16:
+        return None
+    return buf
+
+
 def scale_max(s):
     """``s.max()`` for a tensor of (non-negative) scales, as a 0-dim tensor of its dtype: the scale with which a tensor
     quantized per tensor was divided is the maximum of the per-group scale tensor that travels with it (reference

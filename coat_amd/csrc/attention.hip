@@ -51,6 +51,8 @@ struct AttnArgs {
     int64_t q_sb, q_ss, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_ss, o_sh;  // element strides: batch, token, head
     int batch, heads, kv_heads, seq;
     float scale_log2e;    // softmax scale * log2(e)
+    float* s_max;         // COAT_MAX_WORDS buffer or NULL: receives the largest group scale of the output
+    int fp8_max;          // ... for this FP8 format
 };
 
 __device__ __forceinline__ void attn_lds_dma16(v4i_t rsrc, uint32_t lds_addr, int voff) {
@@ -269,6 +271,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
         l_run = u2f(sw[0]) + u2f(sw[1]);
     }
     const float inv_l = 1.0f / l_run;
+    float amax = 0.0f;  // of the values as stored (rows beyond the sequence excluded)
     if (my_q < A.seq) {
         uint16_t* orow = A.out + b * A.o_sb + (int64_t)my_q * A.o_ss + head * A.o_sh;
 #pragma unroll
@@ -276,11 +279,18 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
 #pragma unroll
             for (int g = 0; g < 4; g++) {  // accumulator registers 4 g .. 4 g + 3: dimensions 32 dt + 8 g + 4 h .. + 3
                 const v16f& o = o_acc[dt];
-                *(uint2*)(orow + 32 * dt + 8 * g + 4 * h32) =
-                    make_uint2(pack_bf16x2(o[4 * g] * inv_l, o[4 * g + 1] * inv_l), pack_bf16x2(o[4 * g + 2] * inv_l, o[4 * g + 3] * inv_l));
+                const uint32_t w0 = pack_bf16x2(o[4 * g] * inv_l, o[4 * g + 1] * inv_l), w1 = pack_bf16x2(o[4 * g + 2] * inv_l, o[4 * g + 3] * inv_l);
+                *(uint2*)(orow + 32 * dt + 8 * g + 4 * h32) = make_uint2(w0, w1);
+                if (A.s_max) amax = fmaxf(amax, fmaxf(fmaxf(fabsf(bf16lo(w0)), fabsf(bf16hi(w0))), fmaxf(fabsf(bf16lo(w1)), fabsf(bf16hi(w1)))));
             }
         if (h32 == 0 && A.lse)
             A.lse[((int64_t)b * A.heads + head) * A.seq + my_q] = (m_ref * c2 + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
+    }
+    // the largest 1 x QB group scale of the output, for a consumer that quantizes it per tensor: one lazy atomic per wave
+    if (A.s_max) {
+        amax = cluster_max<64>(amax);
+        const float sc = A.fp8_max == kE4M3 ? group_scale<kE4M3>(amax) : group_scale<kE5M2>(amax);
+        if (lane == 0) atomic_max_nonneg(max_slot(A.s_max), sc);
     }
 }
 
@@ -292,7 +302,8 @@ extern "C" int coat_attention_forward_bf16(const void* q, const void* k, const v
                                            int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int64_t q_sb,
                                            int64_t q_ss, int64_t q_sh, int64_t k_sb, int64_t k_ss, int64_t k_sh, int64_t v_sb,
                                            int64_t v_ss, int64_t v_sh, int64_t o_sb, int64_t o_ss, int64_t o_sh, float scale,
-                                           int causal, void* stream) {
+                                           int causal, float* s_max, int fp8_max, void* stream) {
+    if (s_max && fp8_max != kE4M3 && fp8_max != kE5M2) return COAT_EINVAL;
     if (batch < 0 || seq < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0) return COAT_EINVAL;
     if (head_dim != kHeadDim) return COAT_ESHAPE;
     if (batch * seq == 0) return COAT_OK;
@@ -303,7 +314,7 @@ extern "C" int coat_attention_forward_bf16(const void* q, const void* k, const v
     // 32-bit byte offsets inside one (batch, head) of k and of v
     if ((seq + kTileK) * k_ss * 2 >= ((int64_t)1 << 31) || (seq + kTileK) * v_ss * 2 >= ((int64_t)1 << 31)) return COAT_ESHAPE;
     AttnArgs A;
-    A.q = (const uint16_t*)q; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v; A.out = (uint16_t*)out; A.lse = lse;
+    A.q = (const uint16_t*)q; A.k = (const uint16_t*)k; A.v = (const uint16_t*)v; A.out = (uint16_t*)out; A.lse = lse; A.s_max = s_max; A.fp8_max = fp8_max;
     A.q_sb = q_sb; A.q_ss = q_ss; A.q_sh = q_sh; A.k_sb = k_sb; A.k_ss = k_ss; A.k_sh = k_sh;
     A.v_sb = v_sb; A.v_ss = v_ss; A.v_sh = v_sh; A.o_sb = o_sb; A.o_ss = o_ss; A.o_sh = o_sh;
     A.batch = (int)batch; A.heads = (int)heads; A.kv_heads = (int)kv_heads; A.seq = (int)seq;

@@ -8,16 +8,23 @@
 //   cos_tab, sin_tab: fp32 [n_pos, head_dim/2];  position of a row = pos[row] if pos is given, else row % seq_len;
 //   a position outside the tables (only possible with pos) gets its angle p * theta^(-2d/head_dim) computed in the kernel
 //   y1 = x1 cos - x2 sin,  y2 = x2 cos + x1 sin   (inverse: sin -> -sin), computed in fp32, rounded once to bf16.
+// With s_max the kernel also merges (max|y| + 1e-10) / fp8max, the largest 1 x QB group scale of y for any QB (dividing
+// and rounding are monotone), into the maximum buffer: what the scale pass of fp8_quantize_pertensor(_transpose)
+// (coat/activation/real_quantization/_quantize_pertensor_transpose.py:123-139) would find on y, so a caller that quantizes
+// the rotated gradient per tensor goes straight to the division pass.
 #include "coat_device.h"
 #include "coat_host.h"
 
 namespace coat {
 
+template <int MAXKIND>  // -1: no maximum; kE4M3 / kE5M2: merge the largest group scale of y for that format into s_max
 __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab,
                                                     int64_t n_pos, float theta, const int64_t* __restrict__ pos,
                                                     int64_t rows, int seq_len, int heads, int head_dim, float sign,
-                                                    int64_t x_pitch, int64_t y_pitch) {
+                                                    int64_t x_pitch, int64_t y_pitch, float* __restrict__ s_max) {
+    __shared__ float smem[4];
+    float amax = 0.0f;
     const int half = head_dim >> 1;
     const int cpr = half >> 3;                      // 16-byte chunks per half row
     const int64_t total = rows * heads * cpr;       // one job = 8 pairs
@@ -58,7 +65,16 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
         uint16_t* dst = y + row * y_pitch + head * head_dim + c * 8;
         *(uint4*)dst = make_uint4(o1[0], o1[1], o1[2], o1[3]);
         *(uint4*)(dst + half) = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+        if (MAXKIND >= 0) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {  // of the values as stored
+                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(bf16lo(o1[k])), fabsf(bf16hi(o1[k]))),
+                                         fmaxf(fabsf(bf16lo(o2[k])), fabsf(bf16hi(o2[k])))));
+            }
+        }
     }
+    constexpr int KIND = MAXKIND < 0 ? (int)kE4M3 : MAXKIND;
+    if (MAXKIND >= 0) block_atomic_max_nonneg(s_max, group_scale<KIND>(amax), smem);
 }
 
 }  // namespace coat
@@ -67,7 +83,8 @@ using namespace coat;
 
 extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, int64_t n_pos, float theta,
                               const int64_t* pos, int64_t rows, int seq_len, int heads, int head_dim, int inverse,
-                              int64_t x_pitch, int64_t y_pitch, void* stream) {
+                              int64_t x_pitch, int64_t y_pitch, float* s_max, int fp8_max, void* stream) {
+    if (s_max && fp8_max != kE4M3 && fp8_max != kE5M2) return COAT_EINVAL;
     if (rows < 0 || heads <= 0 || head_dim <= 0 || seq_len <= 0 || n_pos <= 0 || !(theta > 0.0f)) return COAT_EINVAL;
     if (!pos && seq_len > n_pos) return COAT_ESHAPE;  // positions 0 .. seq_len-1 must all be in the tables
     if (head_dim % 16 != 0) return COAT_ESHAPE;  // 8 pairs per lane
@@ -82,7 +99,10 @@ extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, cons
     const int64_t total = rows * heads * (head_dim / 16);
     int64_t blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;
-    hipLaunchKernelGGL(k_rope_bf16, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x,
-                       (uint16_t*)y, cos_tab, sin_tab, n_pos, theta, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f, x_pitch, y_pitch);
+    if (s_max && blocks > 2048) blocks = 2048;  // one atomic per block: fewer, longer blocks
+    auto* kern = !s_max ? k_rope_bf16<-1> : fp8_max == kE4M3 ? k_rope_bf16<kE4M3> : k_rope_bf16<kE5M2>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x, (uint16_t*)y,
+                       cos_tab, sin_tab, n_pos, theta, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f, x_pitch,
+                       y_pitch, s_max);
     return coat_launch_status();
 }

@@ -21,10 +21,11 @@ def _strides_bshd(t):
     return t.stride(0), t.stride(2), t.stride(1)
 
 
-def attention_forward(q, k, v, causal=True, scale=None, need_lse=True):
+def attention_forward(q, k, v, causal=True, scale=None, need_lse=True, out_scale_max=None, out_fp8=None):
     """q [B, H, S, 128], k / v [B, Hkv, S, 128], bf16, any strides with a contiguous last dimension (the transposed views
     of [B, S, H, 128] projections are used where they lie).  Returns (out [B, H, S, 128] laid out as [B, S, H, 128],
-    lse fp32 [B, H, S] or None)."""
+    lse fp32 [B, H, S] or None).  ``out_scale_max`` (a ``new_max`` buffer) receives the maximum of the output's group
+    scales for the FP8 format ``out_fp8``."""
     from .. import _hip
     B, H, S, D = q.shape
     Hkv = k.shape[1]
@@ -37,7 +38,8 @@ def attention_forward(q, k, v, causal=True, scale=None, need_lse=True):
     lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device) if need_lse else None
     _hip.check(lib.coat_attention_forward_bf16(_hip.ptr(q), _hip.ptr(k), _hip.ptr(v), _hip.ptr(out), _hip.ptr(lse), B, H, Hkv, S, D,
                                                *_strides_bshd(q), *_strides_bshd(k), *_strides_bshd(v), *_strides_bshd(out),
-                                               scale, 1 if causal else 0, st), "attention forward")
+                                               scale, 1 if causal else 0, _hip.ptr(out_scale_max),
+                                               _hip.fp8(out_fp8) if out_scale_max is not None else 0, st), "attention forward")
     return out, lse
 
 
@@ -45,8 +47,8 @@ class _CausalAttention(torch.autograd.Function):
     """Forward: this library's kernel.  Backward: torch's memory-efficient attention backward on (q, k, v, out, lse)."""
 
     @staticmethod
-    def forward(ctx, q, k, v):
-        out, lse = attention_forward(q, k, v, causal=True)
+    def forward(ctx, q, k, v, out_scale_max=None, out_fp8=None):
+        out, lse = attention_forward(q, k, v, causal=True, out_scale_max=out_scale_max, out_fp8=out_fp8)
         ctx.save_for_backward(q, k, v, out, lse)
         return out
 
@@ -56,7 +58,7 @@ class _CausalAttention(torch.autograd.Function):
         zero = torch.zeros((), dtype=torch.int64)  # dropout state, unused with dropout_p = 0
         dq, dk, dv, _ = torch.ops.aten._scaled_dot_product_efficient_attention_backward(
             g, q, k, v, None, out, lse, zero, zero, 0.0, [True, True, True, False], True)
-        return dq, dk, dv
+        return dq, dk, dv, None, None
 
 
 def _own_kernel_applies(q, k, v, attn_mask, dropout_p, is_causal):
@@ -75,7 +77,12 @@ def torch_sdpa(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False):
         return F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal)
 
 
-def sdpa(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False):
+def sdpa(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False, out_scale_max=None, out_fp8=None):
+    """Attention of the decoder layers.  With ``out_scale_max`` (a ``new_max`` buffer) returns (out, filled): the library's
+    kernel also merges the maximum of the output's group scales for the FP8 format ``out_fp8`` into the buffer; filled is
+    False when torch's attention ran instead and the buffer was left alone."""
     if _own_kernel_applies(q, k, v, attn_mask, dropout_p, is_causal):
-        return _CausalAttention.apply(q, k, v)
-    return torch_sdpa(q, k, v, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal)
+        out = _CausalAttention.apply(q, k, v, out_scale_max, out_fp8)
+        return out if out_scale_max is None else (out, True)
+    out = torch_sdpa(q, k, v, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal)
+    return out if out_scale_max is None else (out, False)

@@ -29,7 +29,7 @@ from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_If
                                             fp8_rmsnorm_backward, fp8_rmsnorm_backward_add, fp8_rmsnorm_forward,
                                             fp8_silu_mul_backward,
                                             fp8_silu_mul_forward, fp8_transpose)
-from ..activation.real_quantization.common import scale_max
+from ..activation.real_quantization.common import convert_str_to_fp8, new_max, scale_max, tag_scale_max
 from ..utils._fp8_quantization_config import QuantizationConfig
 from ..utils._fp8_weightcache import FP8CacheWeightModule
 from ..utils._fp8manager import FP8Manager
@@ -219,7 +219,7 @@ class CoatLlamaAfterAttentionResidual(_ResidualBase):
 class _CoatLlamaAfterAttentionResidual(torch.autograd.Function):
     @staticmethod
     def forward(ctx, re_x, flash_x, w4_origin, w4, w4_t, w4_s, group_size, fwobits, layer_id, config, qargs):
-        flash_qx, flash_s, _ = fp8_quantize_pertensor(flash_x, group_size, fwobits["fabit"])
+        flash_qx, flash_s, _ = fp8_quantize_pertensor(flash_x, group_size, fwobits["fabit"], want_pg=False)
         w8 = _forward_weight(w4_origin, w4, w4_s, qargs, fwobits)
         # fp8_linear_forward + fp8_add_Ifp_Ifp_Ofp_Og16 of the reference (:440-441): the addition runs in the GEMM epilogue
         fp_x, (out_x, out_s) = fp8_linear_forward_add(flash_qx, flash_s, w8, w4_s, re_x, flash_qx.dtype, group_size)
@@ -380,16 +380,17 @@ class _FusedRoPE(torch.autograd.Function):
     (``coat_rope_bf16``; the backward pass is the rotation by the negated angle)."""
 
     @staticmethod
-    def forward(ctx, x, cos_tab, sin_tab, pos, heads, head_dim, theta):
+    def forward(ctx, x, cos_tab, sin_tab, pos, heads, head_dim, theta, grad_fp8=None):
         from .. import _hip
         B, S, _ = x.shape
         x = _hip.dense(x)
         y = torch.empty_like(x)
         _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(x), _hip.ptr(y), _hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0],
-                                             theta, _hip.ptr(pos), B * S, S, heads, head_dim, 0, 0, 0,
+                                             theta, _hip.ptr(pos), B * S, S, heads, head_dim, 0, 0, 0, None, 0,
                                              _hip.stream(x.device)), "rope forward")
         ctx.save_for_backward(cos_tab, sin_tab, pos)
         ctx.dims = (B, S, heads, head_dim, theta)
+        ctx.grad_fp8 = grad_fp8
         return y.view(B, S, heads, head_dim).transpose(1, 2)
 
     @staticmethod
@@ -399,10 +400,16 @@ class _FusedRoPE(torch.autograd.Function):
         B, S, heads, head_dim, theta = ctx.dims
         g = _hip.dense(g.transpose(1, 2).to(torch.bfloat16))  # physically [B, S, heads, head_dim]
         dx = torch.empty_like(g)
+        # the consumer quantizes this gradient per tensor (reference :318-326): the kernel hands it the scale maximum
+        s_max = new_max(g.device) if ctx.grad_fp8 is not None else None
         _hip.check(_hip.lib().coat_rope_bf16(_hip.ptr(g), _hip.ptr(dx), _hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0],
-                                             theta, _hip.ptr(pos), B * S, S, heads, head_dim, 1, 0, 0,
+                                             theta, _hip.ptr(pos), B * S, S, heads, head_dim, 1, 0, 0, _hip.ptr(s_max),
+                                             _hip.fp8(ctx.grad_fp8) if s_max is not None else 0,
                                              _hip.stream(g.device)), "rope backward")
-        return dx.view(B, S, heads * head_dim), None, None, None, None, None, None
+        dx = dx.view(B, S, heads * head_dim)
+        if s_max is not None:
+            tag_scale_max(dx, s_max, ctx.grad_fp8)
+        return dx, None, None, None, None, None, None, None
 
 
 class _FusedQKVRoPE(torch.autograd.Function):
@@ -423,10 +430,10 @@ class _FusedQKVRoPE(torch.autograd.Function):
         k = torch.empty((B, S, Dkv), dtype=qkv.dtype, device=qkv.device)
         lib, st = _hip.lib(), _hip.stream(qkv.device)
         tabs = (_hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0], theta, None)
-        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, :Dq]), _hip.ptr(q), *tabs, B * S, S, heads, head_dim, 0, W, 0, st),
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, :Dq]), _hip.ptr(q), *tabs, B * S, S, heads, head_dim, 0, W, 0, None, 0, st),
                    "rope forward (q of qkv)")
         _hip.check(lib.coat_rope_bf16(_hip.ptr(flat[:, Dq:Dq + Dkv]), _hip.ptr(k), *tabs, B * S, S, kv_heads, head_dim, 0, W,
-                                      0, st), "rope forward (k of qkv)")
+                                      0, None, 0, st), "rope forward (k of qkv)")
         ctx.save_for_backward(cos_tab, sin_tab)
         ctx.dims = (B, S, heads, kv_heads, head_dim, theta)
         v = qkv[..., Dq + Dkv:].view(B, S, kv_heads, head_dim).transpose(1, 2)
@@ -445,10 +452,10 @@ class _FusedQKVRoPE(torch.autograd.Function):
         flat = dqkv.view(B * S, W)
         lib, st = _hip.lib(), _hip.stream(gq.device)
         tabs = (_hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0], theta, None)
-        _hip.check(lib.coat_rope_bf16(_hip.ptr(gq), _hip.ptr(flat[:, :Dq]), *tabs, B * S, S, heads, head_dim, 1, 0, W, st),
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(gq), _hip.ptr(flat[:, :Dq]), *tabs, B * S, S, heads, head_dim, 1, 0, W, None, 0, st),
                    "rope backward (q of qkv)")
         _hip.check(lib.coat_rope_bf16(_hip.ptr(gk), _hip.ptr(flat[:, Dq:Dq + Dkv]), *tabs, B * S, S, kv_heads, head_dim, 1, 0,
-                                      W, st), "rope backward (k of qkv)")
+                                      W, None, 0, st), "rope backward (k of qkv)")
         dqkv[..., Dq + Dkv:].copy_(gv.transpose(1, 2).reshape(B, S, Dkv))
         return dqkv, None, None, None, None, None, None
 
@@ -460,8 +467,10 @@ def fused_qkv_rotary(qkv, heads, kv_heads, head_dim, theta):
     return _FusedQKVRoPE.apply(qkv, cos_tab, sin_tab, heads, kv_heads, head_dim, float(theta))
 
 
-def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=None):
-    """RoPE on a projection output x [B, S, heads * head_dim] (bf16, on the GPU); returns [B, heads, S, head_dim]."""
+def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=None, grad_fp8=None):
+    """RoPE on a projection output x [B, S, heads * head_dim] (bf16, on the GPU); returns [B, heads, S, head_dim].
+    ``grad_fp8`` (an FP8 dtype): the backward also hands the consumer of x's gradient the maximum of its group scales for
+    that format (``common.tag_scale_max``)."""
     B, S, _ = x.shape
     if position_ids is None:
         cos_tab, sin_tab = rotary_tables(S, head_dim, theta, x.device)
@@ -471,7 +480,7 @@ def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=Non
         cos_tab, sin_tab = rotary_tables(n_pos, head_dim, theta, x.device)
         # positions beyond the table are not clamped: the kernel computes their angles itself (no read outside the table)
         pos = position_ids.expand(B, S).reshape(-1).to(torch.int64).contiguous()
-    return _FusedRoPE.apply(x, cos_tab, sin_tab, pos, heads, head_dim, float(theta))
+    return _FusedRoPE.apply(x, cos_tab, sin_tab, pos, heads, head_dim, float(theta), grad_fp8)
 
 
 class LlamaSdpaAttentionWithoutLinear(nn.Module):
@@ -489,6 +498,11 @@ class LlamaSdpaAttentionWithoutLinear(nn.Module):
         self.num_key_value_heads = config.num_key_value_heads
         self.num_key_value_groups = self.num_heads // self.num_key_value_heads
         self.rope_theta = config.rope_theta
+        # formats in which the neighbouring FP8 modules quantize this module's output (forward) and the gradients of its
+        # inputs (backward) per tensor: the kernels here hand them the scale maximum
+        qargs = QuantizationConfig(**getattr(config, "coat_fp8_args", {}))
+        self._out_fp8 = convert_str_to_fp8[qargs.fabit]
+        self._grad_fp8 = convert_str_to_fp8[qargs.babit]
 
     def forward(self, query_states, key_states, value_states, attention_mask=None, position_ids=None,
                 past_key_value=None, output_attentions=False, use_cache=False, cache_position=None,
@@ -500,8 +514,10 @@ class LlamaSdpaAttentionWithoutLinear(nn.Module):
         if position_embeddings is None and query_states.is_cuda and query_states.dtype == torch.bfloat16:
             # one fused kernel per tensor and direction instead of mul / neg / cat / add passes
             max_pos = getattr(self.config, "max_position_embeddings", None)
-            q = fused_rotary(query_states, self.num_heads, self.head_dim, self.rope_theta, position_ids, max_pos)
-            k = fused_rotary(key_states, self.num_key_value_heads, self.head_dim, self.rope_theta, position_ids, max_pos)
+            grad_fp8 = self._grad_fp8 if self.training else None
+            q = fused_rotary(query_states, self.num_heads, self.head_dim, self.rope_theta, position_ids, max_pos, grad_fp8)
+            k = fused_rotary(key_states, self.num_key_value_heads, self.head_dim, self.rope_theta, position_ids, max_pos,
+                             grad_fp8)
         else:
             q = query_states.view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
             k = key_states.view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
@@ -518,10 +534,14 @@ class LlamaSdpaAttentionWithoutLinear(nn.Module):
         mask = attention_mask
         if mask is not None:
             mask = mask[:, :, :, : k.shape[-2]]
-        out = sdpa(q, k, v, attn_mask=mask,
-                                             dropout_p=self.attention_dropout if self.training else 0.0,
-                                             is_causal=mask is None and q_len > 1)
+        # in training the next module quantizes this output per tensor (reference :434): the kernel hands it the scale maximum
+        out_max = new_max(q.device) if self.training and q.is_cuda else None
+        out = sdpa(q, k, v, attn_mask=mask, dropout_p=self.attention_dropout if self.training else 0.0,
+                   is_causal=mask is None and q_len > 1, out_scale_max=out_max, out_fp8=self._out_fp8)
+        out, used_max = out if out_max is not None else (out, False)
         out = out.transpose(1, 2).contiguous().view(bsz, q_len, -1)
+        if used_max:
+            tag_scale_max(out, out_max, self._out_fp8)
         return out, None, past_key_value
 
 

@@ -255,10 +255,13 @@ int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_d
  * computes that row's angles from theta itself;
  * y1 = x1 cos - x2 sin, y2 = x2 cos + x1 sin on the (d, d + head_dim/2) pairs; inverse != 0 negates the angle, which
  * is the backward pass.  head_dim % 16 == 0.  x_pitch / y_pitch: row pitches in elements, 0 = contiguous; a multiple
- * of 8 (16-byte rows), for x or y that is a column slice of a fused q/k/v tensor (coat/models/coat_olmo.py:1003-1006). */
+ * of 8 (16-byte rows), for x or y that is a column slice of a fused q/k/v tensor (coat/models/coat_olmo.py:1003-1006).
+ * s_max (may be NULL): a COAT_MAX_WORDS buffer as above; the kernel merges (max|y| + 1e-10) / fp8max of format fp8_max
+ * into it, which is what coat_fp8_group_scales would merge for y with any group size, so a caller that quantizes the
+ * rotated tensor per tensor (the gradients at coat/models/coat_llama.py:318-326) skips that pass. */
 int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, int64_t n_pos, float theta,
                    const int64_t* pos, int64_t rows, int seq_len, int heads, int head_dim, int inverse, int64_t x_pitch,
-                   int64_t y_pitch, void* stream);
+                   int64_t y_pitch, float* s_max, int fp8_max, void* stream);
 
 /* ---- bf16 attention (forward) ------------------------------------------------------------------------
  * The attention between the FP8 projections: the reference calls the flash-attn library here
@@ -267,12 +270,14 @@ int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* si
  * through element strides (batch, token, head; the head dimension is contiguous; all strides multiples of 8), so the
  * projections' outputs are used where they lie.  k and v have kv_heads heads (heads % kv_heads == 0).  lse (may be
  * NULL): fp32 [batch, heads, seq], natural logarithm of each query's sum of exponentials, as backward kernels expect it.
- * head_dim must be 128. */
+ * head_dim must be 128. s_max (may be NULL): a COAT_MAX_WORDS buffer; the kernel merges (max|out| + 1e-10) / fp8max of
+ * format fp8_max into it, what coat_fp8_group_scales would merge for out, so the per-tensor quantization of the attention
+ * output (coat/models/coat_llama.py:434, fp8_quantize_pertensor) goes straight to its division pass. */
 int coat_attention_forward_bf16(const void* q, const void* k, const void* v, void* out, float* lse, int64_t batch,
                                 int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int64_t q_sb, int64_t q_ss,
                                 int64_t q_sh, int64_t k_sb, int64_t k_ss, int64_t k_sh, int64_t v_sb, int64_t v_ss,
                                 int64_t v_sh, int64_t o_sb, int64_t o_ss, int64_t o_sh, float scale, int causal,
-                                void* stream);
+                                float* s_max, int fp8_max, void* stream);
 
 /* ---- GEMM -------------------------------------------------------------------------------------------
  * rq/linear.py:172 fp8matmul (kernel :61-169): C[M,N] = (A[M,K] . B[N,K]^T) * (float(*scale_a) * float(*scale_b))

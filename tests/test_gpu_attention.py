@@ -77,3 +77,76 @@ def test_attention_autograd_matches_fp32_autograd(dev):
         rel = ((got.float() - want).norm() / want.norm()).item()
         print(f"[measured] attention backward {name}: relative Frobenius {rel:.2e} (bar 1e-2)")
         assert rel < 1e-2, (name, rel)
+
+
+def _scale_pass_max(t, fp8):
+    """What the scale pass of fp8_quantize_pertensor would merge for the bf16 tensor t: the maximum fp32 group scale."""
+    from coat_amd.activation.real_quantization._quantize_pertensor import group_scales_and_max
+    from coat_amd.activation.real_quantization.common import read_max
+    t2 = t.reshape(-1, t.shape[-1]).contiguous()
+    return read_max(group_scales_and_max(t2, 16, fp8, want_pg=False)[1])
+
+
+@pytest.mark.parametrize("fp8", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_forward_hands_over_the_scale_maximum_of_its_output(dev, fp8):
+    """coat_attention_forward_bf16 with s_max: the buffer holds, bit for bit, the maximum group scale that
+    coat_fp8_group_scales finds on the stored output (ragged length: rows beyond the sequence do not count)."""
+    from coat_amd.activation.real_quantization.common import new_max, read_max
+    from coat_amd.models._attention import attention_forward
+    B, H, S, D = 2, 4, 333, 128
+    g = torch.Generator().manual_seed(11)
+    q, k, v = [(torch.randn(B, S, H, D, generator=g) * 3).bfloat16().to(dev).transpose(1, 2) for _ in range(3)]
+    buf = new_max(dev)
+    out, _ = attention_forward(q, k, v, causal=True, out_scale_max=buf, out_fp8=fp8)
+    ref, _ = attention_forward(q, k, v, causal=True)
+    assert torch.equal(out, ref)
+    assert read_max(buf).item() == _scale_pass_max(out.transpose(1, 2).reshape(B * S, H * D), fp8).item() > 0
+
+
+def test_layer_quantizations_fed_by_handed_over_maxima_are_bit_identical(dev, monkeypatch):
+    """The attention module tags its output (forward) and the RoPE backward tags the q / k gradients with the scale maximum
+    their kernels merged; fp8_quantize_pertensor(_transpose) then skip their scale pass.  Same codes, same scale and the
+    scale pass really skipped: compared with the untagged path on the same tensors."""
+    import coat_amd.activation.real_quantization._quantize_pertensor as QP
+    from coat_amd.activation.real_quantization import fp8_quantize_pertensor, fp8_quantize_pertensor_transpose
+    from coat_amd.activation.real_quantization.common import known_scale_max
+    from coat_amd.models.coat_llama import CoatLlamaConfig, LlamaSdpaAttentionWithoutLinear
+    cfg = CoatLlamaConfig(hidden_size=512, intermediate_size=1024, num_attention_heads=4, num_key_value_heads=4)
+    attn = LlamaSdpaAttentionWithoutLinear(cfg, 0).train()
+    B, S, Hd = 2, 160, 512
+    g = torch.Generator().manual_seed(12)
+    qs, ks, vs = [torch.randn(B, S, Hd, generator=g).bfloat16().to(dev).requires_grad_(True) for _ in range(3)]
+    out, _, _ = attn(qs, ks, vs)
+    assert known_scale_max(out, torch.float8_e4m3fn) is not None and known_scale_max(out, torch.float8_e5m2) is None
+    calls = []
+    real = QP.group_scales_and_max
+    monkeypatch.setattr(QP, "group_scales_and_max", lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    import coat_amd.activation.real_quantization._quantize_pertensor_transpose as QPT
+    monkeypatch.setattr(QPT, "group_scales_and_max", QP.group_scales_and_max)
+    q1, s1, _ = fp8_quantize_pertensor(out, 16, "E4M3", want_pg=False)
+    assert not calls
+    q0, s0, _ = fp8_quantize_pertensor(out.detach().clone(), 16, "E4M3", want_pg=False)
+    assert len(calls) == 1 and torch.equal(q0.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(s0, s1)
+    # an in-place change after the hand-over invalidates the tag
+    from coat_amd.activation.real_quantization.common import tag_scale_max
+    out2 = tag_scale_max(out.detach().clone(), out._coat_scale_max[0], torch.float8_e4m3fn)
+    assert known_scale_max(out2, torch.float8_e4m3fn) is not None
+    out2.mul_(2)
+    assert known_scale_max(out2, torch.float8_e4m3fn) is None
+    # backward: the gradients of the q and k projections arrive tagged for e5m2, the one of v (torch's backward) untagged
+    seen = {}
+    qs.register_hook(lambda gr: seen.__setitem__("q", gr))
+    ks.register_hook(lambda gr: seen.__setitem__("k", gr))
+    vs.register_hook(lambda gr: seen.__setitem__("v", gr))
+    out.backward(torch.randn(B, S, Hd, generator=g).bfloat16().to(dev) * 1e-2)
+    assert known_scale_max(seen["v"], torch.float8_e5m2) is None
+    for name in ("q", "k"):
+        gr = seen[name]
+        assert known_scale_max(gr, torch.float8_e5m2) is not None
+        n = len(calls)
+        a = fp8_quantize_pertensor_transpose(gr, 16, "E5M2", transpose_output_2d=True)
+        assert len(calls) == n
+        b = fp8_quantize_pertensor_transpose(gr.detach().clone(), 16, "E5M2", transpose_output_2d=True)
+        assert len(calls) == n + 1
+        for x, y in zip(a, b):
+            assert torch.equal(x.view(torch.uint8) if x.dtype != torch.bfloat16 else x, y.view(torch.uint8) if y.dtype != torch.bfloat16 else y)

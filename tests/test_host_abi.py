@@ -124,8 +124,9 @@ def test_argument_validation_of_the_remaining_entry_points_without_gpu():
     assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 24, 16, None) == ESHAPE   # K % 16
     assert L.coat_fp8_gemm_grouped(3, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 0, 64, 16, None) == 0         # empty
     # RoPE, cross-entropy
-    assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 24, 0, 0, 0, None) == ESHAPE                      # head_dim % 16
-    assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 48, 0, None) == ESHAPE                     # pitch < heads * head_dim
+    assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 24, 0, 0, 0, None, 0, None) == ESHAPE             # head_dim % 16
+    assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 48, 0, None, 0, None) == ESHAPE            # pitch < heads * head_dim
+    assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 0, 0, p, 7, None) == EINVAL                # unknown format for the maximum
     assert L.coat_cross_entropy_forward(p, 0, 8, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # stride < columns
     assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, None, 4, 16, -100, 0.0, 0.0, 1, 0.0, 0, None) == EINVAL  # mean without a count
     assert L.coat_cross_entropy_forward(p, 0, 16, p, p, None, p, 4, 16, -100, 0.0, 0.0, 7, 0.0, 0, None) == EINVAL
