@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("COAT_HIP_LIB") or os.path.join(_HERE, "libcoat_hip.so
 F32, BF16, F16 = 0, 1, 2
 MAX_SLOTS, MAX_SLOT_STRIDE = 16, 32  # COAT_MAX_SLOTS, COAT_MAX_SLOT_STRIDE of include/coat_hip.h
 MAX_WORDS = MAX_SLOTS * MAX_SLOT_STRIDE
-ABI_VERSION = 3  # COAT_ABI_VERSION of include/coat_hip.h: a library built from another header is refused
+ABI_VERSION = 4  # COAT_ABI_VERSION of include/coat_hip.h: a library built from another header is refused
 E4M3, E5M2 = 0, 1
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
@@ -69,6 +69,9 @@ SIGNATURES = {
     "coat_fp8_adamw_expand_step": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _i,
                                    _i64, _i64, _vp],
     "coat_fp8_adamw_step": [_vp, _vp, _i, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _i64, _i64, _vp],
+    "coat_fp8_adamw_expand_step_multi": [_i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f,
+                                         _i, _i, _i, _vp],
+    "coat_fp8_adamw_step_multi": [_i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp],
 }
 
 _lib = None

@@ -468,9 +468,71 @@ __global__ __launch_bounds__(256) void k_fp8_adamw_expand(void* __restrict__ par
                                       sqrtmm_v, A, numel, ngroups, wave, lane);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Several tensors in one launch (the reference's optimizer loops over the parameters and launches once per parameter,
+// coat/optimizer/fp8_adamw.py:419-515; a model's many small tensors, norm weights and biases, then cost a launch each for a
+// few microseconds of work).  The records of up to kAdamMultiMax tensors travel in the kernel arguments; a block finds
+// its tensor from the table of first block indices and then runs the very wave routine of the single-tensor kernels, so
+// every tensor's result is bit-identical to its own launch.
+constexpr int kAdamMultiMax = 32;
+struct AdamMultiTensor {
+    void* params;
+    const void* grads;
+    uint8_t* exp_avg;
+    float *scale_m, *expand_m, *sqrtmm_m;
+    uint8_t* exp_avg_sq;
+    float *scale_v, *expand_v, *sqrtmm_v;
+    int64_t numel;
+};
+struct AdamMultiArgs {
+    AdamMultiTensor t[kAdamMultiMax];
+    unsigned first_block[kAdamMultiMax + 1];  // first_block[count] = grid size
+    int count;
+};
+
+template <int PDT, bool EXPAND>
+__global__ __launch_bounds__(256) void k_fp8_adamw_multi(AdamMultiArgs M, AdamArgs A) {
+    enable_fp8_saturation();
+    int ti = 0;  // the last tensor whose first block is not after this one (block-uniform, scalar registers)
+    for (int i = 1; i < M.count; i++)
+        if (blockIdx.x >= M.first_block[i]) ti = i;
+    const AdamMultiTensor& T = M.t[ti];
+    const int64_t numel = T.numel, ngroups = (numel + kGroup - 1) / kGroup;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)(blockIdx.x - M.first_block[ti]) * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (wave * 8 >= ngroups) return;
+    const bool full = (wave * 8 + 8) * kGroup <= numel;
+    if (EXPAND) {
+        if (full)
+            adamw_expand_wave<PDT, true>(T.params, T.grads, T.exp_avg, T.scale_m, T.expand_m, T.sqrtmm_m, T.exp_avg_sq, T.scale_v,
+                                         T.expand_v, T.sqrtmm_v, A, numel, ngroups, wave, lane);
+        else
+            adamw_expand_wave<PDT, false>(T.params, T.grads, T.exp_avg, T.scale_m, T.expand_m, T.sqrtmm_m, T.exp_avg_sq, T.scale_v,
+                                          T.expand_v, T.sqrtmm_v, A, numel, ngroups, wave, lane);
+    } else {
+        if (full)
+            adamw_plain_wave<PDT, true>(T.params, T.grads, T.exp_avg, T.scale_m, T.exp_avg_sq, T.scale_v, A, numel, ngroups, wave, lane);
+        else
+            adamw_plain_wave<PDT, false>(T.params, T.grads, T.exp_avg, T.scale_m, T.exp_avg_sq, T.scale_v, A, numel, ngroups, wave, lane);
+    }
+}
+
 }  // namespace coat
 
 using namespace coat;
+
+static AdamArgs adam_args(float beta1, float beta2, float lr, float wd, float eps, int step, int expand_min) {
+    AdamArgs A;
+    A.beta1 = beta1; A.beta2 = beta2; A.lr = lr; A.wd = wd; A.eps = eps;
+    A.one_minus_beta1 = 1 - beta1;
+    A.one_minus_beta2 = 1 - beta2;
+    // correctly rounded powf(beta, step): double pow rounded once
+    A.correction1 = 1.0f - (float)pow((double)beta1, (double)(float)step);
+    A.correction2_sqrt = sqrtf(1.0f - (float)pow((double)beta2, (double)(float)step));
+    A.expand_min = (float)expand_min;
+    A.inv_expand_min = (expand_min > 0 && (expand_min & (expand_min - 1)) == 0) ? 1.0f / (float)expand_min : 0.0f;
+    return A;
+}
 
 static int adamw_common(void* params, const void* grads, int p_dtype, void* exp_avg, float* scale_m, float* expand_m,
                         float* sqrtmm_m, void* exp_avg_sq, float* scale_v, float* expand_v, float* sqrtmm_v,
@@ -485,15 +547,7 @@ static int adamw_common(void* params, const void* grads, int p_dtype, void* exp_
     if (expand && (!expand_m || !expand_v || !sqrtmm_m || !sqrtmm_v)) return COAT_EINVAL;
     if (!coat_aligned16(params) || !coat_aligned16(grads) || !coat_aligned16(exp_avg) || !coat_aligned16(exp_avg_sq))
         return COAT_EALIGN;
-    AdamArgs A;
-    A.beta1 = beta1; A.beta2 = beta2; A.lr = lr; A.wd = wd; A.eps = eps;
-    A.one_minus_beta1 = 1 - beta1;
-    A.one_minus_beta2 = 1 - beta2;
-    // correctly rounded powf(beta, step): double pow rounded once
-    A.correction1 = 1.0f - (float)pow((double)beta1, (double)(float)step);
-    A.correction2_sqrt = sqrtf(1.0f - (float)pow((double)beta2, (double)(float)step));
-    A.expand_min = (float)expand_min;
-    A.inv_expand_min = (expand_min > 0 && (expand_min & (expand_min - 1)) == 0) ? 1.0f / (float)expand_min : 0.0f;
+    const AdamArgs A = adam_args(beta1, beta2, lr, wd, eps, step, expand_min);
     const int64_t waves = (ngroups + 7) / 8;
     const int64_t blocks = (waves + 3) / 4;
     hipStream_t st = (hipStream_t)stream;
@@ -532,4 +586,89 @@ extern "C" int coat_fp8_adamw_step(void* params, const void* grads, int p_dtype,
                                    void* stream) {
     return adamw_common(params, grads, p_dtype, exp_avg, scale_exp_avg, nullptr, nullptr, exp_avg_sq, scale_exp_avg_sq,
                         nullptr, nullptr, beta1, beta2, lr, wd, eps, step, qgroup_size, 0, false, numel, n_scale, stream);
+}
+
+// Host side of the multi-tensor launches: validates every tensor like the single-tensor entry points, then launches the
+// tensors in chunks of kAdamMultiMax (and of fewer than 2^31 blocks).
+static int adamw_multi(int count, void* const* params, const void* const* grads, int p_dtype, void* const* exp_avg,
+                       float* const* scale_m, float* const* expand_m, float* const* sqrtmm_m, void* const* exp_avg_sq,
+                       float* const* scale_v, float* const* expand_v, float* const* sqrtmm_v, const int64_t* numel,
+                       const int64_t* n_scale, float beta1, float beta2, float lr, float wd, float eps, int step,
+                       int qgroup_size, int expand_min, bool expand, void* stream) {
+    if (qgroup_size != kGroup) return COAT_EQGROUP;
+    if (count < 0) return COAT_EINVAL;
+    if (count == 0) return COAT_OK;
+    if (!params || !grads || !exp_avg || !exp_avg_sq || !scale_m || !scale_v || !numel || !n_scale) return COAT_EINVAL;
+    if (expand && (!expand_m || !expand_v || !sqrtmm_m || !sqrtmm_v)) return COAT_EINVAL;
+    if (p_dtype != COAT_F32 && p_dtype != COAT_BF16 && p_dtype != COAT_F16) return COAT_EDTYPE;
+    for (int i = 0; i < count; i++) {  // everything is checked before the first launch
+        if (numel[i] < 0) return COAT_EINVAL;
+        if (n_scale[i] != (numel[i] + kGroup - 1) / kGroup) return COAT_ESHAPE;
+        if (numel[i] == 0) continue;
+        if (!params[i] || !grads[i] || !exp_avg[i] || !exp_avg_sq[i] || !scale_m[i] || !scale_v[i]) return COAT_EINVAL;
+        if (expand && (!expand_m[i] || !expand_v[i] || !sqrtmm_m[i] || !sqrtmm_v[i])) return COAT_EINVAL;
+        if (!coat_aligned16(params[i]) || !coat_aligned16(grads[i]) || !coat_aligned16(exp_avg[i]) || !coat_aligned16(exp_avg_sq[i]))
+            return COAT_EALIGN;
+    }
+    const AdamArgs A = adam_args(beta1, beta2, lr, wd, eps, step, expand_min);
+    hipStream_t st = (hipStream_t)stream;
+    AdamMultiArgs M;
+    int i = 0;
+    while (i < count) {
+        M.count = 0;
+        uint64_t blocks = 0;
+        for (; i < count && M.count < kAdamMultiMax; i++) {
+            if (numel[i] == 0) continue;
+            const int64_t ngroups = (numel[i] + kGroup - 1) / kGroup;
+            const uint64_t b = (uint64_t)((ngroups + 31) / 32);  // 4 waves of 8 groups per block
+            if (blocks + b > 0x7fffffffull) {
+                if (M.count == 0) return COAT_ESHAPE;  // one tensor beyond 2^31 blocks (2^43 elements)
+                break;
+            }
+            AdamMultiTensor& T = M.t[M.count];
+            T.params = params[i]; T.grads = grads[i]; T.exp_avg = (uint8_t*)exp_avg[i]; T.scale_m = scale_m[i];
+            T.expand_m = expand ? expand_m[i] : nullptr; T.sqrtmm_m = expand ? sqrtmm_m[i] : nullptr;
+            T.exp_avg_sq = (uint8_t*)exp_avg_sq[i]; T.scale_v = scale_v[i];
+            T.expand_v = expand ? expand_v[i] : nullptr; T.sqrtmm_v = expand ? sqrtmm_v[i] : nullptr;
+            T.numel = numel[i];
+            M.first_block[M.count++] = (unsigned)blocks;
+            blocks += b;
+        }
+        if (M.count == 0) break;  // only empty tensors were left
+        M.first_block[M.count] = (unsigned)blocks;
+#define LAUNCH_MULTI(PDT)                                                                                             \
+    if (expand) hipLaunchKernelGGL((k_fp8_adamw_multi<PDT, true>), dim3((unsigned)blocks), dim3(256), 0, st, M, A);   \
+    else hipLaunchKernelGGL((k_fp8_adamw_multi<PDT, false>), dim3((unsigned)blocks), dim3(256), 0, st, M, A);
+        switch (p_dtype) {
+            case COAT_F32: LAUNCH_MULTI(kF32); break;
+            case COAT_BF16: LAUNCH_MULTI(kBF16); break;
+            default: LAUNCH_MULTI(kF16); break;
+        }
+#undef LAUNCH_MULTI
+        const int rc = coat_launch_status();
+        if (rc != COAT_OK) return rc;
+    }
+    return COAT_OK;
+}
+
+extern "C" int coat_fp8_adamw_expand_step_multi(int count, void* const* params, const void* const* grads, int p_dtype,
+                                                void* const* exp_avg, float* const* scale_exp_avg,
+                                                float* const* expand_exp_avg, float* const* sqrtminmax_exp_avg,
+                                                void* const* exp_avg_sq, float* const* scale_exp_avg_sq,
+                                                float* const* expand_exp_avg_sq, float* const* sqrtminmax_exp_avg_sq,
+                                                const int64_t* numel, const int64_t* n_scale, float beta1, float beta2,
+                                                float lr, float wd, float eps, int step, int qgroup_size, int expand_min,
+                                                void* stream) {
+    return adamw_multi(count, params, grads, p_dtype, exp_avg, scale_exp_avg, expand_exp_avg, sqrtminmax_exp_avg, exp_avg_sq,
+                       scale_exp_avg_sq, expand_exp_avg_sq, sqrtminmax_exp_avg_sq, numel, n_scale, beta1, beta2, lr, wd, eps,
+                       step, qgroup_size, expand_min, true, stream);
+}
+
+extern "C" int coat_fp8_adamw_step_multi(int count, void* const* params, const void* const* grads, int p_dtype,
+                                         void* const* exp_avg, float* const* scale_exp_avg, void* const* exp_avg_sq,
+                                         float* const* scale_exp_avg_sq, const int64_t* numel, const int64_t* n_scale,
+                                         float beta1, float beta2, float lr, float wd, float eps, int step, int qgroup_size,
+                                         void* stream) {
+    return adamw_multi(count, params, grads, p_dtype, exp_avg, scale_exp_avg, nullptr, nullptr, exp_avg_sq, scale_exp_avg_sq,
+                       nullptr, nullptr, numel, n_scale, beta1, beta2, lr, wd, eps, step, qgroup_size, 0, false, stream);
 }

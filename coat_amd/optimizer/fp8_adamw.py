@@ -41,7 +41,10 @@ class CoatAdamW(Optimizer):
         qargs: QuantizationConfig = None,
         *,
         fused: Optional[bool] = None,
+        multi_tensor: bool = True,
     ):
+        # multi_tensor (not in the reference): parameters of one dtype, device and step count share kernel launches
+        self.multi_tensor = multi_tensor
         self.qargs = QuantizationConfig() if qargs is None else qargs
         assert self.qargs.first_order_expansion == self.qargs.second_order_expansion, (
             "We expect the first order and second order momentum to use dynamic range expansion at the same time.")
@@ -150,6 +153,9 @@ class CoatAdamW(Optimizer):
             lr, wd, eps = group["lr"], group["weight_decay"], group["eps"]
             if isinstance(lr, torch.Tensor):
                 lr = lr.item()
+            # parameters of one dtype, device and step count are stepped together, 32 to a launch (the reference launches
+            # once per parameter, :419-515); a parameter alone in its bucket takes the single-tensor entry point
+            buckets = {}
             for p in group["params"]:
                 if p.grad is None:
                     continue
@@ -163,14 +169,30 @@ class CoatAdamW(Optimizer):
                 grad = p.grad if p.grad.is_contiguous() else p.grad.contiguous()
                 if not p.is_contiguous():
                     raise RuntimeError("CoatAdamW needs contiguous parameters (the state is laid out flat)")
+                buckets.setdefault((p.dtype, p.device, step), []).append((p, grad, state))
+            for (_, _, step), items in buckets.items():
+                if len(items) == 1 or not getattr(self, "multi_tensor", True):
+                    for p, grad, state in items:
+                        if expand:
+                            qoptim_cuda.fp8_adamw_expand_step(
+                                p, grad, state["exp_avg"], state["scale_exp_avg"], state["expand_exp_avg"],
+                                state["sqrt_minmax_exp_avg"], state["exp_avg_sq"], state["scale_exp_avg_sq"],
+                                state["expand_exp_avg_sq"], state["sqrt_minmax_exp_avg_sq"],
+                                beta1, beta2, lr, wd, eps, step, qgroup_size, expand_min)
+                        else:
+                            qoptim_cuda.fp8_adamw_step(
+                                p, grad, state["exp_avg"], state["scale_exp_avg"], state["exp_avg_sq"],
+                                state["scale_exp_avg_sq"], beta1, beta2, lr, wd, eps, step, qgroup_size)
+                    continue
+                ps, gs, sts = [i[0] for i in items], [i[1] for i in items], [i[2] for i in items]
+                col = lambda key: [st[key] for st in sts]  # noqa: E731
                 if expand:
-                    qoptim_cuda.fp8_adamw_expand_step(
-                        p, grad, state["exp_avg"], state["scale_exp_avg"], state["expand_exp_avg"],
-                        state["sqrt_minmax_exp_avg"], state["exp_avg_sq"], state["scale_exp_avg_sq"],
-                        state["expand_exp_avg_sq"], state["sqrt_minmax_exp_avg_sq"],
+                    qoptim_cuda.fp8_adamw_expand_step_multi(
+                        ps, gs, col("exp_avg"), col("scale_exp_avg"), col("expand_exp_avg"), col("sqrt_minmax_exp_avg"),
+                        col("exp_avg_sq"), col("scale_exp_avg_sq"), col("expand_exp_avg_sq"), col("sqrt_minmax_exp_avg_sq"),
                         beta1, beta2, lr, wd, eps, step, qgroup_size, expand_min)
                 else:
-                    qoptim_cuda.fp8_adamw_step(
-                        p, grad, state["exp_avg"], state["scale_exp_avg"], state["exp_avg_sq"],
-                        state["scale_exp_avg_sq"], beta1, beta2, lr, wd, eps, step, qgroup_size)
+                    qoptim_cuda.fp8_adamw_step_multi(
+                        ps, gs, col("exp_avg"), col("scale_exp_avg"), col("exp_avg_sq"), col("scale_exp_avg_sq"),
+                        beta1, beta2, lr, wd, eps, step, qgroup_size)
         return loss

@@ -47,9 +47,10 @@ enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.f
 
 /* Bumped whenever an entry point's argument list or the size of a buffer it writes changes (2: every s_max / amax
  * argument became COAT_MAX_WORDS words; 3: coat_fp8_gemm_residual, coat_fp8_rmsnorm_backward_add and coat_attention_forward_bf16 added,
- * coat_hbm_probe removed).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
+ * coat_hbm_probe removed; 4: coat_rope_bf16 and coat_attention_forward_bf16 take a maximum buffer, the multi-tensor optimizer
+ * steps added).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
  * loads the library. */
-#define COAT_ABI_VERSION 3
+#define COAT_ABI_VERSION 4
 int coat_abi_version(void);
 const char* coat_version(void);
 const char* coat_status_string(int status);
@@ -332,6 +333,24 @@ int coat_fp8_adamw_expand_step(void* params, const void* grads, int p_dtype, voi
 int coat_fp8_adamw_step(void* params, const void* grads, int p_dtype, void* exp_avg, float* scale_exp_avg,
                         void* exp_avg_sq, float* scale_exp_avg_sq, float beta1, float beta2, float lr, float wd,
                         float eps, int step, int qgroup_size, int64_t numel, int64_t n_scale, void* stream);
+
+/* The two steps above for several tensors in one launch (no single counterpart: the reference's optimizer launches once
+ * per parameter, coat/optimizer/fp8_adamw.py:419-515).  Every argument that is a device pointer above is a host array of
+ * `count` such pointers here, numel / n_scale host arrays of `count` sizes; dtype, hyperparameters and step are common to
+ * the tensors of a call.  The arrays are read before the call returns.  Tensors are launched 32 to a kernel; every
+ * tensor's result is bit-identical to its own coat_fp8_adamw_expand_step / coat_fp8_adamw_step call; empty tensors are
+ * skipped; all tensors are validated before the first launch. */
+int coat_fp8_adamw_expand_step_multi(int count, void* const* params, const void* const* grads, int p_dtype,
+                                     void* const* exp_avg, float* const* scale_exp_avg, float* const* expand_exp_avg,
+                                     float* const* sqrtminmax_exp_avg, void* const* exp_avg_sq,
+                                     float* const* scale_exp_avg_sq, float* const* expand_exp_avg_sq,
+                                     float* const* sqrtminmax_exp_avg_sq, const int64_t* numel, const int64_t* n_scale,
+                                     float beta1, float beta2, float lr, float wd, float eps, int step, int qgroup_size,
+                                     int expand_min, void* stream);
+int coat_fp8_adamw_step_multi(int count, void* const* params, const void* const* grads, int p_dtype, void* const* exp_avg,
+                              float* const* scale_exp_avg, void* const* exp_avg_sq, float* const* scale_exp_avg_sq,
+                              const int64_t* numel, const int64_t* n_scale, float beta1, float beta2, float lr, float wd,
+                              float eps, int step, int qgroup_size, void* stream);
 
 /* coat/activation/liger/cross_entropy.py:24-198 liger_cross_entropy_kernel as launched by cross_entropy_forward
  * (:212-278): softmax cross-entropy over x [n_rows, n_cols] (row pitch x_stride elements, fp32 / bf16 / fp16).

@@ -272,3 +272,72 @@ def test_coatadamw_trajectory_and_state_dict(dev):
         w.grad, w2.grad = g, g.clone()
         opt.step(); opt2.step()
         assert torch.equal(w.detach(), w2.detach())
+
+
+@pytest.mark.parametrize("expand", [True, False])
+@pytest.mark.parametrize("pdtype", [torch.float32, torch.bfloat16])
+def test_multi_tensor_step_equals_separate_launches(dev, expand, pdtype):
+    """coat_fp8_adamw_expand_step_multi / coat_fp8_adamw_step_multi: 70 tensors (three launches of at most 32), sizes from
+    one element over ragged groups to whole waves and an empty tensor in between, three steps: parameters, codes and all
+    group vectors bit-identical to one launch per tensor."""
+    q = _q()
+    sizes = [1, 127, 128, 129, 1024, 1024 * 3 + 5, 4096, 0, 128 * 9 + 37, 128 * 64] * 7
+    gen = torch.Generator().manual_seed(5)
+    ps = [(torch.randn(n, generator=gen) * 0.02).to(pdtype) for n in sizes]
+    keys = KEYS_EXP if expand else KEYS_PLAIN
+    single = [(p.to(dev), to_dev(A.fresh_state(p, expand=expand), dev)) for p in ps]
+    multi = [(p.to(dev), to_dev(A.fresh_state(p, expand=expand), dev)) for p in ps]
+    hp = (HP["beta1"], HP["beta2"], HP["lr"], HP["wd"], HP["eps"])
+    for step in (1, 2, 3):
+        gs = [(torch.randn(n, generator=gen) * 1e-3).to(pdtype).to(dev) for n in sizes]
+        for (p, st), g in zip(single, gs):
+            gpu_step(q, p, g, st, step, expand)
+        cols = [[st[k] for _, st in multi] for k in keys]
+        if expand:
+            q.fp8_adamw_expand_step_multi([p for p, _ in multi], gs, *cols, *hp, step, 128, 16)
+        else:
+            q.fp8_adamw_step_multi([p for p, _ in multi], gs, *cols, *hp, step, 128)
+        for i, ((p1, s1), (p2, s2)) in enumerate(zip(single, multi)):
+            assert torch.equal(p1, p2), (i, sizes[i], step, "params")
+            for k in keys:
+                a, b = s1[k], s2[k]
+                if a.dtype != torch.float32:
+                    a, b = a.view(torch.uint8), b.view(torch.uint8)
+                assert torch.equal(a, b) or (torch.equal(a.isnan(), b.isnan()) and torch.equal(a.nan_to_num(), b.nan_to_num())), (i, sizes[i], step, k)
+
+
+def test_coatadamw_multi_tensor_switch_gives_the_same_trajectory(dev):
+    """CoatAdamW buckets the parameters of one dtype and step count into multi-tensor launches; with multi_tensor=False it
+    launches once per parameter like the reference.  Same parameters and state after five steps, two dtypes, a parameter
+    without gradient and one that joins late (its step count differs, so it gets a bucket of its own)."""
+    from coat_amd.optimizer.fp8_adamw import CoatAdamW
+    gen = torch.Generator().manual_seed(6)
+    shapes = [(64, 128), (300,), (4096,), (17, 33), (1,), (128,)]
+
+    def build():
+        g = torch.Generator().manual_seed(7)
+        ps = [torch.nn.Parameter((torch.randn(sh, generator=g) * 0.02).to(dev)) for sh in shapes]
+        ps += [torch.nn.Parameter((torch.randn(sh, generator=g) * 0.02).bfloat16().to(dev)) for sh in shapes[:3]]
+        return ps
+
+    pa, pb = build(), build()
+    oa = CoatAdamW(pa, lr=1e-3, weight_decay=0.05)
+    ob = CoatAdamW(pb, lr=1e-3, weight_decay=0.05, multi_tensor=False)
+    for step in range(5):
+        for i, (a, b) in enumerate(zip(pa, pb)):
+            if i == 1 or (i == 3 and step < 2):
+                a.grad = b.grad = None
+                continue
+            gr = (torch.randn(a.shape, generator=gen) * 1e-3).to(a.dtype).to(dev)
+            a.grad, b.grad = gr, gr.clone()
+        oa.step()
+        ob.step()
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)
+        sa, sb = oa.state[a], ob.state[b]
+        assert sa.keys() == sb.keys()
+        for k in sa:
+            x, y = sa[k], sb[k]
+            if x.dtype not in (torch.float32,):
+                x, y = x.view(torch.uint8), y.view(torch.uint8)
+            assert torch.equal(x, y), k

@@ -123,7 +123,19 @@ def test_argument_validation_of_the_remaining_entry_points_without_gpu():
     assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, pa, pn, 1, pa, 1, pa, 1, None, 0, 64, 64, 64, 16, None) == ESHAPE     # second scale output missing
     assert L.coat_fp8_gemm_grouped(2, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 64, 24, 16, None) == ESHAPE   # K % 16
     assert L.coat_fp8_gemm_grouped(3, pa, 0, pa, 0, pa, None, 0, pa, 1, pa, 1, None, 0, 64, 0, 64, 16, None) == 0         # empty
-    # RoPE, cross-entropy
+    # multi-tensor optimizer steps: host arrays of pointers and sizes
+    i64 = ctypes.c_int64
+    n1, g1, g0 = (i64 * 2)(128, 256), (i64 * 2)(1, 2), (i64 * 2)(1, 3)
+    hp = (0.9, 0.95, 1e-3, 0.1, 1e-8, 1)
+    assert L.coat_fp8_adamw_expand_step_multi(2, pa, pa, 0, pa, pa, pa, pa, pa, pa, pa, pa, n1, g1, *hp, 64, 16, None) == -4   # group size
+    assert L.coat_fp8_adamw_expand_step_multi(2, pa, pa, 0, pa, pa, pa, pa, pa, pa, pa, pa, n1, g0, *hp, 128, 16, None) == ESHAPE  # second scale count
+    assert L.coat_fp8_adamw_expand_step_multi(2, pa, pn, 0, pa, pa, pa, pa, pa, pa, pa, pa, n1, g1, *hp, 128, 16, None) == EINVAL  # second gradient missing
+    assert L.coat_fp8_adamw_expand_step_multi(2, pa, pa, 0, pa, pa, pa, None, pa, pa, pa, pa, n1, g1, *hp, 128, 16, None) == EINVAL  # no centre array
+    assert L.coat_fp8_adamw_expand_step_multi(2, po, pa, 0, pa, pa, pa, pa, pa, pa, pa, pa, n1, g1, *hp, 128, 16, None) == EALIGN  # second parameter misaligned
+    assert L.coat_fp8_adamw_expand_step_multi(2, pa, pa, 7, pa, pa, pa, pa, pa, pa, pa, pa, n1, g1, *hp, 128, 16, None) == -3   # dtype
+    assert L.coat_fp8_adamw_step_multi(-1, pa, pa, 0, pa, pa, pa, pa, n1, g1, *hp, 128, None) == EINVAL
+    assert L.coat_fp8_adamw_step_multi(0, None, None, 0, None, None, None, None, None, None, *hp, 128, None) == 0            # nothing to do
+    assert L.coat_fp8_adamw_step_multi(2, pn, pn, 0, pn, pn, pn, pn, (i64 * 2)(0, 0), (i64 * 2)(0, 0), *hp, 128, None) == 0   # only empty tensors
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 24, 0, 0, 0, None, 0, None) == ESHAPE             # head_dim % 16
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 48, 0, None, 0, None) == ESHAPE            # pitch < heads * head_dim
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 0, 0, p, 7, None) == EINVAL                # unknown format for the maximum
