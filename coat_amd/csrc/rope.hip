@@ -17,7 +17,9 @@
 
 namespace coat {
 
-template <int MAXKIND>  // -1: no maximum; kE4M3 / kE5M2: merge the largest group scale of y for that format into s_max
+// MAXKIND: -1 no maximum; kE4M3 / kE5M2: merge the largest group scale of y for that format into s_max.
+// COPY: no rotation, y = x (for the part of a fused q / k / v gradient that has no rotary embedding but shares the maximum)
+template <int MAXKIND, bool COPY>
 __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab,
                                                     int64_t n_pos, float theta, const int64_t* __restrict__ pos,
@@ -37,7 +39,9 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
         const uint16_t* src = x + row * x_pitch + head * head_dim + c * 8;
         const uint4 a = *(const uint4*)src, b = *(const uint4*)(src + half);
         float cs[8], sn[8];
-        if (p >= 0 && p < n_pos) {
+        if (COPY) {
+            // nothing to look up
+        } else if (p >= 0 && p < n_pos) {
             const float4* ct = (const float4*)(cos_tab + p * half + c * 8);
             const float4* st = (const float4*)(sin_tab + p * half + c * 8);
             const float4 c0 = ct[0], c1 = ct[1], s0 = st[0], s1 = st[1];
@@ -57,6 +61,11 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint16_t* __restrict__ 
         uint32_t o1[4], o2[4];
 #pragma unroll
         for (int k = 0; k < 4; k++) {
+            if (COPY) {
+                o1[k] = aw[k];
+                o2[k] = bw[k];
+                continue;
+            }
             const float x1l = bf16lo(aw[k]), x1h = bf16hi(aw[k]), x2l = bf16lo(bw[k]), x2h = bf16hi(bw[k]);
             const float sl = sign * sn[2 * k], sh = sign * sn[2 * k + 1];
             o1[k] = pack_bf16x2(x1l * cs[2 * k] - x2l * sl, x1h * cs[2 * k + 1] - x2h * sh);
@@ -85,6 +94,7 @@ extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, cons
                               const int64_t* pos, int64_t rows, int seq_len, int heads, int head_dim, int inverse,
                               int64_t x_pitch, int64_t y_pitch, float* s_max, int fp8_max, void* stream) {
     if (s_max && fp8_max != kE4M3 && fp8_max != kE5M2) return COAT_EINVAL;
+    if (inverse < 0 || inverse > 2) return COAT_EINVAL;
     if (rows < 0 || heads <= 0 || head_dim <= 0 || seq_len <= 0 || n_pos <= 0 || !(theta > 0.0f)) return COAT_EINVAL;
     if (!pos && seq_len > n_pos) return COAT_ESHAPE;  // positions 0 .. seq_len-1 must all be in the tables
     if (head_dim % 16 != 0) return COAT_ESHAPE;  // 8 pairs per lane
@@ -100,9 +110,13 @@ extern "C" int coat_rope_bf16(const void* x, void* y, const float* cos_tab, cons
     int64_t blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;
     if (s_max && blocks > 2048) blocks = 2048;  // one atomic per block: fewer, longer blocks
-    auto* kern = !s_max ? k_rope_bf16<-1> : fp8_max == kE4M3 ? k_rope_bf16<kE4M3> : k_rope_bf16<kE5M2>;
+    auto* kern = !s_max ? k_rope_bf16<-1, false> : fp8_max == kE4M3 ? k_rope_bf16<kE4M3, false> : k_rope_bf16<kE5M2, false>;
+    if (inverse == 2) {  // plain copy with the maximum
+        if (!s_max) return COAT_EINVAL;
+        kern = fp8_max == kE4M3 ? k_rope_bf16<kE4M3, true> : k_rope_bf16<kE5M2, true>;
+    }
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)x, (uint16_t*)y,
-                       cos_tab, sin_tab, n_pos, theta, pos, rows, seq_len, heads, head_dim, inverse ? -1.0f : 1.0f, x_pitch,
+                       cos_tab, sin_tab, n_pos, theta, pos, rows, seq_len, heads, head_dim, inverse == 1 ? -1.0f : 1.0f, x_pitch,
                        y_pitch, s_max);
     return coat_launch_status();
 }

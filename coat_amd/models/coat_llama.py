@@ -419,7 +419,7 @@ class _FusedQKVRoPE(torch.autograd.Function):
     neither the ``.contiguous()`` copies of the slices nor the concatenation of the three gradients are needed."""
 
     @staticmethod
-    def forward(ctx, qkv, cos_tab, sin_tab, heads, kv_heads, head_dim, theta):
+    def forward(ctx, qkv, cos_tab, sin_tab, heads, kv_heads, head_dim, theta, grad_fp8=None):
         from .. import _hip
         B, S, W = qkv.shape
         Dq, Dkv = heads * head_dim, kv_heads * head_dim
@@ -436,6 +436,7 @@ class _FusedQKVRoPE(torch.autograd.Function):
                                       0, None, 0, st), "rope forward (k of qkv)")
         ctx.save_for_backward(cos_tab, sin_tab)
         ctx.dims = (B, S, heads, kv_heads, head_dim, theta)
+        ctx.grad_fp8 = grad_fp8
         v = qkv[..., Dq + Dkv:].view(B, S, kv_heads, head_dim).transpose(1, 2)
         return (q.view(B, S, heads, head_dim).transpose(1, 2), k.view(B, S, kv_heads, head_dim).transpose(1, 2), v)
 
@@ -452,19 +453,29 @@ class _FusedQKVRoPE(torch.autograd.Function):
         flat = dqkv.view(B * S, W)
         lib, st = _hip.lib(), _hip.stream(gq.device)
         tabs = (_hip.ptr(cos_tab), _hip.ptr(sin_tab), cos_tab.shape[0], theta, None)
-        _hip.check(lib.coat_rope_bf16(_hip.ptr(gq), _hip.ptr(flat[:, :Dq]), *tabs, B * S, S, heads, head_dim, 1, 0, W, None, 0, st),
+        # the consumer quantizes the fused gradient per tensor (reference coat_olmo.py:318-326 on the fused projection): the
+        # three kernels that write its parts merge the maximum of its group scales into one buffer
+        s_max = new_max(gq.device) if ctx.grad_fp8 is not None else None
+        mx = (_hip.ptr(s_max), _hip.fp8(ctx.grad_fp8) if s_max is not None else 0)
+        _hip.check(lib.coat_rope_bf16(_hip.ptr(gq), _hip.ptr(flat[:, :Dq]), *tabs, B * S, S, heads, head_dim, 1, 0, W, *mx, st),
                    "rope backward (q of qkv)")
         _hip.check(lib.coat_rope_bf16(_hip.ptr(gk), _hip.ptr(flat[:, Dq:Dq + Dkv]), *tabs, B * S, S, kv_heads, head_dim, 1, 0,
-                                      W, None, 0, st), "rope backward (k of qkv)")
-        dqkv[..., Dq + Dkv:].copy_(gv.transpose(1, 2).reshape(B, S, Dkv))
-        return dqkv, None, None, None, None, None, None
+                                      W, *mx, st), "rope backward (k of qkv)")
+        if s_max is not None:
+            gv = _hip.dense(gv.transpose(1, 2).to(torch.bfloat16))  # physically [B, S, kv_heads, head_dim]
+            _hip.check(lib.coat_rope_bf16(_hip.ptr(gv), _hip.ptr(flat[:, Dq + Dkv:]), *tabs, B * S, S, kv_heads, head_dim, 2, 0,
+                                          W, *mx, st), "copy with maximum (v of qkv)")
+            tag_scale_max(dqkv, s_max, ctx.grad_fp8)
+        else:
+            dqkv[..., Dq + Dkv:].copy_(gv.transpose(1, 2).reshape(B, S, Dkv))
+        return dqkv, None, None, None, None, None, None, None
 
 
-def fused_qkv_rotary(qkv, heads, kv_heads, head_dim, theta):
+def fused_qkv_rotary(qkv, heads, kv_heads, head_dim, theta, grad_fp8=None):
     """RoPE on the q and k parts of a fused projection output qkv [B, S, (heads + 2 kv_heads) * head_dim] (bf16, GPU);
-    returns (q [B, heads, S, hd], k [B, kv_heads, S, hd], v [B, kv_heads, S, hd])."""
+    returns (q [B, heads, S, hd], k [B, kv_heads, S, hd], v [B, kv_heads, S, hd]).  ``grad_fp8`` as in ``fused_rotary``."""
     cos_tab, sin_tab = rotary_tables(qkv.shape[1], head_dim, theta, qkv.device)
-    return _FusedQKVRoPE.apply(qkv, cos_tab, sin_tab, heads, kv_heads, head_dim, float(theta))
+    return _FusedQKVRoPE.apply(qkv, cos_tab, sin_tab, heads, kv_heads, head_dim, float(theta), grad_fp8)
 
 
 def fused_rotary(x, heads, head_dim, theta, position_ids=None, max_positions=None, grad_fp8=None):

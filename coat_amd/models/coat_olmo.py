@@ -21,7 +21,7 @@ from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_If
                                             fp8_linear_forward_add,
                                             fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
                                             fp8_silu_mul_backward_joined, fp8_silu_mul_forward, fp8_transpose)
-from ..activation.real_quantization.common import scale_max
+from ..activation.real_quantization.common import convert_str_to_fp8, new_max, scale_max, tag_scale_max
 from ..utils._fp8_quantization_config import QuantizationConfig
 from .coat_llama import (E4M3, _as_e4m3_input, _as_e5m2_grad, _backward_weight_t, _forward_weight, _ResidualBase,
                          apply_rotary_pos_emb, fused_qkv_rotary, fused_rotary, rotary_cos_sin)
@@ -127,7 +127,7 @@ class CoatOLMoAfterAttentionResidual(_ResidualBase):
 class _CoatOLMoAfterAttentionResidual(torch.autograd.Function):
     @staticmethod
     def forward(ctx, re_x, flash_x, w2_origin, w2, w2_t, w2_s, group_size, fwobits, layer_id, config, qargs):
-        flash_qx, flash_s, _ = fp8_quantize_pertensor(flash_x, group_size, fwobits["fabit"])
+        flash_qx, flash_s, _ = fp8_quantize_pertensor(flash_x, group_size, fwobits["fabit"], want_pg=False)
         # projection + residual addition (fp8_linear_forward then fp8_add_Ifp_Ifp_Ofp_Og16 in the reference) in one kernel
         fp_x, (out_x, out_s) = fp8_linear_forward_add(flash_qx, flash_s, _forward_weight(w2_origin, w2, w2_s, qargs, fwobits),
                                                       w2_s, re_x, flash_qx.dtype, group_size)
@@ -242,6 +242,9 @@ class CoatOLMoSequentialBlock(nn.Module):
         self.layer_id = layer_id
         self.config = config
         self.qargs = QuantizationConfig(**config.coat_fp8_args) if qargs is None else qargs
+        # formats in which the neighbouring modules quantize the attention output and the fused q / k / v gradient per tensor
+        self._out_fp8 = convert_str_to_fp8[self.qargs.fabit]
+        self._grad_fp8 = convert_str_to_fp8[self.qargs.babit]
         self.hidden_size = config.mlp_hidden_size if config.mlp_hidden_size is not None else config.mlp_ratio * config.d_model
         head_dim = config.d_model // config.n_heads
         self.fused_dims = (config.d_model, config.effective_n_kv_heads * head_dim, config.effective_n_kv_heads * head_dim)
@@ -281,10 +284,15 @@ class CoatOLMoSequentialBlock(nn.Module):
         if k.size(1) != q.size(1):
             rep = q.size(1) // k.size(1)
             k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
-        att = sdpa(q, k, v, attn_mask=attention_bias,
-                                             dropout_p=self.config.attention_dropout if self.training else 0.0,
-                                             is_causal=attention_bias is None)
-        return att.transpose(1, 2).contiguous().view(B, T, C)
+        # in training the next module quantizes this output per tensor: the attention kernel hands it the scale maximum
+        out_max = new_max(q.device) if self.training and q.is_cuda else None
+        att = sdpa(q, k, v, attn_mask=attention_bias, dropout_p=self.config.attention_dropout if self.training else 0.0,
+                   is_causal=attention_bias is None, out_scale_max=out_max, out_fp8=self._out_fp8)
+        att, used_max = att if out_max is not None else (att, False)
+        att = att.transpose(1, 2).contiguous().view(B, T, C)
+        if used_max:
+            tag_scale_max(att, out_max, self._out_fp8)
+        return att
 
     def forward(self, x, qx, sx, attention_bias=None, layer_past=None, use_cache=False, max_doc_len=None,
                 cu_doc_lens=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, None]:
@@ -300,7 +308,7 @@ class CoatOLMoSequentialBlock(nn.Module):
             C = self.fused_dims[0]
             hd = C // self.config.n_heads
             q, k, v = fused_qkv_rotary(qkv, self.config.n_heads, self.config.effective_n_kv_heads, hd,
-                                       self.config.rope_theta)
+                                       self.config.rope_theta, self._grad_fp8 if self.training else None)
             att = self._sdpa(q, k, v, attention_bias, B, T, C)
         else:
             q, k, v = qkv.split(self.fused_dims, dim=-1)

@@ -259,7 +259,9 @@ int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_d
  * of 8 (16-byte rows), for x or y that is a column slice of a fused q/k/v tensor (coat/models/coat_olmo.py:1003-1006).
  * s_max (may be NULL): a COAT_MAX_WORDS buffer as above; the kernel merges (max|y| + 1e-10) / fp8max of format fp8_max
  * into it, which is what coat_fp8_group_scales would merge for y with any group size, so a caller that quantizes the
- * rotated tensor per tensor (the gradients at coat/models/coat_llama.py:318-326) skips that pass. */
+ * rotated tensor per tensor (the gradients at coat/models/coat_llama.py:318-326) skips that pass.  inverse == 2 (needs s_max):
+ * no rotation, y = x with the maximum merged, for the v part of a fused q / k / v gradient (coat/models/coat_olmo.py:1003-1006),
+ * whose three parts are quantized as one tensor. */
 int coat_rope_bf16(const void* x, void* y, const float* cos_tab, const float* sin_tab, int64_t n_pos, float theta,
                    const int64_t* pos, int64_t rows, int seq_len, int heads, int head_dim, int inverse, int64_t x_pitch,
                    int64_t y_pitch, float* s_max, int fp8_max, void* stream);

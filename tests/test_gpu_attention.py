@@ -150,3 +150,32 @@ def test_layer_quantizations_fed_by_handed_over_maxima_are_bit_identical(dev, mo
         assert len(calls) == n + 1
         for x, y in zip(a, b):
             assert torch.equal(x.view(torch.uint8) if x.dtype != torch.bfloat16 else x, y.view(torch.uint8) if y.dtype != torch.bfloat16 else y)
+
+
+def test_fused_qkv_gradient_arrives_with_the_maximum_of_all_three_parts(dev):
+    """OLMo's fused projection: the backward of fused_qkv_rotary writes dq and dk (inverse rotations) and dv (copy) into one
+    gradient and all three kernels merge into one maximum buffer; quantizing that gradient per tensor with and without the
+    hand-over gives the same codes and scale, whichever part holds the largest value."""
+    from coat_amd.activation.real_quantization import fp8_quantize_pertensor_transpose
+    from coat_amd.activation.real_quantization.common import known_scale_max
+    from coat_amd.models.coat_llama import fused_qkv_rotary
+    B, S, H, KV, D = 2, 96, 4, 2, 128
+    g = torch.Generator().manual_seed(13)
+    for big in range(3):  # the largest gradient sits in q, then k, then v
+        qkv = torch.randn(B, S, (H + 2 * KV) * D, generator=g).bfloat16().to(dev).requires_grad_(True)
+        seen = {}
+        qkv.register_hook(lambda gr: seen.__setitem__("g", gr))
+        q, k, v = fused_qkv_rotary(qkv, H, KV, D, 10000.0, grad_fp8=torch.float8_e5m2)
+        grads = [torch.randn(t.shape, generator=g).bfloat16().to(dev) * (8.0 if i == big else 1.0) for i, t in enumerate((q, k, v))]
+        torch.autograd.backward([q, k, v], grads)
+        gr = seen["g"]
+        assert known_scale_max(gr, torch.float8_e5m2) is not None
+        a = fp8_quantize_pertensor_transpose(gr, 16, "E5M2", transpose_output_2d=True)
+        b = fp8_quantize_pertensor_transpose(gr.detach().clone(), 16, "E5M2", transpose_output_2d=True)
+        assert torch.equal(a[0].view(torch.uint8), b[0].view(torch.uint8)) and torch.equal(a[1], b[1])
+        assert torch.equal(a[2].view(torch.uint8), b[2].view(torch.uint8))
+        # and the gradient itself equals the one of the untagged path
+        qkv2 = qkv.detach().clone().requires_grad_(True)
+        q2, k2, v2 = fused_qkv_rotary(qkv2, H, KV, D, 10000.0)
+        torch.autograd.backward([q2, k2, v2], grads)
+        assert torch.equal(qkv2.grad, gr)
