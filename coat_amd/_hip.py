@@ -57,6 +57,8 @@ SIGNATURES = {
     "coat_fp8_layernorm_forward": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _f, _vp],
     "coat_fp8_layernorm_backward": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i,
                                     _vp],
+    "coat_fp8_layernorm_backward_add": [_vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i,
+                                        _i64, _i64, _i, _vp],
     "coat_fp8_silu_mul_forward": [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i64, _i64, _vp],
     "coat_fp8_silu_mul_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _i64,
                                    _i64, _i64, _vp],

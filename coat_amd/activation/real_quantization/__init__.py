@@ -9,7 +9,8 @@ from ._quantize_transpose import fp8_quantize_transpose
 from ._transpose import fp8_transpose
 from .add_bwd import fp8_add_Ifp_Ifp_Ofp_Opt
 from .add_fwd import fp8_add_Ifp_Ifp_Ofp_Og16
-from .func_layernorm_noparam import fp8_layernorm_noparam_backward, fp8_layernorm_noparam_forward
+from .func_layernorm_noparam import (fp8_layernorm_noparam_backward, fp8_layernorm_noparam_backward_add,
+                                     fp8_layernorm_noparam_forward)
 from .func_layernorm_param import fp8_layernorm_param_backward, fp8_layernorm_param_forward
 from .silu_mul import (fp8_silu_mul_backward, fp8_silu_mul_backward_joined, fp8_silu_mul_forward,
                        fp8_silu_mul_forward_from_bf16)

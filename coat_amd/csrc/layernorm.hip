@@ -99,13 +99,24 @@ __global__ __launch_bounds__(256) void k_layernorm_fwd(const uint8_t* __restrict
 
 // Backward: wdy = w * dy; dx = bf16((wdy - (xhat * mean(xhat * wdy) + mean(wdy))) * rstd);
 // per-block partials of dw = sum_rows dy * xhat and db = sum_rows dy (affine variant only).
-template <int KIND, int WMODE, int ITERS>
-__global__ __launch_bounds__(256) void k_layernorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
-                                                        const void* __restrict__ dy, const void* __restrict__ w,
-                                                        const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
-                                                        void* __restrict__ dx, float* __restrict__ dw_partial,
-                                                        float* __restrict__ db_partial, int64_t M, int N, int qb) {
+// ADD: the residual-gradient addition that follows in the block (reference add_bwd.py:107-135 after
+// func_layernorm_noparam.py:248-297, coat/models/coat_olmo.py:318-339) happens here: dx is rounded to bf16 as it would be
+// stored, `radd` (bf16 [M, N]) is added in fp32, and what goes out is bf16 of the sum, the bf16 scale (amax + 1e-10) / fp8max of
+// every 1 x qb group of the fp32 sum and the maximum of those scales (fp32) for the per-tensor division that follows.
+struct LnAddArgs {
+    const void* radd;   // bf16 [M, N]
+    void* s_pg;         // bf16 [M, N / qb]
+    float* s_max;       // COAT_MAX_WORDS
+    int kind_out;       // kE4M3 / kE5M2: the FP8 format the scales are for
+};
+template <int KIND, int WMODE, int ITERS, bool ADD>
+__device__ __forceinline__ void layernorm_bwd_body(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                    const void* __restrict__ dy, const void* __restrict__ w,
+                                                    const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+                                                    void* __restrict__ dx, float* __restrict__ dw_partial,
+                                                    float* __restrict__ db_partial, int64_t M, int N, int qb, const LnAddArgs& A) {
     __shared__ float smem[4];
+    float block_max = 0.0f;  // ADD: largest group scale this thread has seen
     constexpr bool kAffine = WMODE != kNoParam;
     float accw[kAffine ? ITERS : 1][16], accb[kAffine ? ITERS : 1][16];
     if (kAffine) {
@@ -118,10 +129,16 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd(const uint8_t* __restrict
         const int64_t row_off = row * N, srow_off = row * (N / qb);
         const float mean = mean_in[row], rstd = rstd_in[row];
         float xhat[ITERS][16], wdy[ITERS][16];
+        uint4 ra[ADD ? ITERS : 1][2];  // ADD: the residual gradient's chunks, requested before the row is reduced
         float dot = 0.0f, sum = 0.0f;
 #pragma unroll
         for (int it = 0; it < ITERS; it++) {
             const int col = (threadIdx.x + it * 256) * 16;
+            if (ADD) {  // unconditional load from a clamped column (a load under a branch is waited for on the spot)
+                const uint4* rp = (const uint4*)((const uint16_t*)A.radd + row_off + (col < N ? col : 0));
+                ra[it][0] = rp[0];
+                ra[it][1] = rp[1];
+            }
             if (col < N) {
                 float xv[16], wv[16], gv[16];
                 dequant16<KIND>(q, s, s_dt, row_off, srow_off, col, qb, xv);
@@ -145,13 +162,42 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd(const uint8_t* __restrict
 #pragma unroll
         for (int it = 0; it < ITERS; it++) {
             const int col = (threadIdx.x + it * 256) * 16;
+            float gm = 0.0f;  // ADD: max |sum| of this thread's chunk (0 past the row's end)
             if (col < N) {
                 float o[16];
 #pragma unroll
                 for (int i = 0; i < 16; i++) o[i] = (wdy[it][i] - (xhat[it][i] * c1 + c2)) * rstd;
+                if (ADD) {
+                    const uint32_t rw[8] = {ra[it][0].x, ra[it][0].y, ra[it][0].z, ra[it][0].w,
+                                            ra[it][1].x, ra[it][1].y, ra[it][1].z, ra[it][1].w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        o[2 * i] = bf16lo(rw[i]) + round_to<kBF16>(o[2 * i]);
+                        o[2 * i + 1] = bf16hi(rw[i]) + round_to<kBF16>(o[2 * i + 1]);
+                    }
+                }
                 store_bf16_16(dx, row_off + col, o);
+                if (ADD) {
+                    float am = fmaxf(fabsf(o[0]), fabsf(o[1]));
+#pragma unroll
+                    for (int i = 2; i < 16; i++) am = fmaxf(am, fabsf(o[i]));
+                    gm = am;
+                }
+            }
+            if (ADD) {  // neighbouring threads hold neighbouring chunks: a group of qb columns is qb / 16 lanes
+                const int lpg = qb >> 4;
+                const float am = cluster_max_rt(gm, lpg);
+                const float sg = A.kind_out == kE5M2 ? group_scale<kE5M2>(am) : group_scale<kE4M3>(am);
+                if (col < N) {
+                    if ((threadIdx.x & (lpg - 1)) == 0) ((uint16_t*)A.s_pg)[row * (N / qb) + col / qb] = (uint16_t)f2bf16(sg);
+                    block_max = fmaxf(block_max, sg);
+                }
             }
         }
+    }
+    if (ADD) {
+        __syncthreads();  // the last row's sums may still be read from smem
+        block_atomic_max_nonneg(A.s_max, block_max, smem);
     }
     if (kAffine) {
 #pragma unroll
@@ -168,6 +214,23 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd(const uint8_t* __restrict
             }
         }
     }
+}
+
+template <int KIND, int WMODE, int ITERS>
+__global__ __launch_bounds__(256) void k_layernorm_bwd(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                        const void* __restrict__ dy, const void* __restrict__ w,
+                                                        const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+                                                        void* __restrict__ dx, float* __restrict__ dw_partial,
+                                                        float* __restrict__ db_partial, int64_t M, int N, int qb) {
+    layernorm_bwd_body<KIND, WMODE, ITERS, false>(q, s, s_dt, dy, w, mean_in, rstd_in, dx, dw_partial, db_partial, M, N, qb, LnAddArgs{});
+}
+template <int KIND, int WMODE, int ITERS>
+__global__ __launch_bounds__(256) void k_layernorm_bwd_add(const uint8_t* __restrict__ q, const void* __restrict__ s, int s_dt,
+                                                            const void* __restrict__ dy, const void* __restrict__ w,
+                                                            const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+                                                            void* __restrict__ dx, float* __restrict__ dw_partial,
+                                                            float* __restrict__ db_partial, int64_t M, int N, int qb, LnAddArgs A) {
+    layernorm_bwd_body<KIND, WMODE, ITERS, true>(q, s, s_dt, dy, w, mean_in, rstd_in, dx, dw_partial, db_partial, M, N, qb, A);
 }
 
 }  // namespace coat
@@ -218,13 +281,15 @@ extern "C" int coat_fp8_layernorm_forward(const void* x, int fp8, const void* s_
     return coat_launch_status();
 }
 
-extern "C" int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
-                                           const void* w, int w_dtype, const float* mean, const float* rstd, void* dx,
-                                           void* dw, void* db, float* dw_partial, float* db_partial, int n_partial,
-                                           int64_t M, int64_t N, int QB, void* stream) {
+static int layernorm_backward_common(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* w,
+                                     int w_dtype, const float* mean, const float* rstd, void* dx, void* dw, void* db,
+                                     float* dw_partial, float* db_partial, int n_partial, int64_t M, int64_t N, int QB,
+                                     const LnAddArgs* add, void* stream) {
     if (int e = ln_check(M, N, QB)) return e;
+    if (add && QB > 1024) return COAT_ESHAPE;  // a group's chunks sit in the lanes of one wave
     if (M * N == 0) return COAT_OK;
     if (!x || !s_x || !dy || !mean || !rstd || !dx) return COAT_EINVAL;
+    if (add && (!add->radd || !add->s_pg || !add->s_max || !coat_aligned16(add->radd))) return add->radd && add->s_pg && add->s_max ? COAT_EALIGN : COAT_EINVAL;
     if (w_dtype >= 0 && (!w || !dw || !db || !dw_partial || !db_partial || n_partial <= 0)) return COAT_EINVAL;
     if (s_dtype < 0 || s_dtype > 2) return COAT_EDTYPE;
     if (!coat_aligned16(x) || !coat_aligned16(w) || !coat_aligned16(dy) || !coat_aligned16(dx) ||
@@ -232,7 +297,11 @@ extern "C" int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s
         return COAT_EALIGN;
     hipStream_t st = (hipStream_t)stream;
     int64_t grid = w_dtype >= 0 ? (n_partial < M ? n_partial : M) : (M < 2048 ? M : 2048);
-    LN_DISPATCH(k_layernorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, mean, rstd, dx, dw_partial, db_partial, M, (int)N, QB)
+    if (add) {
+        LN_DISPATCH(k_layernorm_bwd_add, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, mean, rstd, dx, dw_partial, db_partial, M, (int)N, QB, *add)
+    } else {
+        LN_DISPATCH(k_layernorm_bwd, grid, (const uint8_t*)x, s_x, s_dtype, dy, w, mean, rstd, dx, dw_partial, db_partial, M, (int)N, QB)
+    }
     if (int e = coat_launch_status()) return e;
     if (w_dtype < 0) return COAT_OK;
     const int cols_blocks = (int)((N + kColsumCols - 1) / kColsumCols);
@@ -251,4 +320,23 @@ extern "C" int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s
             break;
     }
     return coat_launch_status();
+}
+
+extern "C" int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
+                                           const void* w, int w_dtype, const float* mean, const float* rstd, void* dx,
+                                           void* dw, void* db, float* dw_partial, float* db_partial, int n_partial,
+                                           int64_t M, int64_t N, int QB, void* stream) {
+    return layernorm_backward_common(x, fp8, s_x, s_dtype, dy, w, w_dtype, mean, rstd, dx, dw, db, dw_partial, db_partial,
+                                     n_partial, M, N, QB, nullptr, stream);
+}
+
+extern "C" int coat_fp8_layernorm_backward_add(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy,
+                                               const void* w, int w_dtype, const float* mean, const float* rstd,
+                                               const void* residual_grad, void* y, void* s_pg, float* s_max, int fp8_out,
+                                               void* dw, void* db, float* dw_partial, float* db_partial, int n_partial,
+                                               int64_t M, int64_t N, int QB, void* stream) {
+    if (fp8_out != COAT_E4M3 && fp8_out != COAT_E5M2) return COAT_EINVAL;
+    const LnAddArgs add{residual_grad, s_pg, s_max, fp8_out == COAT_E5M2 ? kE5M2 : kE4M3};
+    return layernorm_backward_common(x, fp8, s_x, s_dtype, dy, w, w_dtype, mean, rstd, y, dw, db, dw_partial, db_partial,
+                                     n_partial, M, N, QB, &add, stream);
 }

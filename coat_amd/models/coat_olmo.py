@@ -16,7 +16,7 @@ import torch.nn.functional as F
 
 from ._attention import sdpa
 from ..activation.real_quantization import (fp8_add_Ifp_Ifp_Ofp_Og16, fp8_add_Ifp_Ifp_Ofp_Opt,
-                                            fp8_division_transpose, fp8_layernorm_noparam_backward,
+                                            fp8_division_transpose, fp8_layernorm_noparam_backward, fp8_layernorm_noparam_backward_add,
                                             fp8_layernorm_noparam_forward, fp8_linear_backward, fp8_linear_forward,
                                             fp8_linear_forward_add,
                                             fp8_quantize_pertensor, fp8_quantize_pertensor_transpose,
@@ -103,9 +103,9 @@ class _CoatOLMoBeforeAttentionResidual(torch.autograd.Function):
                                                                         transpose_output_2d=True, stochastic=False)
         w1_t = _backward_weight_t(w_saved, w1_s, qargs, fwobits)
         fc1_g, att_proj_wg = fp8_linear_backward(ln_x_t, ln_s, flash_g, flash_gs, flash_g_t, w1_t, w1_s, group_size)
-        in_g = fp8_layernorm_noparam_backward(in_x, in_s, fc1_g, group_size, mean, rstd, num_warps)
-        re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],
-                                                                stochastic=False)
+        # fp8_layernorm_noparam_backward + fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g) of the reference, the addition inside the kernel
+        re_g, (in_g, in_sg, in_sg_g16) = fp8_layernorm_noparam_backward_add(in_x, in_s, fc1_g, group_size, mean, rstd, num_warps,
+                                                                          fp_grad, fwobits["babit"], stochastic=False)
         return re_g, in_g.view(E4M3), in_sg_g16, att_proj_wg, None, None, None, None, None, None, None, None, None
 
 
@@ -222,9 +222,9 @@ class _CoatOLMoMLPResidual(torch.autograd.Function):
                                                                        group_size, fwobits["babit"])
         w1_t = _backward_weight_t(w1_saved, w1_s, qargs, fwobits)
         fc1_g, weight1_grad = fp8_linear_backward(ln_x_t, ln_s, gateup_g, gateup_gs, gateup_g_t, w1_t, w1_s, group_size)
-        in_g = fp8_layernorm_noparam_backward(in_x, in_s, fc1_g, group_size, mean, rstd, num_warps)
-        re_g, (in_g, in_sg, in_sg_g16) = fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g, group_size, fwobits["babit"],
-                                                                stochastic=False)
+        # fp8_layernorm_noparam_backward + fp8_add_Ifp_Ifp_Ofp_Opt(fp_grad, in_g) of the reference, the addition inside the kernel
+        re_g, (in_g, in_sg, in_sg_g16) = fp8_layernorm_noparam_backward_add(in_x, in_s, fc1_g, group_size, mean, rstd, num_warps,
+                                                                          fp_grad, fwobits["babit"], stochastic=False)
         return (re_g, in_g.view(E4M3), in_sg_g16, weight1_grad, None, None, None, weight2_grad, None, None, None,
                 None, None, None, None, None, None)
 

@@ -48,7 +48,7 @@ enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.f
 /* Bumped whenever an entry point's argument list or the size of a buffer it writes changes (2: every s_max / amax
  * argument became COAT_MAX_WORDS words; 3: coat_fp8_gemm_residual, coat_fp8_rmsnorm_backward_add and coat_attention_forward_bf16 added,
  * coat_hbm_probe removed; 4: coat_rope_bf16 and coat_attention_forward_bf16 take a maximum buffer, the multi-tensor optimizer
- * steps added).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
+ * steps and coat_fp8_layernorm_backward_add added).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
  * loads the library. */
 #define COAT_ABI_VERSION 4
 int coat_abi_version(void);
@@ -247,6 +247,16 @@ int coat_fp8_layernorm_backward(const void* x, int fp8, const void* s_x, int s_d
                                 int w_dtype, const float* mean, const float* rstd, void* dx, void* dw, void* db,
                                 float* dw_partial, float* db_partial, int n_partial, int64_t M, int64_t N, int QB,
                                 void* stream);
+
+/* coat_fp8_layernorm_backward followed by the value pass of fp8_add_Ifp_Ifp_Ofp_Opt (rq/add_bwd.py:147; the sequence at
+ * coat/models/coat_olmo.py:318-339) in one kernel, like coat_fp8_rmsnorm_backward_add: dx is rounded to bf16 as it would be
+ * stored, residual_grad (bf16 [M, N]) is added in fp32; y receives bf16 of the sum, s_pg [M, N / QB] the bf16 scales
+ * (amax + 1e-10) / fp8max of its 1 x QB groups for format fp8_out, s_max (COAT_MAX_WORDS) their maximum;
+ * coat_fp8_division_from_max of y gives the per-tensor codes.  Bit-identical to the two entry points. */
+int coat_fp8_layernorm_backward_add(const void* x, int fp8, const void* s_x, int s_dtype, const void* dy, const void* w,
+                                    int w_dtype, const float* mean, const float* rstd, const void* residual_grad, void* y,
+                                    void* s_pg, float* s_max, int fp8_out, void* dw, void* db, float* dw_partial,
+                                    float* db_partial, int n_partial, int64_t M, int64_t N, int QB, void* stream);
 
 /* Rotary position embedding of the bf16 attention (no single counterpart in the reference, which applies it with
  * several torch kernels: transformers' apply_rotary_pos_emb as called at coat/models/coat_llama.py:1029-1030, olmo's

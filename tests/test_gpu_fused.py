@@ -309,6 +309,33 @@ def test_rmsnorm_backward_with_residual_addition_equals_the_two_kernels(dev, M, 
         assert torch.equal(b(got_q), oq.view(torch.uint8))
 
 
+@pytest.mark.parametrize("M,N,QBv,fp8out", [(208, 512, 16, "E5M2"), (1504, 4096, 16, "E5M2"), (64, 4096 + 64, 32, "E4M3"),
+                                              (48, 8192 + 128, 128, "E5M2"), (16, 16384, 16, "E5M2")])
+def test_layernorm_backward_with_residual_addition_equals_the_two_kernels(dev, M, N, QBv, fp8out):
+    """fp8_layernorm_noparam_backward_add against fp8_layernorm_noparam_backward followed by fp8_add_Ifp_Ifp_Ofp_Opt: the
+    bf16 sum, the per-group scales, the per-tensor scale and the codes, bit for bit, and the addition itself against the
+    oracle.  Widths take the one-, two- and four-chunk kernels, group sizes from one to eight lanes."""
+    rq = _rq()
+    from coat_amd.activation.real_quantization import fp8_layernorm_noparam_backward_add
+    x = rand(80, shape=(M, N))
+    g = rand(81, 0.01, shape=(M, N)).to(dev)
+    res = rand(82, 0.02, shape=(M, N))
+    res[::5, ::3] *= 30
+    res = res.to(dev)
+    q, s = rq.fp8_quantize(x.to(dev), QBv, "E4M3")
+    _, _, _, (mean, rstd, nw) = rq.fp8_layernorm_noparam_forward(q, s, QBv, 1e-5, transpose_output_2d=True)
+    dx = rq.fp8_layernorm_noparam_backward(q, s, g, QBv, mean, rstd, nw)
+    want_y, (want_q, want_s, want_pg) = rq.fp8_add_Ifp_Ifp_Ofp_Opt(res, dx, QBv, fp8out)
+    got_y, (got_q, got_s, got_pg) = fp8_layernorm_noparam_backward_add(q, s, g, QBv, mean, rstd, nw, res, fp8out)
+    assert torch.equal(got_y, want_y), "sum"
+    assert torch.equal(got_pg.view(torch.int16), want_pg.view(torch.int16)), "group scales"
+    assert got_s.dtype == want_s.dtype and got_s.item() == want_s.item(), "tensor scale"
+    assert torch.equal(b(got_q), b(want_q)), "codes"
+    oy, (oq, os_, opg) = R.fp8_add_Ifp_Ifp_Ofp_Opt(res.cpu(), dx.cpu(), QBv, fp8out)
+    assert torch.equal(got_y.cpu(), oy) and torch.equal(got_pg.cpu(), opg) and os_.item() == got_s.item()
+    assert torch.equal(b(got_q), oq.view(torch.uint8))
+
+
 def test_larger_groups_and_float32_scales(dev):
     rq = _rq()
     x1, x2 = rand(13, shape=(128, 512)), rand(14, shape=(128, 512))
