@@ -136,6 +136,16 @@ def test_argument_validation_of_the_remaining_entry_points_without_gpu():
     assert L.coat_fp8_adamw_step_multi(-1, pa, pa, 0, pa, pa, pa, pa, n1, g1, *hp, 128, None) == EINVAL
     assert L.coat_fp8_adamw_step_multi(0, None, None, 0, None, None, None, None, None, None, *hp, 128, None) == 0            # nothing to do
     assert L.coat_fp8_adamw_step_multi(2, pn, pn, 0, pn, pn, pn, pn, (i64 * 2)(0, 0), (i64 * 2)(0, 0), *hp, 128, None) == 0   # only empty tensors
+    # fused norm backward + residual addition, attention forward
+    assert L.coat_fp8_layernorm_backward_add(p, 0, p, 1, p, None, -1, p, p, None, p, p, p, 1, None, None, None, None, 0, 16, 64, 16, None) == EINVAL  # no residual gradient
+    assert L.coat_fp8_layernorm_backward_add(p, 0, p, 1, p, None, -1, p, p, p, p, p, p, 5, None, None, None, None, 0, 16, 64, 16, None) == EINVAL     # unknown output format
+    assert L.coat_fp8_layernorm_backward_add(p, 0, p, 1, p, None, -1, p, p, odd, p, p, p, 1, None, None, None, None, 0, 16, 64, 16, None) == EALIGN
+    st = [64] * 12
+    assert L.coat_attention_forward_bf16(p, p, p, p, None, 1, 4, 4, 64, 64, *st, 0.1, 1, None, 0, None) == ESHAPE   # head dimension
+    assert L.coat_attention_forward_bf16(p, p, p, p, None, 1, 4, 3, 64, 128, *st, 0.1, 1, None, 0, None) == EINVAL  # heads % kv_heads
+    assert L.coat_attention_forward_bf16(p, p, p, p, None, 1, 4, 4, 64, 128, *st, 0.1, 1, p, 9, None) == EINVAL     # unknown format for the maximum
+    assert L.coat_attention_forward_bf16(p, p, p, p, None, 0, 4, 4, 64, 128, *st, 0.1, 1, None, 0, None) == 0       # empty batch
+    # RoPE, cross-entropy
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 24, 0, 0, 0, None, 0, None) == ESHAPE             # head_dim % 16
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 48, 0, None, 0, None) == ESHAPE            # pitch < heads * head_dim
     assert L.coat_rope_bf16(p, p, p, p, 8, 1e4, None, 8, 8, 2, 32, 0, 0, 0, p, 7, None) == EINVAL                # unknown format for the maximum
