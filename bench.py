@@ -619,6 +619,25 @@ def cpu_baseline_gemm(torch, which):
             "kind": "port", "sample": f"oracle/activation_ref.py fp8matmul on {rows} of the {M_} rows of the left operand, median of 3 runs"}
 
 
+def cpu_baseline_attention(torch):
+    """The oracle's attention (oracle/attention_ref.py: fp32 scores, mask, softmax and weighted sum written out) on 4 of the
+    128 (batch, head) pairs of the workload, all host threads, median of 3."""
+    from oracle import attention_ref
+
+    S, D, heads = 2048, 128, 4
+    gen = torch.Generator().manual_seed(0)
+    q, k, v = [torch.randn(1, heads, S, D, generator=gen).bfloat16() for _ in range(3)]
+    attention_ref.attention(q, k, v)
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        attention_ref.attention(q, k, v)
+        ts.append(time.perf_counter() - t0)
+    flops = 2 * 2 * heads * S * S * D // 2  # the same count as the GPU leg: the visible half
+    return {"value": round(flops / _median(ts) / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle/attention_ref.py on {heads} of the 128 (batch, head) pairs (2048 tokens, head dimension 128), median of 3 runs"}
+
+
 def cpu_baseline_silu_mul(torch, nbytes_full):
     """The oracle's chain (quantize x 2, SiLU, mul, mul backward, SiLU backward, all with their per-tensor divisions) on a
     256-row slab of the [8192, 11008] inputs, all host threads, median of 3."""
@@ -911,6 +930,8 @@ def measure_stream(name, args, dev, torch, cpu):
             rec["cpu_baseline"] = cpu_baseline_silu_mul(torch, nbytes)
         elif name == "rmsnorm":
             rec["cpu_baseline"] = cpu_baseline_rmsnorm(torch, nbytes)
+        elif name == "attention":
+            rec["cpu_baseline"] = cpu_baseline_attention(torch)
     return rec
 
 
