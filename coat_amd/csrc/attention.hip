@@ -101,14 +101,16 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
     const v4i_t v_rsrc = attn_rsrc(vbase, (uint32_t)(((int64_t)(A.seq - 1) * A.v_ss + kHeadDim) * 2));
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr3_t)lds;
     // one instruction = 4 rows (keys) of 256 bytes; lane i fills position i % 16 of row i / 16 with the chunk that belongs
-    // there: K position p holds chunk p ^ (row & 15); V position p holds chunk ((p / 2) ^ (row & 7)) * 2 + p % 2 (32-byte
-    // pieces stay whole: a transposing read takes 32 contiguous bytes of each of 4 keys).  Keys past the end read zeros.
+    // there: K position p holds chunk p ^ (row & 15); V position p holds chunk ((p / 2) ^ 2 (row & 3)) * 2 + p % 2 (32-byte
+    // pieces stay whole: a transposing read takes 32 contiguous bytes of each of 4 keys; the two 16-lane groups that are
+    // served together read an even and an odd piece of the same 4 keys, and the swizzle by twice the key keeps the four even
+    // and the four odd pieces apart: all 64 banks once).  Keys past the end read zeros.
     int k_off[4], v_off[4];
 #pragma unroll
     for (int x = 0; x < 4; x++) {
         const int row = 4 * (4 * wave + x) + (lane >> 4), p = lane & 15;
         k_off[x] = row * (int)(A.k_ss * 2) + ((p ^ (row & 15)) << 4);
-        v_off[x] = row * (int)(A.v_ss * 2) + ((((((p >> 1) ^ (row & 7)) << 1) | (p & 1))) << 4);
+        v_off[x] = row * (int)(A.v_ss * 2) + ((((((p >> 1) ^ ((row & 3) << 1)) << 1) | (p & 1))) << 4);
     }
     auto issue_tile = [&](int t, int stage) {
         const uint32_t kdst = lds_base + stage * kStageBytes + (4 * wave) * 1024;
@@ -133,8 +135,8 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
     auto v_frag = [&](int stage, int dt, int j) -> v8bf {
         const int dim = 32 * dt + tr_dim, key = 16 * j + tr_key;
         const uint8_t* base = lds + stage * kStageBytes + kKTileBytes + ((dim & 15) << 1);
-        const uint8_t* a0 = base + key * 256 + (((dim >> 4) ^ (key & 7)) << 5);
-        const uint8_t* a1 = base + (key + 4) * 256 + (((dim >> 4) ^ ((key + 4) & 7)) << 5);
+        const uint8_t* a0 = base + key * 256 + (((dim >> 4) ^ ((key & 3) << 1)) << 5);
+        const uint8_t* a1 = a0 + 4 * 256;  // key + 4: the same piece
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a0);
         const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a1);
         typedef short v8s __attribute__((ext_vector_type(8)));
@@ -168,6 +170,8 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
         ATTN_WAIT_VMCNT0();               // this wave's part of tile t has landed
         __builtin_amdgcn_s_barrier();     // ... and everybody's; everybody is also done reading tile t - 1
         asm volatile("" ::: "memory");
+        // the next tile's loads go out first: issued behind this tile's score products instead (so that the four waves do
+        // not queue 32 KiB at the address unit together) they land too late, 196 us against 182 us
         if (t + 1 < nsteps) issue_tile(t + 1, stage ^ 1);
         const int key0 = t * kTileK;
         // waves whose queries all lie before this tile have nothing to add (causal); they still take part in the loads
