@@ -25,6 +25,8 @@
 // longest first (under the causal mask a block's work grows with its position).
 #include <math.h>
 
+#include <type_traits>
+
 #include "coat_device.h"
 #include "coat_host.h"
 
@@ -60,6 +62,20 @@ __device__ __forceinline__ void attn_lds_dma16(v4i_t rsrc, uint32_t lds_addr, in
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc)
                  : "memory", "m0");
+}
+// Four such loads into four consecutive KiB of LDS with one M0 write: the instruction's immediate offset moves both the
+// LDS and the memory address on by 1024 per load, so the per-lane memory offsets are passed less that amount; `soff`
+// (the tile's offset) is added to the memory address only and takes no part in the range check.
+__device__ __forceinline__ void attn_lds_dma16x4(v4i_t rsrc, uint32_t lds_addr, int v0, int v1, int v2, int v3, int soff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %5, %6 offen lds\n\t"
+        "buffer_load_dwordx4 %2, %5, %6 offen offset:1024 lds\n\t"
+        "buffer_load_dwordx4 %3, %5, %6 offen offset:2048 lds\n\t"
+        "buffer_load_dwordx4 %4, %5, %6 offen offset:3072 lds"
+        :
+        : "s"(lds_addr), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(rsrc), "s"(soff)
+        : "memory", "m0");
 }
 __device__ __forceinline__ v4i_t attn_rsrc(const void* p, uint32_t bytes) {
     const uint64_t a = (uint64_t)p;
@@ -112,19 +128,38 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
         k_off[x] = row * (int)(A.k_ss * 2) + ((p ^ (row & 15)) << 4);
         v_off[x] = row * (int)(A.v_ss * 2) + ((((((p >> 1) ^ ((row & 3) << 1)) << 1) | (p & 1))) << 4);
     }
+    // per-lane offsets for the four-load form (less the immediate offsets; a row is at least 256 bytes, so none is negative)
+    int k_off4[4], v_off4[4];
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+        k_off4[x] = k_off[x] - 1024 * x;
+        v_off4[x] = v_off[x] - 1024 * x;
+    }
     auto issue_tile = [&](int t, int stage) {
         const uint32_t kdst = lds_base + stage * kStageBytes + (4 * wave) * 1024;
         const uint32_t vdst = kdst + kKTileBytes;
         const int kt_off = t * kTileK * (int)(A.k_ss * 2), vt_off = t * kTileK * (int)(A.v_ss * 2);
+        if ((t + 1) * kTileK <= A.seq) {
+            // every key of the tile exists: the tile's offset travels in the scalar offset, outside the range check
+            attn_lds_dma16x4(k_rsrc, kdst, k_off4[0], k_off4[1], k_off4[2], k_off4[3], kt_off);
+            attn_lds_dma16x4(v_rsrc, vdst, v_off4[0], v_off4[1], v_off4[2], v_off4[3], vt_off);
+        } else {
+            // the last, partial tile: the whole offset per lane, so that keys past the end fall outside the buffer and read zeros
 #pragma unroll
-        for (int x = 0; x < 4; x++) attn_lds_dma16(k_rsrc, kdst + x * 1024, k_off[x] + kt_off);
+            for (int x = 0; x < 4; x++) attn_lds_dma16(k_rsrc, kdst + x * 1024, k_off[x] + kt_off);
 #pragma unroll
-        for (int x = 0; x < 4; x++) attn_lds_dma16(v_rsrc, vdst + x * 1024, v_off[x] + vt_off);
+            for (int x = 0; x < 4; x++) attn_lds_dma16(v_rsrc, vdst + x * 1024, v_off[x] + vt_off);
+        }
     };
-    // K fragment (A operand of S^T): row l32 (+ 32 kt), chunk 2 c + h32
-    auto k_frag = [&](int stage, int kt, int c) -> v8bf {
-        const int row = 32 * kt + l32;
-        return *(const v8bf*)(lds + stage * kStageBytes + row * 256 + (((2 * c + h32) ^ (row & 15)) << 4));
+    // K fragment (A operand of S^T): row l32 (+ 32 kt), chunk 2 c + h32.  The lane's byte offset inside a K tile is kept
+    // per chunk (the swizzle is not linear in c); stage and key half are compile-time constants and end up in the
+    // instruction's offset field, so a fragment read costs no address arithmetic.
+    uint32_t k_base[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) k_base[c] = l32 * 256 + (((2 * c + h32) ^ (l32 & 15)) << 4);
+    auto k_frag = [&](auto stage_c, int kt, int c) -> v8bf {
+        constexpr int stage = decltype(stage_c)::value;
+        return *(const v8bf*)(lds + k_base[c] + (stage * kStageBytes + kt * 32 * 256));
     };
     // V^T fragment (A operand of O^T): dimension 32 dt + l32, keys 16 j + 8 h32 .. + 7, through two transposing reads.
     // Within a group of 16 lanes, lane i points at key (16 j + 8 h32) + i / 4 (+ 4 for the second read), dimensions
@@ -132,10 +167,15 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) v4s* lds_v4s_ptr;
     const int tr_i = lane & 15, tr_dim = 16 * ((lane >> 4) & 1) + 4 * (tr_i & 3), tr_key = 8 * h32 + (tr_i >> 2);
-    auto v_frag = [&](int stage, int dt, int j) -> v8bf {
-        const int dim = 32 * dt + tr_dim, key = 16 * j + tr_key;
-        const uint8_t* base = lds + stage * kStageBytes + kKTileBytes + ((dim & 15) << 1);
-        const uint8_t* a0 = base + key * 256 + (((dim >> 4) ^ ((key & 3) << 1)) << 5);
+    uint32_t v_base[4];  // the lane's byte offset inside a V tile for dimension block dt, key block 0 (the swizzle is not linear in dt)
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        const int dim = 32 * dt + tr_dim;
+        v_base[dt] = ((dim & 15) << 1) + tr_key * 256 + (((dim >> 4) ^ ((tr_key & 3) << 1)) << 5);
+    }
+    auto v_frag = [&](auto stage_c, int dt, int j) -> v8bf {
+        constexpr int stage = decltype(stage_c)::value;
+        const uint8_t* a0 = lds + v_base[dt] + (stage * kStageBytes + kKTileBytes + j * 16 * 256);  // key 16 j + tr_key: same key & 3
         const uint8_t* a1 = a0 + 4 * 256;  // key + 4: the same piece
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a0);
         const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a1);
@@ -164,9 +204,9 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
     float m_ref = -INFINITY, l_run = 0.0f;
     const float c2 = A.scale_log2e;
 
-    issue_tile(0, 0);
-    for (int t = 0; t < nsteps; t++) {
-        const int stage = t & 1;
+    // One 64-key step; the ring stage is a compile-time constant (the loop below alternates two instances of this code).
+    auto step = [&](int t, auto stage_c) {
+        constexpr int stage = decltype(stage_c)::value;
         ATTN_WAIT_VMCNT0();               // this wave's part of tile t has landed
         __builtin_amdgcn_s_barrier();     // ... and everybody's; everybody is also done reading tile t - 1
         asm volatile("" ::: "memory");
@@ -175,7 +215,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
         if (t + 1 < nsteps) issue_tile(t + 1, stage ^ 1);
         const int key0 = t * kTileK;
         // waves whose queries all lie before this tile have nothing to add (causal); they still take part in the loads
-        if (CAUSAL && key0 > q0 + wave * 32 + 31) continue;
+        if (CAUSAL && key0 > q0 + wave * 32 + 31) return;
 
         // ---- S^T = K Q^T for the tile's 64 keys
         // The 16 K fragments are read four at a time, each batch while the previous one is multiplied: left to itself the
@@ -183,12 +223,12 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
         v16f s_acc[2];
         v8bf kf[2][4];
 #pragma unroll
-        for (int c = 0; c < 4; c++) kf[0][c] = k_frag(stage, 0, c);
+        for (int c = 0; c < 4; c++) kf[0][c] = k_frag(stage_c, 0, c);
 #pragma unroll
         for (int b = 0; b < 4; b++) {          // batch b: key half b / 2, dimension chunks 4 (b % 2) .. + 3
             if (b < 3) {
 #pragma unroll
-                for (int c = 0; c < 4; c++) kf[(b + 1) & 1][c] = k_frag(stage, (b + 1) >> 1, 4 * ((b + 1) & 1) + c);
+                for (int c = 0; c < 4; c++) kf[(b + 1) & 1][c] = k_frag(stage_c, (b + 1) >> 1, 4 * ((b + 1) & 1) + c);
             }
             __builtin_amdgcn_sched_barrier(0);
             const int kt = b >> 1;
@@ -265,8 +305,13 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
                 const v8bf pfrag = __builtin_bit_cast(v8bf, pw);
 #pragma unroll
                 for (int dt = 0; dt < 4; dt++)
-                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage, dt, 2 * kt + u), pfrag, o_acc[dt], 0, 0, 0);
+                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(stage_c, dt, 2 * kt + u), pfrag, o_acc[dt], 0, 0, 0);
             }
+    };
+    issue_tile(0, 0);
+    for (int t = 0; t < nsteps; t += 2) {
+        step(t, std::integral_constant<int, 0>{});
+        if (t + 1 < nsteps) step(t + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- normalise and store: the two half-waves hold the two parts of each query's sum
