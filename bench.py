@@ -566,14 +566,14 @@ def cpu_baseline_adamw(torch):
 # counters read for a 256 MiB copy).  The counters cannot be read inside this process: the figures come from the separate
 # profiling runs recorded under profiles/, not from this run.
 MEASURED_TRAFFIC = {
-    "adamw": (758.5e6, "profiles/k_fp8_adamw_expand__adamw_11008x4096.txt"),
+    "adamw": (760.3e6, "profiles/k_fp8_adamw_expand__adamw_11008x4096.txt"),
     "quantize": (52.5e6, "profiles/k_quantize_pg__quantize_4096x4096_bf16.txt"),
     "quantize_transpose": (73.6e6, "profiles/k_quantize_transpose__quantize_transpose_4096x4096_bf16.txt"),
-    "gemm_fwd": (743.1e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
-    "gemm_dgrad": (608.4e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
-    "cross_entropy": (2099.7e6, "profiles/k_cross_entropy__llama2_vocab32000_8192tok_fp32.txt"),
-    "silu_mul": (2616.7e6, "profiles/k_silu_mul__silu_mul_8192x11008.txt (the five launches of forward + backward together; two passes over the tensors)"),
-    "rmsnorm": (332.4e6, "profiles/k_rmsnorm__rmsnorm_8192x4096.txt (the four kernels of forward + backward together)"),
+    "gemm_fwd": (696.9e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
+    "gemm_dgrad": (561.4e6, "profiles/k_fp8_gemm__llama7b_mlp_8192tok.txt"),
+    "cross_entropy": (2100.3e6, "profiles/k_cross_entropy__llama2_vocab32000_8192tok_fp32.txt"),
+    "silu_mul": (2620.2e6, "profiles/k_silu_mul__silu_mul_8192x11008.txt (the five launches of forward + backward together; two passes over the tensors)"),
+    "rmsnorm": (332.5e6, "profiles/k_rmsnorm__rmsnorm_8192x4096.txt (the four kernels of forward + backward together)"),
 }
 
 
