@@ -161,12 +161,13 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
         constexpr int stage = decltype(stage_c)::value;
         return *(const v8bf*)(lds + k_base[c] + (stage * kStageBytes + kt * 32 * 256));
     };
-    // V^T fragment (A operand of O^T): dimension 32 dt + l32, keys 16 j + 8 h32 .. + 7, through two transposing reads.
-    // Within a group of 16 lanes, lane i points at key (16 j + 8 h32) + i / 4 (+ 4 for the second read), dimensions
+    // V^T fragment (A operand of O^T): dimension 32 dt + l32; the 8 slots of half-wave h hold keys 16 j + 4 h .. + 3 and
+    // 16 j + 8 + 4 h .. + 3, the order in which the score accumulators hold them, through two transposing reads.
+    // Within a group of 16 lanes, lane i points at key (16 j + 4 h32) + i / 4 (+ 8 for the second read), dimensions
     // d0 + 4 (i % 4) .. + 3 with d0 = 32 dt + 16 * (group % 2); lane i then receives dimension d0 + i of 4 consecutive keys.
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) v4s* lds_v4s_ptr;
-    const int tr_i = lane & 15, tr_dim = 16 * ((lane >> 4) & 1) + 4 * (tr_i & 3), tr_key = 8 * h32 + (tr_i >> 2);
+    const int tr_i = lane & 15, tr_dim = 16 * ((lane >> 4) & 1) + 4 * (tr_i & 3), tr_key = 4 * h32 + (tr_i >> 2);
     uint32_t v_base[4];  // the lane's byte offset inside a V tile for dimension block dt, key block 0 (the swizzle is not linear in dt)
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
     auto v_frag = [&](auto stage_c, int dt, int j) -> v8bf {
         constexpr int stage = decltype(stage_c)::value;
         const uint8_t* a0 = lds + v_base[dt] + (stage * kStageBytes + kKTileBytes + j * 16 * 256);  // key 16 j + tr_key: same key & 3
-        const uint8_t* a1 = a0 + 4 * 256;  // key + 4: the same piece
+        const uint8_t* a1 = a0 + 8 * 256;  // key + 8: the same piece
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a0);
         const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)a1);
         typedef short v8s __attribute__((ext_vector_type(8)));
@@ -297,11 +298,10 @@ __global__ __launch_bounds__(256, 2) void k_attn_fwd(AttnArgs A) {
         for (int kt = 0; kt < 2; kt++)
 #pragma unroll
             for (int u = 0; u < 2; u++) {
-                // packed registers 4 u, 4 u + 1 hold keys 16 u + 4 h .. + 3, registers 4 u + 2, 4 u + 3 keys 16 u + 8 + 4 h .. + 3
-                const auto s0 = __builtin_amdgcn_permlane32_swap(pk[kt][4 * u], pk[kt][4 * u + 2], false, false);
-                const auto s1 = __builtin_amdgcn_permlane32_swap(pk[kt][4 * u + 1], pk[kt][4 * u + 3], false, false);
-                // half-wave h now holds keys 16 u + 8 h .. + 7 in slot order
-                const v4i_t pw = (v4i_t){(int)s0[0], (int)s1[0], (int)s0[1], (int)s1[1]};
+                // The 16 keys of chunk j = 2 kt + u are summed over, so their order inside the product is free as long as P and V
+                // agree: the lane's packed registers 4 u .. 4 u + 3 (keys 16 j + 4 h .. + 3 and 16 j + 8 + 4 h .. + 3) are taken as
+                // its 8 slots as they are, and the V^T fragment reads those keys into the same slots: no lane exchange.
+                const v4i_t pw = (v4i_t){(int)pk[kt][4 * u], (int)pk[kt][4 * u + 1], (int)pk[kt][4 * u + 2], (int)pk[kt][4 * u + 3]};
                 const v8bf pfrag = __builtin_bit_cast(v8bf, pw);
 #pragma unroll
                 for (int dt = 0; dt < 4; dt++)
