@@ -59,6 +59,8 @@ def probe_lib():
         L = ctypes.CDLL(PROBE_LIB)
         vp, i64 = ctypes.c_void_p, ctypes.c_int64
         L.bench_hbm_probe.argtypes = [ctypes.c_int, vp, vp, i64, vp]
+        L.bench_pattern_probe.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, vp]
+        L.bench_pattern_probe.restype = ctypes.c_int
         L.bench_gemm_clock.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, vp, vp]
         L.bench_hbm_probe.restype = L.bench_gemm_clock.restype = ctypes.c_int
         _probe_lib = L
@@ -429,15 +431,43 @@ def make_hbm_probe_workload(dev, torch, kind):
                                                       "kernel": "k_hbm_probe"}
 
 
-def make_division_workload(dev, torch, stochastic, transpose=False):
-    """Per-tensor division bf16 [8192,4096] -> e5m2 with a given scale, deterministic or with the reference's stochastic
+def make_pattern_probe_workload(dev, torch, kind, shape):
+    """The access pattern of the per-tensor division kernels with the arithmetic taken out (bench_pattern_probe of
+    bench_probe.hip): "narrow" = k_division's (16-byte loads of 2-byte elements, 8-byte stores of 1-byte codes), "tile" =
+    k_division_transpose's (128 x 128 tiles, 32 bytes per lane in, 16 bytes into q and 16 into q^T out, no LDS).  Four
+    rotating buffer sets, so the memory-side cache holds nothing of the next launch.  The time of these is what the memory
+    system allows the real kernels at the same shape."""
+    from coat_amd import _hip
+    L = probe_lib()
+    M, N = shape
+    if kind == "tile" and (M % 128 or N % 128):
+        raise SystemExit("hbm_tile needs --shape M N with both multiples of 128")
+    nset = 4
+    xs = [torch.empty(M * N, dtype=torch.bfloat16, device=dev).fill_(1.0) for _ in range(nset)]
+    qs = [torch.empty(M * N, dtype=torch.uint8, device=dev) for _ in range(nset)]
+    qts = [torch.empty(M * N, dtype=torch.uint8, device=dev) for _ in range(nset)] if kind == "tile" else [None] * nset
+    code = {"narrow": 0, "tile": 1}[kind]
+    state = {"i": 0}
+
+    def step():
+        i = state["i"] = (state["i"] + 1) % nset
+        _hip.check(L.bench_pattern_probe(code, _hip.ptr(xs[i]), _hip.ptr(qs[i]), _hip.ptr(qts[i]), M, N, _hip.stream(dev)),
+                   "pattern_probe")
+
+    nbytes = M * N * (3 if kind == "narrow" else 4)
+    return step, nbytes, {"workload": f"pattern probe {kind}: bench_pattern_probe on 2-byte [{M},{N}], {nset} rotating buffer sets",
+                          "kernel": "k_narrow_probe" if kind == "narrow" else "k_tile_probe"}
+
+
+def make_division_workload(dev, torch, stochastic, transpose=False, shape=(8192, 4096)):
+    """Per-tensor division bf16 [8192,4096] (or --shape) -> e5m2 with a given scale, deterministic or with the reference's stochastic
     rounding (coat/activation/real_quantization/_division.py:153-207): 2 bytes read + 1 written per element; with
     ``transpose`` the transposed copy is written too (_division_transpose.py:147-210, 2 + 2 bytes)."""
     import coat_amd.activation.real_quantization as rq
 
-    M, N = 8192, 4096
+    M, N = shape
     gen = torch.Generator(device=dev).manual_seed(0)
-    xs = [torch.randn(M, N, generator=gen, device=dev).bfloat16() for _ in range(6)]
+    xs = [torch.randn(M, N, generator=gen, device=dev).bfloat16() for _ in range(max(4, min(6, (400 << 20) // (M * N * 2) + 1)))]
     scale = torch.tensor(0.01, device=dev, dtype=torch.bfloat16)
     it = {"i": 0}
 
@@ -852,12 +882,15 @@ def make_stream_workload(name, args, dev, torch):
         return make_gemm_workload(dev, torch, name.split("_")[1], args.grad_format)
     if name == "cross_entropy":
         return make_cross_entropy_workload(dev, torch)
+    if name in ("hbm_narrow", "hbm_tile"):
+        return make_pattern_probe_workload(dev, torch, name.split("_")[1], tuple(args.shape) if args.shape != [4096, 4096] else (8192, 4096))
     if name.startswith("hbm_"):
         return make_hbm_probe_workload(dev, torch, name.split("_")[1])
     if name == "layernorm":
         return make_layernorm_workload(dev, torch)
     if name in ("division", "division_sr", "division_transpose"):
-        return make_division_workload(dev, torch, name == "division_sr", transpose=name == "division_transpose")
+        return make_division_workload(dev, torch, name == "division_sr", transpose=name == "division_transpose",
+                                      shape=tuple(args.shape) if args.shape != [4096, 4096] else (8192, 4096))
     if name == "silu_mul":
         return make_silu_mul_workload(dev, torch)
     if name == "rmsnorm":
@@ -947,11 +980,11 @@ def main():
     ap.add_argument("--workload", default="all",
                     choices=["all", "gemm_clock", "adamw", "adamw_class", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad",
                              "gemm_wgrad", "linear", "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr",
-                             "division_transpose", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "layer_7b", "layer_13b", "attention"],
+                             "division_transpose", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "hbm_narrow", "hbm_tile", "layer_7b", "layer_13b", "attention"],
                     help="all (default): the headline AdamW step as `value` plus an `extra` record for every other leg of the metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", type=int, nargs=2, default=[4096, 4096], metavar=("M", "N"),
-                    help="input shape of the quantize / quantize_transpose workloads (default: the headline [4096, 4096])")
+                    help="input shape of the quantize / quantize_transpose workloads (default: the headline [4096, 4096]) and of the division* / hbm_narrow / hbm_tile workloads (default for those: [8192, 4096])")
     ap.add_argument("--cache-weights", action="store_true",
                     help="layer workloads: weight_memory_efficient=False (FP8 weights cached after the first micro-batch)")
     ap.add_argument("--grad-format", default="e5m2", choices=["e5m2", "e4m3"],
