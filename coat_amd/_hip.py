@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("COAT_HIP_LIB") or os.path.join(_HERE, "libcoat_hip.so
 F32, BF16, F16 = 0, 1, 2
 MAX_SLOTS, MAX_SLOT_STRIDE = 16, 32  # COAT_MAX_SLOTS, COAT_MAX_SLOT_STRIDE of include/coat_hip.h
 MAX_WORDS = MAX_SLOTS * MAX_SLOT_STRIDE
-ABI_VERSION = 4  # COAT_ABI_VERSION of include/coat_hip.h: a library built from another header is refused
+ABI_VERSION = 5  # COAT_ABI_VERSION of include/coat_hip.h: a library built from another header is refused
 E4M3, E5M2 = 0, 1
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
@@ -28,6 +28,7 @@ _u64 = ctypes.c_uint64
 SIGNATURES = {
     "coat_fp8_quantize": [_vp, _i, _vp, _vp, _i, _i64, _i64, _i, _i, _vp],
     "coat_fp8_quantize_transpose": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _i, _vp],
+    "coat_fp8_quantize_perblock": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i64, _i, _i, _vp],
     "coat_fp8_group_scales": [_vp, _i, _vp, _i, _vp, _i64, _i64, _i, _i, _vp],
     "coat_absmax": [_vp, _i, _vp, _i64, _vp],
     "coat_fp8_division": [_vp, _i, _vp, _i, _vp, _vp, _i64, _i64, _i, _vp],

@@ -3,6 +3,7 @@ from ._dequantize import fp8_dequantize
 from ._division import fp8_division
 from ._division_transpose import fp8_division_transpose
 from ._quantize import fp8_quantize
+from ._quantize_perblock import fp8_quantize_perblock
 from ._quantize_pertensor import fp8_quantize_pertensor
 from ._quantize_pertensor_transpose import fp8_quantize_pertensor_transpose
 from ._quantize_transpose import fp8_quantize_transpose

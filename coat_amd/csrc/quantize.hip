@@ -1066,3 +1066,117 @@ extern "C" int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, 
 #undef LAUNCH_QT
     return COAT_EINVAL;
 }
+
+// ------------------------------------------------------------------------------------------------
+// Per-block quantize: one scale per QB x QB block, (max|x| + 1e-10) / fp8max, the block divided by the fp32 scale and the
+// scale stored in the scale dtype (reference coat/activation/real_quantization/_quantize_perblock.py:33-104), optionally
+// with the transposed codes and scales (_quantize_perblock_transpose.py:33-133, ONLY_TRANSPOSED = the plain outputs absent)
+// and with a 1 x QB per-group quantization of the same input (_quantize_perblock_transpose_pergroup.py:140-172), which is
+// what the DeepSeek-style linear consumes (coat/activation/deepseek/fp8linear.py:70-110).
+// A block of 512 threads takes a 128 x 128 tile = (128 / QB)^2 quantization blocks: pass 1 leaves every block's maximum
+// in LDS (row-group maximum by DPP, one LDS atomic per row group), pass 2 converts from the registers that still hold the
+// tile, writes the codes and parks them in LDS for the transposed stores.
+namespace coat {
+__device__ __forceinline__ void store_scale_rt(void* p, int64_t i, float v, int dt) {
+    if (dt == kF32) ((float*)p)[i] = v;
+    else if (dt == kBF16) ((uint16_t*)p)[i] = (uint16_t)f2bf16(v);
+    else ((uint16_t*)p)[i] = (uint16_t)f2f16(v);
+}
+
+template <int XDT, int KIND>
+__global__ __launch_bounds__(kDivTThreads) void k_quantize_perblock(const void* __restrict__ x, void* __restrict__ q,
+                                                                    void* __restrict__ s_out, void* __restrict__ qt,
+                                                                    void* __restrict__ st_out, void* __restrict__ qpg,
+                                                                    void* __restrict__ spg_out, int sdt, int64_t M, int64_t N,
+                                                                    int QB) {
+    constexpr int VEC = VecOf<XDT>::kVec, T = kTileN, JPR = T / VEC, NIT = T * JPR / kDivTThreads;
+    static_assert(T * JPR % kDivTThreads == 0 && kDivTThreads % JPR == 0, "whole iterations, whole rows per iteration");
+    __shared__ uint32_t tile[T * kPitchDw];
+    __shared__ uint32_t bmax[64];  // (128 / 16)^2 block maxima at most, as bit patterns (non-negative floats order like integers)
+    enable_fp8_saturation();
+    const int64_t tiles_n = (N + T - 1) / T;
+    const int64_t m0 = (blockIdx.x / tiles_n) * T, n0 = (blockIdx.x % tiles_n) * T;
+    const int nb = T / QB;     // quantization blocks per tile edge
+    const int lpg = QB / VEC;  // lanes that hold one row of a quantization block: aligned runs of consecutive lanes
+    const int64_t SN = N / QB, SM = M / QB;
+    if (threadIdx.x < 64) bmax[threadIdx.x] = 0;
+    uint4 raw[NIT];
+    float gmax[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * kDivTThreads;
+        const int64_t m = m0 + job / JPR, n = n0 + (job % JPR) * VEC;
+        raw[it] = (m < M && n < N) ? *(const uint4*)((const uint8_t*)x + (m * N + n) * (16 / VEC)) : make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * kDivTThreads;
+        const int row = job / JPR, cv = job % JPR;
+        float v[VEC];
+        unpack_vec<XDT>(raw[it], v);
+        gmax[it] = cluster_max_rt(vec_amax<VEC>(v), lpg);
+        if ((threadIdx.x % lpg) == 0) atomicMax(&bmax[(row / QB) * nb + (cv * VEC) / QB], f2u(gmax[it]));
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int job = threadIdx.x + it * kDivTThreads;
+        const int row = job / JPR, cv = job % JPR;
+        const int64_t m = m0 + row, n = n0 + cv * VEC;
+        const bool ok = m < M && n < N;  // M % QB == 0 and N % QB == 0: a quantization block is inside or outside as a whole
+        float v[VEC];
+        unpack_vec<XDT>(raw[it], v);
+        const float sb = group_scale<KIND>(u2f(bmax[(row / QB) * nb + (cv * VEC) / QB]));
+        uint32_t c[VEC / 4];
+        quantize_vec<KIND, VEC>(v, sb, 1.0f / sb, c);
+        if (q && ok) store_codes<VEC>(q, m * N + n, c);
+        if (qt) {
+#pragma unroll
+            for (int k = 0; k < VEC / 4; k++) tile[row * kPitchDw + cv * (VEC / 4) + k] = c[k];
+        }
+        if (ok && (row % QB) == 0 && ((cv * VEC) % QB) == 0) {
+            if (s_out) store_scale_rt(s_out, (m / QB) * SN + n / QB, sb, sdt);
+            if (st_out) store_scale_rt(st_out, (n / QB) * SM + m / QB, sb, sdt);
+        }
+        if (qpg) {
+            const float sg = group_scale<KIND>(gmax[it]);
+            uint32_t cg[VEC / 4];
+            quantize_vec<KIND, VEC>(v, sg, 1.0f / sg, cg);
+            if (ok) {
+                store_codes<VEC>(qpg, m * N + n, cg);
+                if ((threadIdx.x % lpg) == 0) store_scale_rt(spg_out, m * SN + n / QB, sg, sdt);
+            }
+        }
+    }
+    if (qt) {
+        __syncthreads();
+        store_tile_transposed<T>(tile, qt, M, N, m0, n0);
+    }
+}
+}  // namespace coat
+
+// x [M, N] (M % QB == 0, N % QB == 0, QB 16 / 32 / 64 / 128) -> any of: q [M, N] + s [M/QB, N/QB]; qt [N, M] + st [N/QB, M/QB];
+// qpg [M, N] + spg [M, N/QB] (1 x QB groups).  A pair is produced when both of its pointers are given.
+extern "C" int coat_fp8_quantize_perblock(const void* x, int x_dtype, void* q, void* s, void* qt, void* st_out, void* qpg,
+                                          void* spg, int s_dtype, int64_t M, int64_t N, int QB, int fp8, void* stream) {
+    if (M < 0 || N < 0) return COAT_EINVAL;
+    if (QB != 16 && QB != 32 && QB != 64 && QB != 128) return COAT_ESHAPE;
+    if (M % QB != 0 || N % QB != 0) return COAT_ESHAPE;
+    if (s_dtype != COAT_F32 && s_dtype != COAT_BF16 && s_dtype != COAT_F16) return COAT_EDTYPE;
+    if ((q == nullptr) != (s == nullptr) || (qt == nullptr) != (st_out == nullptr) || (qpg == nullptr) != (spg == nullptr)) return COAT_EINVAL;
+    if (!q && !qt && !qpg) return COAT_EINVAL;
+    if (M * N == 0) return COAT_OK;
+    if (!x) return COAT_EINVAL;
+    if (!coat_aligned16(x) || !coat_aligned16(q) || !coat_aligned16(qt) || !coat_aligned16(qpg)) return COAT_EALIGN;
+    const int64_t blocks = ((M + kTileN - 1) / kTileN) * ((N + kTileN - 1) / kTileN);
+    if (blocks >= ((int64_t)1 << 31)) return COAT_ESHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    const int sdt = s_dtype == COAT_F32 ? kF32 : s_dtype == COAT_BF16 ? kBF16 : kF16;
+    DISPATCH_XDT(x_dtype, DISPATCH_KIND(fp8, {
+        hipLaunchKernelGGL((k_quantize_perblock<XDT, KIND>), dim3((unsigned)blocks), dim3(kDivTThreads), 0, st, x, q, s, qt, st_out,
+                           qpg, spg, sdt, M, N, QB);
+        return coat_launch_status();
+    }));
+    return COAT_EINVAL;
+}

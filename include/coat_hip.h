@@ -48,9 +48,9 @@ enum coat_fp8 { COAT_E4M3 = 0, COAT_E5M2 = 1 }; /* torch.float8_e4m3fn / torch.f
 /* Bumped whenever an entry point's argument list or the size of a buffer it writes changes (2: every s_max / amax
  * argument became COAT_MAX_WORDS words; 3: coat_fp8_gemm_residual, coat_fp8_rmsnorm_backward_add and coat_attention_forward_bf16 added,
  * coat_hbm_probe removed; 4: coat_rope_bf16 and coat_attention_forward_bf16 take a maximum buffer, the multi-tensor optimizer
- * steps and coat_fp8_layernorm_backward_add added).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
+ * steps and coat_fp8_layernorm_backward_add added; 5: coat_fp8_quantize_perblock added).  A caller compiled against this header checks coat_abi_version() == COAT_ABI_VERSION when it
  * loads the library. */
-#define COAT_ABI_VERSION 4
+#define COAT_ABI_VERSION 5
 int coat_abi_version(void);
 const char* coat_version(void);
 const char* coat_status_string(int status);
@@ -66,6 +66,16 @@ int coat_fp8_quantize(const void* x, int x_dtype, void* q, void* s, int s_dtype,
  * (groups of QB along M).  qt [N,M], st [N,M/QB].  Also M % QB == 0. */
 int coat_fp8_quantize_transpose(const void* x, int x_dtype, void* q, void* s, void* qt, void* st, int s_dtype,
                                 int64_t M, int64_t N, int QB, int fp8, void* stream);
+
+/* rq/_quantize_perblock.py:107 fp8_quantize_perblock (kernel :33-104), rq/_quantize_perblock_transpose.py:136
+ * fp8_quantize_perblock_transpose (kernel :33-133) and rq/_quantize_perblock_transpose_pergroup.py:175
+ * fp8_quantize_perblock_transpose_pergroup (kernel :33-172): one scale per QB x QB block, s = (amax_block + 1e-10) / fp8max,
+ * q = fp8(x / s32); optionally the transposed codes and scales, and the 1 x QB per-group quantization of the same input.
+ * x [M,N] x_dtype; outputs in pairs, a pair is produced when both pointers are given (at least one pair):
+ *   q [M,N] fp8 + s [M/QB, N/QB];  qt [N,M] fp8 + st [N/QB, M/QB];  qpg [M,N] fp8 + spg [M, N/QB]   (scales: s_dtype).
+ * QB in {16,32,64,128}, M % QB == 0, N % QB == 0. */
+int coat_fp8_quantize_perblock(const void* x, int x_dtype, void* q, void* s, void* qt, void* st, void* qpg, void* spg,
+                               int s_dtype, int64_t M, int64_t N, int QB, int fp8, void* stream);
 
 /* rq/_quantize_pertensor.py:46-103 (+ the `s_y.max()` at :139): per-group scales and their maximum.
  * s_pg [M,N/QB] s_dtype (may be NULL when only the maximum is wanted); s_max: COAT_MAX_WORDS fp32 in device

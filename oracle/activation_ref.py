@@ -22,6 +22,11 @@ Pin status (tests/test_oracle_activation.py unless noted):
                            recomputed in float64; equal-fraction >= 0.95 against the reference
                            test's own definition ``quantize_tensor_ref_test`` (tests/test_utils.py:61-67)
   fp8_quantize_transpose   == fp8_quantize(x.T) (invariant)
+  fp8_quantize_perblock*   block maxima and scales recomputed with plain loops in float64; closed form on hand-made
+                           blocks; error bound of half an fp8 step of the block maximum; a block as large as the
+                           tensor == fp8_division by the fp32 scale; transposed outputs == outputs transposed;
+                           per-group part == fp8_quantize; equal-fraction >= 0.95 against the reference test's own
+                           definition (tests/test_utils.py:53-60)
   fp8_group_scales, fp8_quantize_pertensor*  per-tensor scale == bf16 of the max group scale
                            (monotone rounding); codes == cast(x / s)
   fp8_division*            transposed output == output.T; absmax scale in the input dtype
@@ -79,6 +84,36 @@ def fp8_quantize_transpose(x, QB, fp8type, scale_dtype=torch.bfloat16):
     """rq/_quantize_transpose.py:175-226: per-group quantize of x and of x^T (kernel :127-137)."""
     x32 = x.float()
     return _quantize_pg(x32, QB, fp8type, scale_dtype), _quantize_pg(x32.t().contiguous(), QB, fp8type, scale_dtype)
+
+
+def _block_scale32(v32, QB, fp8type):
+    """rq/_quantize_perblock.py:72-75: max|v| over each QB x QB block, + 1e-10, / fp8max, all fp32."""
+    M, N = v32.shape
+    amax = v32.reshape(M // QB, QB, N // QB, QB).abs().amax(dim=(1, 3))
+    return (amax + SCALE_MIN_THRES) / FP8_MAX_VALUE[_fp8(fp8type)]
+
+
+def fp8_quantize_perblock(x, QB, fp8type, scale_dtype=torch.bfloat16):
+    """rq/_quantize_perblock.py:107-150 (kernel :33-104): the block is divided by its fp32 scale (:78), the scale is
+    stored rounded to ``scale_dtype`` (:82)."""
+    v32 = x.float()
+    s32 = _block_scale32(v32, QB, fp8type)
+    q = cast_fp8(v32 / s32.repeat_interleave(QB, 0).repeat_interleave(QB, 1), fp8type)
+    return q, s32.to(scale_dtype)
+
+
+def fp8_quantize_perblock_transpose(x, QB, fp8type, scale_dtype=torch.bfloat16, only_transposed=False):
+    """rq/_quantize_perblock_transpose.py:136-190 (kernel :33-133): the same codes and scales, also transposed (:84-88)."""
+    q, s = fp8_quantize_perblock(x, QB, fp8type, scale_dtype)
+    q_t, s_t = q.view(torch.uint8).t().contiguous().view(q.dtype), s.t().contiguous()
+    return (q_t, s_t) if only_transposed else ((q, s), (q_t, s_t))
+
+
+def fp8_quantize_perblock_transpose_pergroup(x, QB, fp8type, scale_dtype=torch.bfloat16):
+    """rq/_quantize_perblock_transpose_pergroup.py:175-246 (kernel :33-172): per-block pair, its transpose, and the
+    1 x QB per-group quantization of the same input (:140-172: row maxima inside the block = groups of QB along N)."""
+    (q, s), (q_t, s_t) = fp8_quantize_perblock_transpose(x, QB, fp8type, scale_dtype)
+    return (q, s), (q_t, s_t), _quantize_pg(x.float(), QB, fp8type, scale_dtype)
 
 
 def fp8_group_scales(x, QB, fp8type, scale_dtype=torch.bfloat16):
@@ -366,3 +401,14 @@ def quantize_tensor_ref_test(x, QB, fp8type):
     sx = (g.abs().amax(dim=2) / FP8_MAX_VALUE[fp8type]).to(torch.bfloat16)
     q = (g / sx.float().unsqueeze(2)).to(fp8type).reshape(M, N)
     return q, sx
+
+
+def quantize_tensor_ref_test_perblock(x, QB, fp8type):
+    """tests/test_utils.py:53-60 ("per_block"): scale = bf16(amax_block / fp8max) (no 1e-10), the value divided by the
+    bf16-rounded scale; >= 95 % equal codes is what the reference's test asks of its kernel (tests/test_fp8_quantize.py:42-48)."""
+    fp8type = _fp8(fp8type)
+    M, N = x.shape
+    g = x.float().reshape(M // QB, QB, N // QB, QB).permute(0, 2, 1, 3)
+    sx = (g.abs().amax(dim=(2, 3)) / FP8_MAX_VALUE[fp8type]).to(torch.bfloat16)
+    q = (g / sx.float().unsqueeze(2).unsqueeze(3)).to(fp8type)
+    return q.permute(0, 2, 1, 3).reshape(M, N), sx

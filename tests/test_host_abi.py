@@ -95,6 +95,14 @@ def test_argument_validation_of_the_remaining_entry_points_without_gpu():
     assert L.coat_fp8_division_from_max(p, 1, p, None, 1, p, None, 16, 64, 0, None) == EINVAL  # nowhere to put the scale
     assert L.coat_fp8_division_stochastic(p, 1, p, 1, p, None, 1 << 17, 1 << 16, 0, 0, None) == ESHAPE  # > 2^32 noise indices
     assert L.coat_fp8_dequantize(p, 0, p, 1, p, 4, 64, 24, None) == ESHAPE
+    # per-block quantizers: x, dt, q, s, qt, st, qpg, spg, s_dt, M, N, QB, fp8
+    assert L.coat_fp8_quantize_perblock(p, 1, p, p, None, None, None, None, 0, 96, 96, 48, 0, None) == ESHAPE     # QB
+    assert L.coat_fp8_quantize_perblock(p, 1, p, p, None, None, None, None, 0, 100, 128, 128, 0, None) == ESHAPE  # M % QB
+    assert L.coat_fp8_quantize_perblock(p, 1, p, None, None, None, None, None, 0, 128, 128, 128, 0, None) == EINVAL  # half a pair
+    assert L.coat_fp8_quantize_perblock(p, 1, None, None, None, None, None, None, 0, 128, 128, 128, 0, None) == EINVAL  # no output
+    assert L.coat_fp8_quantize_perblock(p, 1, p, p, odd, p, None, None, 0, 128, 128, 128, 0, None) == EALIGN
+    assert L.coat_fp8_quantize_perblock(p, 1, p, p, None, None, None, None, 9, 128, 128, 128, 0, None) == EDTYPE
+    assert L.coat_fp8_quantize_perblock(p, 1, p, p, None, None, None, None, 0, 0, 128, 128, 0, None) == 0         # empty
     # the divisions that recompute their input
     assert L.coat_fp8_rmsnorm_division(p, 0, p, 1, p, 1, p, p, p, p, p, 24, 64, 16, None) == ESHAPE
     assert L.coat_fp8_rmsnorm_division(p, 0, p, 1, p, 1, None, p, p, p, p, 16, 64, 16, None) == EINVAL

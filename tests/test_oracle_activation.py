@@ -68,6 +68,81 @@ def test_quantize_transpose_is_quantize_of_transpose():
     assert qt.shape == (96, 64) and st.shape == (96, 4)
 
 
+def test_perblock_hand_made_blocks():
+    x = torch.zeros(32, 32)
+    x[:16, :16] = (torch.arange(256).reshape(16, 16) % 16) * 28.0   # block (0,0): amax 420 -> s = 0.9375
+    x[:16, 16:] = -448.0                                            # block (0,1): s = 1, every code 0xFE
+    x[20, 3] = 1.0                                                  # block (1,0): s = 1/448, that element codes 448
+    q, s = R.fp8_quantize_perblock(x, 16, "E4M3")
+    assert s.dtype == torch.bfloat16 and s.shape == (2, 2)
+    assert s[0, 0].item() == 0.9375 and s[0, 1].item() == 1.0
+    assert s[1, 0].float().item() == pytest.approx(1.0 / 448, rel=4e-3) and s[1, 1].float().item() == pytest.approx(1e-10 / 448, rel=1e-2)
+    assert (q[:16, 16:].view(torch.uint8) == 0xFE).all()
+    want = ((torch.arange(256).reshape(16, 16) % 16) * 28.0 / 0.9375).to(E4)
+    assert torch.equal(q[:16, :16].view(torch.uint8), want.view(torch.uint8))
+    assert q[20, 3].view(torch.uint8).item() == 0x7E
+    rest = q[16:, :].view(torch.uint8).clone()
+    rest[4, 3] = 0
+    assert (rest == 0).all()
+
+
+@pytest.mark.parametrize("fp8,QB,sdt", [("E4M3", 16, torch.bfloat16), ("E5M2", 32, torch.float32), ("E4M3", 128, torch.float32)])
+def test_perblock_scales_by_loops_and_error_bound(fp8, QB, sdt):
+    M, N = 2 * QB, 3 * QB
+    x = _x(M, N, 11)
+    q, s = R.fp8_quantize_perblock(x, QB, fp8, scale_dtype=sdt)
+    fmax = R.FP8_MAX_VALUE[R.STR2FP8[fp8]]
+    mant = 3 if fp8 == "E4M3" else 2
+    xl = x.double().tolist()
+    for bi in range(M // QB):
+        for bj in range(N // QB):
+            amax = 0.0
+            for r in range(QB):          # plain loops: nothing shared with the oracle's reshape / amax
+                for c in range(QB):
+                    amax = max(amax, abs(xl[bi * QB + r][bj * QB + c]))
+            s32 = (torch.tensor(amax, dtype=torch.float32) + torch.tensor(1e-10)) / fmax
+            assert s[bi, bj].item() == s32.to(sdt).item()
+            blk = q[bi * QB:(bi + 1) * QB, bj * QB:(bj + 1) * QB].double() * s32.double()
+            err = (blk - x[bi * QB:(bi + 1) * QB, bj * QB:(bj + 1) * QB].double()).abs()
+            assert (err <= amax * 2.0 ** -(mant + 1) * (1 + 1e-6) + 1e-12).all()
+            assert q[bi * QB:(bi + 1) * QB, bj * QB:(bj + 1) * QB].float().abs().max().item() == fmax
+
+
+def test_perblock_of_one_block_is_division_by_the_fp32_scale():
+    x = _x(64, 64, 12, dtype=torch.float32)
+    q, s = R.fp8_quantize_perblock(x, 64, "E4M3", scale_dtype=torch.float32)
+    s32 = (x.abs().max() + torch.tensor(1e-10)) / 448.0
+    qd, _ = R.fp8_division(x, 16, "E4M3", s32)
+    assert s.shape == (1, 1) and s.item() == s32.item()
+    assert torch.equal(q.view(torch.uint8), qd.view(torch.uint8))
+
+
+def test_perblock_transpose_and_pergroup_parts():
+    x = _x(64, 96, 13)
+    (q, s), (qt, st), (qg, sg) = R.fp8_quantize_perblock_transpose_pergroup(x, 32, "E4M3", scale_dtype=torch.float32)
+    q0, s0 = R.fp8_quantize_perblock(x, 32, "E4M3", scale_dtype=torch.float32)
+    assert torch.equal(q.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(s, s0)
+    assert qt.shape == (96, 64) and st.shape == (3, 2)
+    assert torch.equal(qt.view(torch.uint8), q0.view(torch.uint8).t()) and torch.equal(st, s0.t())
+    qg0, sg0 = R.fp8_quantize(x, 32, "E4M3", scale_dtype=torch.float32)       # the pinned per-group quantizer
+    assert torch.equal(qg.view(torch.uint8), qg0.view(torch.uint8)) and torch.equal(sg, sg0)
+    qt1, st1 = R.fp8_quantize_perblock_transpose(x, 32, "E4M3", scale_dtype=torch.float32, only_transposed=True)
+    assert torch.equal(qt1.view(torch.uint8), qt.view(torch.uint8)) and torch.equal(st1, st)
+    # the transposed pair is the per-block quantization of x^T (blocks are square)
+    q2, s2 = R.fp8_quantize_perblock(x.t().contiguous(), 32, "E4M3", scale_dtype=torch.float32)
+    assert torch.equal(qt.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(st, s2)
+
+
+def test_perblock_against_the_reference_tests_definition():
+    """tests/test_fp8_quantize.py:42-48 with tests/test_utils.py:53-60: fp32 [1024, 2048], QB 16, >= 95 % equal codes."""
+    x = _x(1024, 2048, 14, outliers=False, dtype=torch.float32)
+    q, s = R.fp8_quantize_perblock(x, 16, "E4M3")
+    qb, sb = R.quantize_tensor_ref_test_perblock(x, 16, "E4M3")
+    assert torch.equal(s, sb)
+    eq = (q.view(torch.uint8) == qb.view(torch.uint8)).float().mean().item()
+    assert 0.95 <= eq < 1.0
+
+
 @pytest.mark.parametrize("fp8", ["E4M3", "E5M2"])
 def test_pertensor_paths(fp8):
     x = _x(64, 128, 4)
