@@ -162,6 +162,31 @@ def make_quantize_workload(dev, torch, transpose, shape=(4096, 4096)):
                           "kernel": "k_quantize_transpose" if transpose else "k_quantize_pg"}
 
 
+def make_perblock_workload(dev, torch, shape):
+    """fp8_quantize_perblock_transpose_pergroup (coat/activation/real_quantization/_quantize_perblock_transpose_pergroup.py:175)
+    of a bf16 tensor, QB 128, fp32 scales, only_transposed as the DeepSeek-style linear calls it on a gradient
+    (coat/activation/deepseek/fp8linear.py:97-99): 2 bytes read, the transposed per-block codes and the per-group codes
+    written (1 byte each) plus their scales."""
+    from coat_amd.activation.real_quantization._quantize_perblock_transpose_pergroup import \
+        fp8_quantize_perblock_transpose_pergroup
+
+    M, N = shape
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn(M, N, generator=gen) * 1e-2
+    nset = max(4, min(12, (640 << 20) // (M * N * 2) + 1))
+    xs = [x.bfloat16().to(dev).clone() for _ in range(nset)]
+    state = {"i": 0}
+
+    def step():
+        state["i"] += 1
+        fp8_quantize_perblock_transpose_pergroup(xs[state["i"] % nset], 128, "E4M3", scale_dtype=torch.float32,
+                                                 only_transposed=True)
+
+    nbytes = M * N * 4 + (M // 128) * (N // 128) * 4 + M * (N // 128) * 4
+    return step, nbytes, {"workload": f"fp8_quantize_perblock_transpose_pergroup bf16 [{M},{N}] QB128 e4m3 fp32 scales, "
+                                      f"only_transposed, {nset} rotating inputs", "numel": M * N, "kernel": "k_quantize_perblock"}
+
+
 def make_gemm_workload(dev, torch, which, grad_format="e5m2"):
     """The three GEMMs of FP8Linear at BASELINE config 3 on the config's own data: X [8192,4096] ~ N(0, 0.02),
     W [11008,4096] ~ N(0, 0.02), grad_out [8192,11008] ~ N(0, 1e-2), bf16, each quantized with its per-tensor scale by
@@ -882,6 +907,8 @@ def make_stream_workload(name, args, dev, torch):
         return make_gemm_workload(dev, torch, name.split("_")[1], args.grad_format)
     if name == "cross_entropy":
         return make_cross_entropy_workload(dev, torch)
+    if name == "quantize_perblock":
+        return make_perblock_workload(dev, torch, tuple(args.shape) if args.shape != [4096, 4096] else (8192, 4096))
     if name in ("hbm_narrow", "hbm_tile"):
         return make_pattern_probe_workload(dev, torch, name.split("_")[1], tuple(args.shape) if args.shape != [4096, 4096] else (8192, 4096))
     if name.startswith("hbm_"):
@@ -980,7 +1007,7 @@ def main():
     ap.add_argument("--workload", default="all",
                     choices=["all", "gemm_clock", "adamw", "adamw_class", "adamw_plain", "quantize", "quantize_transpose", "gemm_fwd", "gemm_dgrad",
                              "gemm_wgrad", "linear", "silu_mul", "rmsnorm", "cross_entropy", "layernorm", "division", "division_sr",
-                             "division_transpose", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "hbm_narrow", "hbm_tile", "layer_7b", "layer_13b", "attention"],
+                             "division_transpose", "quantize_perblock", "olmo_block", "hbm_copy", "hbm_read", "hbm_fill", "hbm_narrow", "hbm_tile", "layer_7b", "layer_13b", "attention"],
                     help="all (default): the headline AdamW step as `value` plus an `extra` record for every other leg of the metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", type=int, nargs=2, default=[4096, 4096], metavar=("M", "N"),
