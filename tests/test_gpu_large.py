@@ -63,6 +63,22 @@ def test_quantize_transpose_past_2_31_elements(dev):
     _free(dev)
 
 
+def test_quantize_perblock_past_2_31_elements(dev):
+    from coat_amd.activation.real_quantization._quantize_perblock_transpose_pergroup import \
+        fp8_quantize_perblock_transpose_pergroup
+    x = _big(dev, 4)
+    (q, s), (qt, st), (qg, sg) = fp8_quantize_perblock_transpose_pergroup(x, 32, "E4M3", scale_dtype=torch.float32)
+    assert qt.shape == (COLS, ROWS) and st.shape == (COLS // 32, ROWS // 32) and sg.shape == (ROWS, COLS // 32)
+    for r0, r1 in [(0, 32), (16384, 16416), (ROWS - 32, ROWS)]:  # whole rows of 32 x 32 blocks, the middle one at element 2^30
+        (wq, ws), (wqt, wst), (wqg, wsg) = fp8_quantize_perblock_transpose_pergroup(x[r0:r1].contiguous(), 32, "E4M3",
+                                                                                    scale_dtype=torch.float32)
+        assert torch.equal(q[r0:r1].view(torch.uint8), wq.view(torch.uint8)) and torch.equal(s[r0 // 32:r1 // 32], ws)
+        assert torch.equal(qt[:, r0:r1].view(torch.uint8), wqt.view(torch.uint8)) and torch.equal(st[:, r0 // 32:r1 // 32], wst)
+        assert torch.equal(qg[r0:r1].view(torch.uint8), wqg.view(torch.uint8)) and torch.equal(sg[r0:r1], wsg)
+    del x, q, s, qt, st, qg, sg
+    _free(dev)
+
+
 def test_adamw_expand_past_2_31_elements(dev):
     from coat_amd.optimizer import qoptim_cuda
     numel = (1 << 31) + 3 * 4096 + 77  # ragged last group
